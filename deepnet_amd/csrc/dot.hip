@@ -1,0 +1,290 @@
+// dnh_dot: ITensorBackend VecVecDot / MatVecDot / MatMatDot / BatchedMatMatDot (Tensor/Tensor/TensorBackend.fs:137-140;
+// dispatch by rank as Tensor.FillDot, Tensor/Tensor/Tensor.fs:2714-2730; Host semantics Host/HostBackend.fs:463-546).
+//
+// One strided-batched GEMM kernel, C[b] = A[b] * B[b] (alpha 1, beta 0), written for gfx950:
+//   - 128x128 block tile, K step 16, 256 threads = 4 wavefronts in a 2x2 arrangement, each owning a 64x64 sub-tile;
+//   - fp32: four 32x32 accumulators per wavefront on v_mfma_f32_32x32x2_f32 (A and B operands one dword per lane);
+//     fp64: an 8x8 register micro-tile per thread on vector FMA;
+//   - A is staged k-major ([k][m]) and B as [k][n] in LDS, double buffered, so every MFMA operand fetch is a
+//     conflict-free 4-byte LDS read of consecutive addresses; the next K step's global loads are issued before the
+//     MFMAs of the current one;
+//   - operands are addressed straight from the descriptors (any strides, broadcast batch dimensions, row-major
+//     target written directly): no pointer arrays, no column-major temporary and transposing copy-back as on the
+//     reference's BLAS paths (Tensor/Tensor/BlasSupport.fs:173-190, Cuda/CudaBLAS.fs:28-38).
+// The "fast" instantiation requires row-major, 16-byte aligned A and B and full tiles and uses 16-byte global loads;
+// every other case runs the same kernel with guarded scalar loads.
+#include "map_kernels.h"
+
+using namespace dnh;
+
+namespace {
+
+constexpr int BM = 128, BN = 128, PAD = 4;
+template <class T> constexpr int kBK = sizeof(T) == 8 ? 8 : 16;  // K step: keeps the double-buffered tiles within 64 KB of LDS
+
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+struct GemmArgs {
+    int64_t M, N, K;
+    int64_t sam, sak, sbk, sbn, scm, scn;
+    int nbatch;                                   // batch dimensions
+    uint32_t bshape[DNH_MAX_DIMS];
+    int64_t bsa[DNH_MAX_DIMS], bsb[DNH_MAX_DIMS], bsc[DNH_MAX_DIMS];
+    uint32_t tiles_m, tiles_n;
+};
+
+template <class T, bool FAST>
+__global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, const T* __restrict__ a, const T* __restrict__ b, GemmArgs g) {
+    constexpr int BK = kBK<T>;
+    __shared__ T As[2][BK][BM + PAD];
+    __shared__ T Bs[2][BK][BN + PAD];
+
+    uint32_t bid = blockIdx.x;
+    const uint32_t tn = bid % g.tiles_n;
+    bid /= g.tiles_n;
+    const uint32_t tm = bid % g.tiles_m;
+    bid /= g.tiles_m;
+    int64_t oa = 0, ob = 0, oc = 0;
+    for (int d = g.nbatch - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
+        const uint32_t i = bid - q * g.bshape[d];
+        bid = q;
+        oa += (int64_t)i * g.bsa[d];
+        ob += (int64_t)i * g.bsb[d];
+        oc += (int64_t)i * g.bsc[d];
+    }
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    a += oa;
+    b += ob;
+    c += oc;
+
+    const int tid = threadIdx.x;
+    // global -> register staging
+    constexpr int SPT = BM * BK / kBlock;  // elements of each tile per thread
+    T ra[SPT], rb[SPT];
+
+    auto load_tiles = [&](int64_t k0) {
+        if constexpr (FAST) {
+            constexpr int V = 16 / (int)sizeof(T);           // elements per 16-byte load
+            constexpr int APT = (BM * BK) / (kBlock * V);     // loads per thread for A (fp32: 2, fp64: 4)
+            constexpr int KV = BK / V;                        // vectors per A row
+#pragma unroll
+            for (int i = 0; i < APT; i++) {
+                const int idx = tid + i * kBlock;
+                const int row = idx / KV, kv = (idx % KV) * V;
+                const Pack<T, V> v = load_pack<T, V>(a + (m0 + row) * g.sam + (k0 + kv));
+#pragma unroll
+                for (int e = 0; e < V; e++) ra[i * V + e] = v.v[e];
+            }
+            constexpr int NV = BN / V;                        // vectors per B row
+#pragma unroll
+            for (int i = 0; i < APT; i++) {
+                const int idx = tid + i * kBlock;
+                const int kk = idx / NV, nv = (idx % NV) * V;
+                const Pack<T, V> v = load_pack<T, V>(b + (k0 + kk) * g.sbk + (n0 + nv));
+#pragma unroll
+                for (int e = 0; e < V; e++) rb[i * V + e] = v.v[e];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < SPT; i++) {
+                const int idx = tid + i * kBlock;
+                {
+                    const int row = idx / BK, kk = idx % BK;
+                    const int64_t m = m0 + row, k = k0 + kk;
+                    ra[i] = (m < g.M && k < g.K) ? a[m * g.sam + k * g.sak] : T(0);
+                }
+                {
+                    const int kk = idx / BN, col = idx % BN;
+                    const int64_t k = k0 + kk, n = n0 + col;
+                    rb[i] = (k < g.K && n < g.N) ? b[k * g.sbk + n * g.sbn] : T(0);
+                }
+            }
+        }
+    };
+    auto store_tiles = [&](int buf) {
+        if constexpr (FAST) {
+            constexpr int V = 16 / (int)sizeof(T);
+            constexpr int APT = (BM * BK) / (kBlock * V);
+            constexpr int KV = BK / V;
+#pragma unroll
+            for (int i = 0; i < APT; i++) {
+                const int idx = tid + i * kBlock;
+                const int row = idx / KV, kv = (idx % KV) * V;
+#pragma unroll
+                for (int e = 0; e < V; e++) As[buf][kv + e][row] = ra[i * V + e];
+            }
+            constexpr int NV = BN / V;
+#pragma unroll
+            for (int i = 0; i < APT; i++) {
+                const int idx = tid + i * kBlock;
+                const int kk = idx / NV, nv = (idx % NV) * V;
+#pragma unroll
+                for (int e = 0; e < V; e++) Bs[buf][kk][nv + e] = rb[i * V + e];
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < SPT; i++) {
+                const int idx = tid + i * kBlock;
+                As[buf][idx % BK][idx / BK] = ra[i];
+                Bs[buf][idx / BN][idx % BN] = rb[i];
+            }
+        }
+    };
+
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+
+    if constexpr (std::is_same<T, float>::value) {
+        f32x16 acc[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+
+        load_tiles(0);
+        store_tiles(0);
+        __syncthreads();
+        int cur = 0;
+        const int lk = lane >> 5, lm = lane & 31;
+        for (int64_t k0 = 0; k0 < g.K; k0 += BK) {
+            const bool more = k0 + BK < g.K;
+            if (more) load_tiles(k0 + BK);
+#pragma unroll
+            for (int kk = 0; kk < BK; kk += 2) {
+                const float a0 = As[cur][kk + lk][wm + lm];
+                const float a1 = As[cur][kk + lk][wm + 32 + lm];
+                const float b0 = Bs[cur][kk + lk][wn + lm];
+                const float b1 = Bs[cur][kk + lk][wn + 32 + lm];
+                acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+                acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+                acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+                acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+            }
+            if (more) {
+                store_tiles(cur ^ 1);
+                __syncthreads();
+                cur ^= 1;
+            }
+        }
+        // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+#pragma unroll
+                for (int r = 0; r < 16; r++) {
+                    const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
+                    const int64_t n = n0 + wn + j * 32 + lm;
+                    if (FAST || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
+                }
+    } else {
+        // fp64: each thread owns an 8x8 micro-tile (rows ty*8.., columns tx*8..)
+        const int ty = tid / 16, tx = tid % 16;
+        T acc[8][8];
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) acc[i][j] = T(0);
+        load_tiles(0);
+        store_tiles(0);
+        __syncthreads();
+        int cur = 0;
+        for (int64_t k0 = 0; k0 < g.K; k0 += BK) {
+            const bool more = k0 + BK < g.K;
+            if (more) load_tiles(k0 + BK);
+#pragma unroll 4
+            for (int kk = 0; kk < BK; kk++) {
+                T av[8], bv[8];
+#pragma unroll
+                for (int i = 0; i < 8; i++) av[i] = As[cur][kk][ty * 8 + i];
+#pragma unroll
+                for (int j = 0; j < 8; j++) bv[j] = Bs[cur][kk][tx * 8 + j];
+#pragma unroll
+                for (int i = 0; i < 8; i++)
+#pragma unroll
+                    for (int j = 0; j < 8; j++) acc[i][j] = fma(av[i], bv[j], acc[i][j]);
+            }
+            if (more) {
+                store_tiles(cur ^ 1);
+                __syncthreads();
+                cur ^= 1;
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++)
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+                const int64_t m = m0 + ty * 8 + i, n = n0 + tx * 8 + j;
+                if (FAST || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j];
+            }
+    }
+}
+
+template <class T>
+int32_t launch_gemm(const GemmArgs& g, T* c, const T* a, const T* b, int64_t batch, hipStream_t stream) {
+    const int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
+    if (blocks == 0) return DNH_OK;
+    if (blocks > 0x7FFFFFFF) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: too many output tiles");
+    constexpr int V = 16 / (int)sizeof(T);
+    bool fast = g.sak == 1 && g.sbn == 1 && (g.M % BM) == 0 && (g.N % BN) == 0 && (g.K % kBK<T>) == 0 && g.K > 0 &&
+                (g.sam % V) == 0 && (g.sbk % V) == 0 && aligned_to(a, 16) && aligned_to(b, 16);
+    for (int d = 0; d < g.nbatch && fast; d++) fast = (g.bsa[d] % V) == 0 && (g.bsb[d] % V) == 0;
+    if (fast) hipLaunchKernelGGL((gemm_kernel<T, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+    else hipLaunchKernelGGL((gemm_kernel<T, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+    DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
+
+}  // namespace
+
+extern "C" int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream) {
+    DNH_TRY(ensure_init());
+    DNH_TRY(check_tensor(t, "dnh_dot"));
+    DNH_TRY(check_tensor(a, "dnh_dot"));
+    DNH_TRY(check_tensor(b, "dnh_dot"));
+    if (t->dtype != a->dtype || t->dtype != b->dtype) return fail(DNH_ERR_INVALID_ARG, "dnh_dot: dtypes differ");
+    if (t->dtype != DNH_F32 && t->dtype != DNH_F64)
+        return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: only single and double have a device kernel; the frontend computes other types as multiply + sumAxis (Host/HostBackend.fs:544-546)");
+    const int nt = t->ndims, na = a->ndims, nb = b->ndims;
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    int64_t batch = 1;
+    if (nt == 0 && na == 1 && nb == 1) {
+        if (a->shape[0] != b->shape[0]) return fail(DNH_ERR_INVALID_ARG, "dnh_dot: vector lengths differ");
+        g.M = 1; g.N = 1; g.K = a->shape[0];
+        g.sak = a->stride[0]; g.sbk = b->stride[0];
+    } else if (nt == 1 && na == 2 && nb == 1) {
+        if (t->shape[0] != a->shape[0] || a->shape[1] != b->shape[0]) return fail(DNH_ERR_INVALID_ARG, "dnh_dot: matrix-vector shapes do not agree");
+        g.M = a->shape[0]; g.N = 1; g.K = a->shape[1];
+        g.sam = a->stride[0]; g.sak = a->stride[1]; g.sbk = b->stride[0]; g.scm = t->stride[0];
+    } else if (nt >= 2 && na == nt && nb == nt) {
+        g.M = a->shape[na - 2]; g.K = a->shape[na - 1]; g.N = b->shape[nb - 1];
+        if (b->shape[nb - 2] != g.K || t->shape[nt - 2] != g.M || t->shape[nt - 1] != g.N)
+            return fail(DNH_ERR_INVALID_ARG, "dnh_dot: matrix shapes do not agree");
+        g.sam = a->stride[na - 2]; g.sak = a->stride[na - 1];
+        g.sbk = b->stride[nb - 2]; g.sbn = b->stride[nb - 1];
+        g.scm = t->stride[nt - 2]; g.scn = t->stride[nt - 1];
+        for (int d = 0; d < nt - 2; d++) {
+            if (a->shape[d] != t->shape[d] || b->shape[d] != t->shape[d]) return fail(DNH_ERR_INVALID_ARG, "dnh_dot: batch dimensions are not broadcast to the target's");
+            if (t->shape[d] == 1) continue;
+            if (t->shape[d] > 0xFFFFFFFFLL) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: batch extent too large");
+            g.bshape[g.nbatch] = (uint32_t)t->shape[d];
+            g.bsa[g.nbatch] = a->stride[d];
+            g.bsb[g.nbatch] = b->stride[d];
+            g.bsc[g.nbatch] = t->stride[d];
+            g.nbatch++;
+            batch *= t->shape[d];
+        }
+    } else {
+        return fail(DNH_ERR_INVALID_ARG, "dnh_dot: ranks (%d, %d, %d) match no dot variant", nt, na, nb);
+    }
+    if (g.M == 0 || g.N == 0 || batch == 0) return DNH_OK;
+    g.tiles_m = cdiv(g.M, BM);
+    g.tiles_n = cdiv(g.N, BN);
+    hipStream_t s = (hipStream_t)stream;
+    if (t->dtype == DNH_F32) return launch_gemm<float>(g, (float*)elem_ptr(t), (const float*)elem_ptr(a), (const float*)elem_ptr(b), batch, s);
+    return launch_gemm<double>(g, (double*)elem_ptr(t), (const double*)elem_ptr(a), (const double*)elem_ptr(b), batch, s);
+}

@@ -1,0 +1,55 @@
+// dnh_binary: ITensorBackend Add..MinElemwise, And/Or/Xor (Tensor/Tensor/TensorBackend.fs:97-104, 114-116).
+#include "map_kernels.h"
+#include "ops.h"
+
+using namespace dnh;
+
+namespace {
+
+template <template <class> class OpT>
+int32_t run_numeric(int dt, const MapPlan& p, hipStream_t s) {
+    switch (dt) {
+        case DNH_U8: return launch_map(OpT<uint8_t>{}, p, s);
+        case DNH_I8: return launch_map(OpT<int8_t>{}, p, s);
+        case DNH_I32: return launch_map(OpT<int32_t>{}, p, s);
+        case DNH_U32: return launch_map(OpT<uint32_t>{}, p, s);
+        case DNH_I64: return launch_map(OpT<int64_t>{}, p, s);
+        case DNH_U64: return launch_map(OpT<uint64_t>{}, p, s);
+        case DNH_F32: return launch_map(OpT<float>{}, p, s);
+        case DNH_F64: return launch_map(OpT<double>{}, p, s);
+    }
+    return fail(DNH_ERR_NOT_SUPPORTED, "binary arithmetic op is not defined for %s", dtype_name(dt));
+}
+
+}  // namespace
+
+extern "C" int32_t dnh_binary(int32_t op, const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream) {
+    DNH_TRY(ensure_init());
+    const DnhTensor* ops[3] = {t, a, b};
+    MapPlan p;
+    DNH_TRY(make_map_plan(&p, 3, ops, "dnh_binary"));
+    if (t->dtype != a->dtype || t->dtype != b->dtype)
+        return fail(DNH_ERR_INVALID_ARG, "dnh_binary: operand dtypes differ (%s, %s, %s)", dtype_name(t->dtype), dtype_name(a->dtype), dtype_name(b->dtype));
+    hipStream_t s = (hipStream_t)stream;
+    const int dt = t->dtype;
+    if (op == DNH_AND || op == DNH_OR || op == DNH_XOR) {
+        if (dt != DNH_BOOL) return fail(DNH_ERR_NOT_SUPPORTED, "logic op on %s", dtype_name(dt));
+        if (op == DNH_AND) return launch_map(OpAnd{}, p, s);
+        if (op == DNH_OR) return launch_map(OpOr{}, p, s);
+        return launch_map(OpXor{}, p, s);
+    }
+    switch (op) {
+        case DNH_ADD: return run_numeric<OpAdd>(dt, p, s);
+        case DNH_SUBTRACT: return run_numeric<OpSub>(dt, p, s);
+        case DNH_MULTIPLY: return run_numeric<OpMul>(dt, p, s);
+        case DNH_DIVIDE: return run_numeric<OpDiv>(dt, p, s);
+        case DNH_MODULO: return run_numeric<OpMod>(dt, p, s);
+        case DNH_MAX_ELEMWISE: return run_numeric<OpMax>(dt, p, s);
+        case DNH_MIN_ELEMWISE: return run_numeric<OpMin>(dt, p, s);
+        case DNH_POWER:
+            if (dt == DNH_F32) return launch_map(OpPow<float>{}, p, s);
+            if (dt == DNH_F64) return launch_map(OpPow<double>{}, p, s);
+            return fail(DNH_ERR_NOT_SUPPORTED, "Power is defined for single and double only, not %s", dtype_name(dt));
+    }
+    return fail(DNH_ERR_INVALID_ARG, "dnh_binary: unknown op %d", op);
+}

@@ -1,0 +1,379 @@
+// dnh_gather, dnh_scatter, dnh_masked_get, dnh_masked_set, dnh_true_indices:
+// ITensorBackend Gather / Scatter / MaskedGet / MaskedSet / TrueIndices (Tensor/Tensor/TensorBackend.fs:119-123);
+// semantics Tensor/Tensor/Host/ScalarOps.fs:583-604 and :667-707.
+//
+// Gather/Scatter: one lane per target (gather) or source (scatter) element; an index outside the indexed tensor sets the
+// library's error word and skips the element (the host reference raises, Host/FastAccess.fs:51-61).
+// MaskedGet/MaskedSet/TrueIndices are order-preserving stream compactions over the row-major element order:
+//   pass 1 counts selected elements per 4096-element block, pass 2 scans the block counts (one block),
+//   pass 3 re-evaluates the selection, ranks within the block (wavefront shuffle scan + LDS) and moves the data.
+#include "map_kernels.h"
+
+using namespace dnh;
+
+namespace {
+
+struct Lay {
+    int nd;
+    uint32_t shape[DNH_MAX_DIMS];
+    int64_t stride[DNH_MAX_DIMS];
+};
+
+Lay lay_of(const DnhTensor* t) {
+    Lay l;
+    l.nd = t->ndims;
+    for (int d = 0; d < DNH_MAX_DIMS; d++) {
+        l.shape[d] = d < t->ndims ? (uint32_t)t->shape[d] : 1;
+        l.stride[d] = d < t->ndims ? t->stride[d] : 0;
+    }
+    return l;
+}
+
+// row-major position of linear index i; returns the element offset
+__device__ __forceinline__ int64_t unravel(const Lay& l, uint32_t i, uint32_t* pos) {
+    int64_t off = 0;
+    for (int d = l.nd - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : i / l.shape[d];
+        const uint32_t p = i - q * l.shape[d];
+        i = q;
+        pos[d] = p;
+        off += (int64_t)p * l.stride[d];
+    }
+    return off;
+}
+__device__ __forceinline__ int64_t offset_of(const Lay& l, uint32_t i) {
+    int64_t off = 0;
+    for (int d = l.nd - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : i / l.shape[d];
+        off += (int64_t)(i - q * l.shape[d]) * l.stride[d];
+        i = q;
+    }
+    return off;
+}
+
+// ---- gather / scatter -------------------------------------------------------------------------------------------------------
+
+struct IndexArgs {
+    Lay iter;                              // the iteration space: target (gather) or source (scatter)
+    Lay other;                             // the indexed tensor: source (gather) or target (scatter)
+    const int64_t* idx[DNH_MAX_DIMS];      // per dimension of `other`; nullptr = identity
+    int64_t idx_stride[DNH_MAX_DIMS][DNH_MAX_DIMS];
+};
+
+__device__ __forceinline__ bool indexed_offset(const IndexArgs& a, const uint32_t* pos, int64_t* off) {
+    int64_t o = 0;
+    bool ok = true;
+    for (int d = 0; d < a.other.nd; d++) {
+        int64_t j;
+        if (a.idx[d]) {
+            int64_t io = 0;
+            for (int e = 0; e < a.iter.nd; e++) io += (int64_t)pos[e] * a.idx_stride[d][e];
+            j = a.idx[d][io];
+        } else {
+            j = pos[d];
+        }
+        ok = ok && j >= 0 && j < (int64_t)a.other.shape[d];
+        o += j * a.other.stride[d];
+    }
+    *off = o;
+    return ok;
+}
+
+template <class W>
+__global__ __launch_bounds__(kBlock) void gather_kernel(W* t, const W* s, IndexArgs a, uint32_t n, int32_t* err) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    uint32_t pos[DNH_MAX_DIMS];
+    const int64_t toff = unravel(a.iter, i, pos);
+    int64_t soff;
+    if (indexed_offset(a, pos, &soff)) t[toff] = s[soff];
+    else *err = 1;
+}
+
+template <class X> __device__ __forceinline__ void atomic_add_any(X* p, X v) { atomicAdd(p, v); }
+template <> __device__ __forceinline__ void atomic_add_any<int64_t>(int64_t* p, int64_t v) { atomicAdd((unsigned long long*)p, (unsigned long long)v); }
+template <> __device__ __forceinline__ void atomic_add_any<uint64_t>(uint64_t* p, uint64_t v) { atomicAdd((unsigned long long*)p, (unsigned long long)v); }
+// one-byte integers: compare-and-swap on the containing 32-bit word
+template <> __device__ __forceinline__ void atomic_add_any<uint8_t>(uint8_t* p, uint8_t v) {
+    uint32_t* w = (uint32_t*)((uintptr_t)p & ~(uintptr_t)3);
+    const unsigned sh = ((uintptr_t)p & 3) * 8;
+    uint32_t old = *w, assumed;
+    do {
+        assumed = old;
+        const uint32_t b = ((assumed >> sh) + v) & 0xFFu;
+        old = atomicCAS(w, assumed, (assumed & ~(0xFFu << sh)) | (b << sh));
+    } while (old != assumed);
+}
+
+template <class X>
+__global__ __launch_bounds__(kBlock) void scatter_kernel(X* t, const X* s, IndexArgs a, uint32_t n, int32_t* err) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= n) return;
+    uint32_t pos[DNH_MAX_DIMS];
+    const int64_t soff = unravel(a.iter, i, pos);
+    int64_t toff;
+    if (indexed_offset(a, pos, &toff)) atomic_add_any<X>(t + toff, s[soff]);
+    else *err = 1;
+}
+
+int32_t make_index_args(IndexArgs* a, const DnhTensor* iter, const DnhTensor* other, const DnhTensor* const* idx, int32_t n_idx, const char* what) {
+    DNH_TRY(check_tensor(iter, what));
+    DNH_TRY(check_tensor(other, what));
+    if (iter->dtype != other->dtype) return fail(DNH_ERR_INVALID_ARG, "%s: source and target dtypes differ", what);
+    if (n_idx != other->ndims) return fail(DNH_ERR_INVALID_ARG, "%s: %d index tensors given for a tensor of rank %d", what, n_idx, other->ndims);
+    if (n_idx > 0 && !idx) return fail(DNH_ERR_INVALID_ARG, "%s: null index list", what);
+    memset(a, 0, sizeof(*a));
+    a->iter = lay_of(iter);
+    a->other = lay_of(other);
+    for (int d = 0; d < n_idx; d++) {
+        if (idx[d]) {
+            DNH_TRY(check_tensor(idx[d], what));
+            if (idx[d]->dtype != DNH_I64) return fail(DNH_ERR_INVALID_ARG, "%s: index tensors must be int64", what);
+            if (!same_shape(idx[d], iter)) return fail(DNH_ERR_INVALID_ARG, "%s: index tensor %d is not broadcast to the iteration shape", what, d);
+            a->idx[d] = (const int64_t*)elem_ptr(idx[d]);
+            for (int e = 0; e < iter->ndims; e++) a->idx_stride[d][e] = idx[d]->stride[e];
+        } else if (d >= iter->ndims) {
+            return fail(DNH_ERR_INVALID_ARG, "%s: dimension %d has no index tensor and no matching dimension to map identically", what, d);
+        }
+    }
+    return DNH_OK;
+}
+
+// ---- compaction -------------------------------------------------------------------------------------------------------------
+
+constexpr int kItems = 16;                     // consecutive elements per thread
+constexpr int kChunk = kBlock * kItems;        // elements per block
+
+struct MaskArgs {
+    Lay full;                                  // the masked tensor (source of MaskedGet, target of MaskedSet, source of TrueIndices)
+    const uint8_t* mask[DNH_MAX_DIMS];         // per-dimension rank-1 masks (nullptr = all true) — or mask[0] = the bool tensor itself
+    int64_t mask_stride[DNH_MAX_DIMS];
+    int whole;                                 // 1: mask[0] is a bool tensor with layout `full` (TrueIndices)
+};
+
+__device__ __forceinline__ bool selected(const MaskArgs& m, const uint32_t* pos, int64_t off) {
+    if (m.whole) return m.mask[0][off] != 0;
+    bool s = true;
+    for (int d = 0; d < m.full.nd; d++)
+        if (m.mask[d]) s = s && m.mask[d][(int64_t)pos[d] * m.mask_stride[d]] != 0;
+    return s;
+}
+
+// exclusive prefix of `c` over the block; `total` receives the block sum
+__device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t c, uint32_t* total) {
+    __shared__ uint32_t wave_sum[kBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inc = c;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t y = (uint32_t)__shfl_up((int)inc, d, 64);
+        if (lane >= d) inc += y;
+    }
+    if (lane == 63) wave_sum[wave] = inc;
+    __syncthreads();
+    uint32_t base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; w++) {
+        if (w < wave) base += wave_sum[w];
+        tot += wave_sum[w];
+    }
+    *total = tot;
+    return base + inc - c;
+}
+
+__global__ __launch_bounds__(kBlock) void compact_count_kernel(MaskArgs m, uint32_t n, uint32_t* counts) {
+    const uint32_t i0 = blockIdx.x * (uint32_t)kChunk + threadIdx.x * kItems;
+    uint32_t c = 0;
+    if (i0 < n) {
+        if (m.full.nd == 1 && !m.whole && m.mask[0] && m.mask_stride[0] == 1 && i0 + kItems <= n && (((uintptr_t)(m.mask[0] + i0)) & 15) == 0) {
+            const Pack<uint8_t, kItems> v = load_pack<uint8_t, kItems>(m.mask[0] + i0);
+#pragma unroll
+            for (int e = 0; e < kItems; e++) c += v.v[e] != 0;
+        } else {
+            for (int e = 0; e < kItems && i0 + e < n; e++) {
+                uint32_t pos[DNH_MAX_DIMS];
+                const int64_t off = unravel(m.full, i0 + e, pos);
+                c += selected(m, pos, off);
+            }
+        }
+    }
+    uint32_t total;
+    block_exclusive_scan(c, &total);
+    if (threadIdx.x == 0) counts[blockIdx.x] = total;
+}
+
+// in-place exclusive scan of counts[0..nb) by one block
+__global__ __launch_bounds__(kBlock) void compact_scan_kernel(uint32_t* counts, uint32_t nb) {
+    const uint32_t seg = (nb + kBlock - 1) / kBlock;
+    const uint32_t b0 = threadIdx.x * seg;
+    uint32_t sum = 0;
+    for (uint32_t i = b0; i < b0 + seg && i < nb; i++) sum += counts[i];
+    uint32_t total;
+    uint32_t run = block_exclusive_scan(sum, &total);
+    for (uint32_t i = b0; i < b0 + seg && i < nb; i++) {
+        const uint32_t c = counts[i];
+        counts[i] = run;
+        run += c;
+    }
+}
+
+enum CompactMode { kMaskedGet = 0, kMaskedSet = 1, kTrueIndices = 2 };
+
+// MODE kMaskedGet : out[k]        = full[i]      for the k-th selected element i
+//      kMaskedSet : full[i]       = out[k]       (`out` is the value tensor)
+//      kTrueIndices: out[k, 0..nd) = position of i
+template <class W, int MODE>
+__global__ __launch_bounds__(kBlock) void compact_move_kernel(MaskArgs m, W* full, W* out, Lay olay, uint32_t n, uint32_t nout,
+                                                              const uint32_t* block_base) {
+    const uint32_t i0 = blockIdx.x * (uint32_t)kChunk + threadIdx.x * kItems;
+    uint32_t flags = 0, c = 0;
+    if (i0 < n) {
+        if (m.full.nd == 1 && !m.whole && m.mask[0] && m.mask_stride[0] == 1 && i0 + kItems <= n && (((uintptr_t)(m.mask[0] + i0)) & 15) == 0) {
+            const Pack<uint8_t, kItems> v = load_pack<uint8_t, kItems>(m.mask[0] + i0);
+#pragma unroll
+            for (int e = 0; e < kItems; e++) flags |= (uint32_t)(v.v[e] != 0) << e;
+        } else {
+            for (int e = 0; e < kItems && i0 + e < n; e++) {
+                uint32_t pos[DNH_MAX_DIMS];
+                const int64_t off = unravel(m.full, i0 + e, pos);
+                flags |= (uint32_t)selected(m, pos, off) << e;
+            }
+        }
+        c = __popc(flags);
+    }
+    uint32_t total;
+    uint32_t k = block_base[blockIdx.x] + block_exclusive_scan(c, &total);
+    while (flags) {
+        const int e = __ffs(flags) - 1;
+        flags &= flags - 1;
+        if (k < nout) {
+            uint32_t pos[DNH_MAX_DIMS];
+            const int64_t foff = unravel(m.full, i0 + e, pos);
+            if constexpr (MODE == kMaskedGet) out[offset_of(olay, k)] = full[foff];
+            else if constexpr (MODE == kMaskedSet) full[foff] = out[offset_of(olay, k)];
+            else {
+                for (int d = 0; d < m.full.nd; d++) out[(int64_t)k * olay.stride[0] + (int64_t)d * olay.stride[1]] = (W)pos[d];
+            }
+        }
+        k++;
+    }
+}
+
+template <int MODE>
+int32_t run_compaction(const MaskArgs& m, void* full, void* out, const Lay& olay, int esize, int64_t n64, int64_t nout64, hipStream_t stream) {
+    if (n64 == 0 || nout64 == 0) return DNH_OK;
+    if (n64 > (int64_t)kMaxItems) return fail(DNH_ERR_NOT_SUPPORTED, "masked op over more than 2^32 elements");
+    const uint32_t n = (uint32_t)n64;
+    const uint32_t nout = (uint32_t)(nout64 > (int64_t)kMaxItems ? kMaxItems : nout64);
+    const uint32_t nb = cdiv(n, kChunk);
+    uint32_t* counts;
+    DNH_TRY(workspace(stream, sizeof(uint32_t) * (size_t)nb, (void**)&counts));
+    hipLaunchKernelGGL(compact_count_kernel, dim3(nb), dim3(kBlock), 0, stream, m, n, counts);
+    DNH_LAUNCH_CHECK();
+    hipLaunchKernelGGL(compact_scan_kernel, dim3(1), dim3(kBlock), 0, stream, counts, nb);
+    DNH_LAUNCH_CHECK();
+    switch (esize) {
+        case 1: hipLaunchKernelGGL((compact_move_kernel<uint8_t, MODE>), dim3(nb), dim3(kBlock), 0, stream, m, (uint8_t*)full, (uint8_t*)out, olay, n, nout, counts); break;
+        case 4: hipLaunchKernelGGL((compact_move_kernel<uint32_t, MODE>), dim3(nb), dim3(kBlock), 0, stream, m, (uint32_t*)full, (uint32_t*)out, olay, n, nout, counts); break;
+        case 8: hipLaunchKernelGGL((compact_move_kernel<uint64_t, MODE>), dim3(nb), dim3(kBlock), 0, stream, m, (uint64_t*)full, (uint64_t*)out, olay, n, nout, counts); break;
+        default: return fail(DNH_ERR_NOT_SUPPORTED, "masked op: unsupported element width");
+    }
+    DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
+
+int32_t make_mask_args(MaskArgs* m, const DnhTensor* full, const DnhTensor* const* masks, int32_t n_masks, const char* what) {
+    memset(m, 0, sizeof(*m));
+    m->full = lay_of(full);
+    if (n_masks != full->ndims) return fail(DNH_ERR_INVALID_ARG, "%s: %d masks given for a tensor of rank %d", what, n_masks, full->ndims);
+    if (n_masks > 0 && !masks) return fail(DNH_ERR_INVALID_ARG, "%s: null mask list", what);
+    for (int d = 0; d < n_masks; d++) {
+        if (!masks[d]) continue;
+        DNH_TRY(check_tensor(masks[d], what));
+        if (masks[d]->dtype != DNH_BOOL || masks[d]->ndims != 1 || masks[d]->shape[0] != full->shape[d])
+            return fail(DNH_ERR_INVALID_ARG, "%s: mask %d must be a rank-1 bool tensor of length %lld", what, d, (long long)full->shape[d]);
+        m->mask[d] = (const uint8_t*)elem_ptr(masks[d]);
+        m->mask_stride[d] = masks[d]->stride[0];
+    }
+    return DNH_OK;
+}
+
+}  // namespace
+
+extern "C" int32_t dnh_gather(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    IndexArgs a;
+    DNH_TRY(make_index_args(&a, t, src, idx, n_idx, "dnh_gather"));
+    const int64_t n = nelems(t);
+    if (n == 0) return DNH_OK;
+    if (n > (int64_t)kMaxItems) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_gather: more than 2^32 elements");
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(cdiv(n, kBlock));
+    switch (dtype_size(t->dtype)) {
+        case 1: hipLaunchKernelGGL(gather_kernel<uint8_t>, grid, dim3(kBlock), 0, s, (uint8_t*)elem_ptr(t), (const uint8_t*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
+        case 4: hipLaunchKernelGGL(gather_kernel<uint32_t>, grid, dim3(kBlock), 0, s, (uint32_t*)elem_ptr(t), (const uint32_t*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
+        case 8: hipLaunchKernelGGL(gather_kernel<uint64_t>, grid, dim3(kBlock), 0, s, (uint64_t*)elem_ptr(t), (const uint64_t*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
+        default: return fail(DNH_ERR_NOT_SUPPORTED, "dnh_gather: unsupported element width");
+    }
+    DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
+
+extern "C" int32_t dnh_scatter(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    IndexArgs a;
+    DNH_TRY(make_index_args(&a, src, t, idx, n_idx, "dnh_scatter"));
+    const int64_t n = nelems(src);
+    if (n == 0) return DNH_OK;
+    if (n > (int64_t)kMaxItems) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_scatter: more than 2^32 elements");
+    hipStream_t s = (hipStream_t)stream;
+    const dim3 grid(cdiv(n, kBlock));
+#define CASE(DT, X) case DT: hipLaunchKernelGGL(scatter_kernel<X>, grid, dim3(kBlock), 0, s, (X*)elem_ptr(t), (const X*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
+    switch (t->dtype) {
+        CASE(DNH_U8, uint8_t)
+        case DNH_I8: hipLaunchKernelGGL(scatter_kernel<uint8_t>, grid, dim3(kBlock), 0, s, (uint8_t*)elem_ptr(t), (const uint8_t*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
+        CASE(DNH_I32, int32_t) CASE(DNH_U32, uint32_t) CASE(DNH_I64, int64_t) CASE(DNH_U64, uint64_t) CASE(DNH_F32, float) CASE(DNH_F64, double)
+        default: return fail(DNH_ERR_NOT_SUPPORTED, "dnh_scatter on %s", dtype_name(t->dtype));
+    }
+#undef CASE
+    DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
+
+extern "C" int32_t dnh_masked_get(const DnhTensor* t, const DnhTensor* src, const DnhTensor* const* masks, int32_t n_masks, void* stream) {
+    DNH_TRY(ensure_init());
+    DNH_TRY(check_tensor(t, "dnh_masked_get"));
+    DNH_TRY(check_tensor(src, "dnh_masked_get"));
+    if (t->dtype != src->dtype) return fail(DNH_ERR_INVALID_ARG, "dnh_masked_get: dtypes differ");
+    MaskArgs m;
+    DNH_TRY(make_mask_args(&m, src, masks, n_masks, "dnh_masked_get"));
+    return run_compaction<kMaskedGet>(m, elem_ptr(src), elem_ptr(t), lay_of(t), dtype_size(t->dtype), nelems(src), nelems(t), (hipStream_t)stream);
+}
+
+extern "C" int32_t dnh_masked_set(const DnhTensor* t, const DnhTensor* const* masks, int32_t n_masks, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    DNH_TRY(check_tensor(t, "dnh_masked_set"));
+    DNH_TRY(check_tensor(src, "dnh_masked_set"));
+    if (t->dtype != src->dtype) return fail(DNH_ERR_INVALID_ARG, "dnh_masked_set: dtypes differ");
+    MaskArgs m;
+    DNH_TRY(make_mask_args(&m, t, masks, n_masks, "dnh_masked_set"));
+    return run_compaction<kMaskedSet>(m, elem_ptr(t), elem_ptr(src), lay_of(src), dtype_size(t->dtype), nelems(t), nelems(src), (hipStream_t)stream);
+}
+
+extern "C" int32_t dnh_true_indices(const DnhTensor* t, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    DNH_TRY(check_tensor(t, "dnh_true_indices"));
+    DNH_TRY(check_tensor(src, "dnh_true_indices"));
+    if (t->dtype != DNH_I64 || src->dtype != DNH_BOOL) return fail(DNH_ERR_INVALID_ARG, "dnh_true_indices: needs an int64 target and a bool source");
+    if (t->ndims != 2 || t->shape[1] != src->ndims) return fail(DNH_ERR_INVALID_ARG, "dnh_true_indices: target must have shape [nTrue; %d]", src->ndims);
+    MaskArgs m;
+    memset(&m, 0, sizeof(m));
+    m.full = lay_of(src);
+    m.whole = 1;
+    m.mask[0] = (const uint8_t*)elem_ptr(src);
+    if (src->ndims == 0) {
+        // a 0-d source has one element and no coordinates: nothing to write
+        return DNH_OK;
+    }
+    return run_compaction<kTrueIndices>(m, nullptr, elem_ptr(t), lay_of(t), 8, nelems(src), t->shape[0], (hipStream_t)stream);
+}

@@ -1,0 +1,393 @@
+// Element-wise map kernels (target + up to three sources) for gfx950 and the launcher that picks one from a MapPlan.
+//
+//  map_flat  : every operand is one contiguous run (or a stride-0 scalar): 16-byte loads/stores per lane, several in
+//              flight per thread, one pass over HBM.
+//  map_nd    : collapsed n-d strided operands; lanes run along the target's fastest dimension (coalesced stores), 16-byte
+//              vectors when the last dimension allows it, per-item index decomposition in 32-bit arithmetic.
+//  map_tr    : a source whose unit-stride dimension differs from the target's is staged through LDS in 64x64 (32x32 for
+//              8-byte elements) tiles: global reads run along the source's fast dimension, global writes along the target's.
+//
+// An Op is a small functor: `using T/A/B/C` (target and source element types, `char` when absent), `NSRC`, and
+// `__device__ T operator()(A[,B[,C]]) const`.  State (a fill value) travels by value as a kernel argument.
+#pragma once
+
+#include "common.h"
+
+namespace dnh {
+
+constexpr int kBlock = 256;
+
+// raw N-byte words for vector memory access
+template <int BYTES> struct RawWord;
+template <> struct RawWord<1> { using type = uint8_t; };
+template <> struct RawWord<2> { using type = uint16_t; };
+template <> struct RawWord<4> { using type = uint32_t; };
+template <> struct RawWord<8> { typedef uint32_t type __attribute__((ext_vector_type(2))); };
+template <> struct RawWord<16> { typedef uint32_t type __attribute__((ext_vector_type(4))); };
+
+template <class T, int N>
+struct Pack {
+    T v[N];
+};
+
+template <class T, int N>
+__device__ __forceinline__ Pack<T, N> load_pack(const T* p) {
+    using W = typename RawWord<sizeof(T) * N>::type;
+    W w = __builtin_nontemporal_load((const W*)p);
+    Pack<T, N> r;
+    __builtin_memcpy(&r, &w, sizeof(w));
+    return r;
+}
+
+template <class T, int N>
+__device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& r) {
+    using W = typename RawWord<sizeof(T) * N>::type;
+    W w;
+    __builtin_memcpy(&w, &r, sizeof(w));
+    __builtin_nontemporal_store(w, (W*)p);
+}
+
+template <class T, int N>
+__device__ __forceinline__ Pack<T, N> splat_pack(T x) {
+    Pack<T, N> r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = x;
+    return r;
+}
+
+template <class Op>
+__device__ __forceinline__ typename Op::T apply_op(const Op& op, typename Op::A a, typename Op::B b, typename Op::C c) {
+    if constexpr (Op::NSRC == 0) return op();
+    else if constexpr (Op::NSRC == 1) return op(a);
+    else if constexpr (Op::NSRC == 2) return op(a, b);
+    else return op(a, b, c);
+}
+
+// ---- flat ---------------------------------------------------------------------------------------------------------------
+
+template <class Op, int VEC, int UNROLL>
+__global__ __launch_bounds__(kBlock) void map_flat_kernel(Op op, typename Op::T* __restrict__ t, const typename Op::A* a,
+                                                          const typename Op::B* b, const typename Op::C* c, int sa, int sb, int sc,
+                                                          int64_t n) {
+    using T = typename Op::T;
+    using A = typename Op::A;
+    using B = typename Op::B;
+    using C = typename Op::C;
+    const int64_t nvec = n / VEC;
+    const int64_t base = (int64_t)blockIdx.x * (kBlock * UNROLL) + threadIdx.x;
+    Pack<A, VEC> va[UNROLL];
+    Pack<B, VEC> vb[UNROLL];
+    Pack<C, VEC> vc[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const int64_t i = base + (int64_t)u * kBlock;
+        if (i < nvec) {
+            if constexpr (Op::NSRC >= 1) va[u] = sa ? load_pack<A, VEC>(a + i * VEC) : splat_pack<A, VEC>(a[0]);
+            if constexpr (Op::NSRC >= 2) vb[u] = sb ? load_pack<B, VEC>(b + i * VEC) : splat_pack<B, VEC>(b[0]);
+            if constexpr (Op::NSRC >= 3) vc[u] = sc ? load_pack<C, VEC>(c + i * VEC) : splat_pack<C, VEC>(c[0]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const int64_t i = base + (int64_t)u * kBlock;
+        if (i < nvec) {
+            Pack<T, VEC> r;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) r.v[e] = apply_op(op, va[u].v[e], vb[u].v[e], vc[u].v[e]);
+            store_pack<T, VEC>(t + i * VEC, r);
+        }
+    }
+    // the n % VEC trailing elements
+    if (blockIdx.x == 0) {
+        const int64_t i = nvec * VEC + threadIdx.x;
+        if (threadIdx.x < VEC && i < n) {
+            A xa = A();
+            B xb = B();
+            C xc = C();
+            if constexpr (Op::NSRC >= 1) xa = a[sa ? i : 0];
+            if constexpr (Op::NSRC >= 2) xb = b[sb ? i : 0];
+            if constexpr (Op::NSRC >= 3) xc = c[sc ? i : 0];
+            t[i] = apply_op(op, xa, xb, xc);
+        }
+    }
+}
+
+// ---- n-d ----------------------------------------------------------------------------------------------------------------
+
+struct NdArgs {
+    int nd;                                      // >= 1
+    uint32_t shape[DNH_MAX_DIMS];                // shape[nd-1] counts items of VEC elements
+    int64_t stride[kMaxOperands][DNH_MAX_DIMS];  // element strides; last dimension already multiplied by VEC
+    int vecload[kMaxOperands];                   // source k is read as a vector (last-dim stride 1) rather than splat (stride 0)
+};
+
+template <class Op, int VEC, int UNROLL>
+__global__ __launch_bounds__(kBlock) void map_nd_kernel(Op op, typename Op::T* t, const typename Op::A* a, const typename Op::B* b,
+                                                        const typename Op::C* c, NdArgs p, uint32_t nitems) {
+    using T = typename Op::T;
+    using A = typename Op::A;
+    using B = typename Op::B;
+    using C = typename Op::C;
+    const uint32_t base = blockIdx.x * (uint32_t)(kBlock * UNROLL) + threadIdx.x;
+    int64_t ot[UNROLL], oa[UNROLL], ob[UNROLL], oc[UNROLL];
+    Pack<A, VEC> va[UNROLL];
+    Pack<B, VEC> vb[UNROLL];
+    Pack<C, VEC> vc[UNROLL];
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const uint32_t item = base + (uint32_t)u * kBlock;
+        ot[u] = oa[u] = ob[u] = oc[u] = 0;
+        if (item < nitems) {
+            uint32_t rem = item;
+            for (int d = p.nd - 1; d >= 0; d--) {
+                uint32_t q = (d == 0) ? 0u : rem / p.shape[d];
+                uint32_t idx = rem - q * p.shape[d];
+                rem = q;
+                ot[u] += (int64_t)idx * p.stride[0][d];
+                if constexpr (Op::NSRC >= 1) oa[u] += (int64_t)idx * p.stride[1][d];
+                if constexpr (Op::NSRC >= 2) ob[u] += (int64_t)idx * p.stride[2][d];
+                if constexpr (Op::NSRC >= 3) oc[u] += (int64_t)idx * p.stride[3][d];
+            }
+            if constexpr (VEC == 1) {
+                if constexpr (Op::NSRC >= 1) va[u].v[0] = a[oa[u]];
+                if constexpr (Op::NSRC >= 2) vb[u].v[0] = b[ob[u]];
+                if constexpr (Op::NSRC >= 3) vc[u].v[0] = c[oc[u]];
+            } else {
+                if constexpr (Op::NSRC >= 1) va[u] = p.vecload[1] ? load_pack<A, VEC>(a + oa[u]) : splat_pack<A, VEC>(a[oa[u]]);
+                if constexpr (Op::NSRC >= 2) vb[u] = p.vecload[2] ? load_pack<B, VEC>(b + ob[u]) : splat_pack<B, VEC>(b[ob[u]]);
+                if constexpr (Op::NSRC >= 3) vc[u] = p.vecload[3] ? load_pack<C, VEC>(c + oc[u]) : splat_pack<C, VEC>(c[oc[u]]);
+            }
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UNROLL; u++) {
+        const uint32_t item = base + (uint32_t)u * kBlock;
+        if (item < nitems) {
+            Pack<T, VEC> r;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) r.v[e] = apply_op(op, va[u].v[e], vb[u].v[e], vc[u].v[e]);
+            if constexpr (VEC == 1) t[ot[u]] = r.v[0];
+            else store_pack<T, VEC>(t + ot[u], r);
+        }
+    }
+}
+
+// ---- LDS-staged transpose -------------------------------------------------------------------------------------------------
+
+struct TrArgs {
+    int nouter;                                   // dimensions other than A (staged sources' fast dim) and B (target's fast dim)
+    uint32_t oshape[DNH_MAX_DIMS];
+    int64_t ostride[kMaxOperands][DNH_MAX_DIMS];
+    uint32_t na, nb, tiles_a, tiles_b;
+    int64_t sa[kMaxOperands], sb[kMaxOperands];   // element strides along A and B
+    int staged[kMaxOperands];                     // source k goes through LDS
+};
+
+template <class Op, int TILE>
+__global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t, const typename Op::A* a, const typename Op::B* b,
+                                                        const typename Op::C* c, TrArgs p) {
+    using T = typename Op::T;
+    using A = typename Op::A;
+    using B = typename Op::B;
+    using C = typename Op::C;
+    constexpr int ROWS = kBlock / TILE;  // rows of the tile covered per pass
+    __shared__ A la[Op::NSRC >= 1 ? TILE : 1][TILE + 1];
+    __shared__ B lb[Op::NSRC >= 2 ? TILE : 1][TILE + 1];
+    __shared__ C lc[Op::NSRC >= 3 ? TILE : 1][TILE + 1];
+
+    uint32_t bid = blockIdx.x;
+    const uint32_t tb = bid % p.tiles_b;
+    bid /= p.tiles_b;
+    const uint32_t ta = bid % p.tiles_a;
+    bid /= p.tiles_a;
+    int64_t off[kMaxOperands] = {0, 0, 0, 0};
+    for (int d = p.nouter - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bid / p.oshape[d];
+        const uint32_t idx = bid - q * p.oshape[d];
+        bid = q;
+#pragma unroll
+        for (int k = 0; k <= Op::NSRC; k++) off[k] += (int64_t)idx * p.ostride[k][d];
+    }
+    const uint32_t a0 = ta * TILE, b0 = tb * TILE;
+    const uint32_t tx = threadIdx.x % TILE, ty = threadIdx.x / TILE;
+
+    // stage: lanes run along A (the staged sources' unit-stride dimension); LDS tile is [b][a]
+    {
+        const uint32_t ia = a0 + tx;
+        if (ia < p.na) {
+            for (uint32_t r = ty; r < TILE; r += ROWS) {
+                const uint32_t ib = b0 + r;
+                if (ib < p.nb) {
+                    if constexpr (Op::NSRC >= 1)
+                        if (p.staged[1]) la[r][tx] = a[off[1] + (int64_t)ia * p.sa[1] + (int64_t)ib * p.sb[1]];
+                    if constexpr (Op::NSRC >= 2)
+                        if (p.staged[2]) lb[r][tx] = b[off[2] + (int64_t)ia * p.sa[2] + (int64_t)ib * p.sb[2]];
+                    if constexpr (Op::NSRC >= 3)
+                        if (p.staged[3]) lc[r][tx] = c[off[3] + (int64_t)ia * p.sa[3] + (int64_t)ib * p.sb[3]];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    // compute + store: lanes run along B (the target's unit-stride dimension)
+    {
+        const uint32_t ib = b0 + tx;
+        if (ib < p.nb) {
+            for (uint32_t r = ty; r < TILE; r += ROWS) {
+                const uint32_t ia = a0 + r;
+                if (ia < p.na) {
+                    A xa = A();
+                    B xb = B();
+                    C xc = C();
+                    if constexpr (Op::NSRC >= 1) xa = p.staged[1] ? la[tx][r] : a[off[1] + (int64_t)ia * p.sa[1] + (int64_t)ib * p.sb[1]];
+                    if constexpr (Op::NSRC >= 2) xb = p.staged[2] ? lb[tx][r] : b[off[2] + (int64_t)ia * p.sa[2] + (int64_t)ib * p.sb[2]];
+                    if constexpr (Op::NSRC >= 3) xc = p.staged[3] ? lc[tx][r] : c[off[3] + (int64_t)ia * p.sa[3] + (int64_t)ib * p.sb[3]];
+                    t[off[0] + (int64_t)ia * p.sa[0] + (int64_t)ib * p.sb[0]] = apply_op(op, xa, xb, xc);
+                }
+            }
+        }
+    }
+}
+
+// ---- launcher -------------------------------------------------------------------------------------------------------------
+
+template <class Op>
+constexpr int op_vec() {
+    int m = (int)sizeof(typename Op::T);
+    if (Op::NSRC >= 1 && (int)sizeof(typename Op::A) > m) m = (int)sizeof(typename Op::A);
+    if (Op::NSRC >= 2 && (int)sizeof(typename Op::B) > m) m = (int)sizeof(typename Op::B);
+    if (Op::NSRC >= 3 && (int)sizeof(typename Op::C) > m) m = (int)sizeof(typename Op::C);
+    return 16 / m;
+}
+
+inline bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
+
+constexpr uint32_t kMaxItems = 0xFFFF0000u;
+
+template <class Op>
+int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
+    using T = typename Op::T;
+    using A = typename Op::A;
+    using B = typename Op::B;
+    using C = typename Op::C;
+    constexpr int VEC = op_vec<Op>();
+    constexpr int NOPS = Op::NSRC + 1;
+    if (p.total == 0) return DNH_OK;
+    T* t = (T*)p.ptr[0];
+    const A* a = (const A*)p.ptr[1];
+    const B* b = (const B*)p.ptr[2];
+    const C* c = (const C*)p.ptr[3];
+    const size_t es[kMaxOperands] = {sizeof(T), sizeof(A), sizeof(B), sizeof(C)};
+    const int nd = p.nd;
+    const int last = nd - 1;
+
+    // flat: one contiguous run per operand (or a broadcast scalar)
+    bool flat = nd <= 1;
+    if (flat && nd == 1) {
+        flat = p.stride[0][0] == 1;
+        for (int k = 1; k < NOPS; k++) flat = flat && (p.stride[k][0] == 1 || p.stride[k][0] == 0);
+    }
+    if (flat && nd == 1) {
+        bool al = aligned_to(t, VEC * es[0]);
+        for (int k = 1; k < NOPS; k++)
+            if (p.stride[k][0] == 1) al = al && aligned_to(p.ptr[k], VEC * es[k]);
+        if (al) {
+            constexpr int UNROLL = 4;
+            const int64_t nvec = p.total / VEC;
+            const unsigned blocks = nvec ? cdiv(nvec, (int64_t)kBlock * UNROLL) : 1;
+            hipLaunchKernelGGL((map_flat_kernel<Op, VEC, UNROLL>), dim3(blocks), dim3(kBlock), 0, stream, op, t, a, b, c,
+                               (int)p.stride[1][0], (int)p.stride[2][0], (int)p.stride[3][0], p.total);
+            DNH_LAUNCH_CHECK();
+            return DNH_OK;
+        }
+    }
+
+    if (nd >= 1 && p.total > (int64_t)kMaxItems) {
+        // split the outermost dimension so each launch indexes fewer than 2^32 items
+        MapPlan q = p;
+        const int64_t inner = p.total / p.shape[0];
+        if (inner > (int64_t)kMaxItems) return fail(DNH_ERR_NOT_SUPPORTED, "element-wise op: inner extent of %lld elements exceeds the 32-bit index range", (long long)inner);
+        const int64_t chunk = (int64_t)kMaxItems / inner;
+        for (int64_t s = 0; s < p.shape[0]; s += chunk) {
+            const int64_t len = (p.shape[0] - s) < chunk ? (p.shape[0] - s) : chunk;
+            q.shape[0] = len;
+            q.total = len * inner;
+            for (int k = 0; k < NOPS; k++) q.ptr[k] = p.ptr[k] + s * p.stride[k][0] * (int64_t)es[k];
+            DNH_TRY(launch_map(op, q, stream));
+        }
+        return DNH_OK;
+    }
+
+    // transposing path: the target runs along `last`, some source along another dimension
+    if (nd >= 2 && p.stride[0][last] == 1) {
+        int dA = -1;
+        for (int k = 1; k < NOPS && dA < 0; k++) {
+            if (p.stride[k][last] == 0 || p.stride[k][last] == 1) continue;
+            for (int d = 0; d < last; d++)
+                if (p.stride[k][d] == 1 && p.shape[d] >= 16) { dA = d; break; }
+        }
+        if (dA >= 0 && p.shape[last] >= 16) {
+            constexpr int TILE = (sizeof(T) > 4 || (Op::NSRC >= 1 && sizeof(A) > 4) || (Op::NSRC >= 2 && sizeof(B) > 4) ||
+                                  (Op::NSRC >= 3 && sizeof(C) > 4)) ? 32 : 64;
+            TrArgs q;
+            memset(&q, 0, sizeof(q));
+            q.na = (uint32_t)p.shape[dA];
+            q.nb = (uint32_t)p.shape[last];
+            q.tiles_a = cdiv(q.na, TILE);
+            q.tiles_b = cdiv(q.nb, TILE);
+            int64_t outer = 1;
+            for (int d = 0; d < last; d++) {
+                if (d == dA) continue;
+                q.oshape[q.nouter] = (uint32_t)p.shape[d];
+                for (int k = 0; k < NOPS; k++) q.ostride[k][q.nouter] = p.stride[k][d];
+                outer *= p.shape[d];
+                q.nouter++;
+            }
+            for (int k = 0; k < NOPS; k++) {
+                q.sa[k] = p.stride[k][dA];
+                q.sb[k] = p.stride[k][last];
+                q.staged[k] = (k >= 1 && p.stride[k][dA] == 1 && p.stride[k][last] != 0 && p.stride[k][last] != 1) ? 1 : 0;
+            }
+            const int64_t blocks = (int64_t)q.tiles_a * q.tiles_b * outer;
+            if (blocks <= 0x7FFFFFFF) {
+                hipLaunchKernelGGL((map_tr_kernel<Op, TILE>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, op, t, a, b, c, q);
+                DNH_LAUNCH_CHECK();
+                return DNH_OK;
+            }
+        }
+    }
+
+    // generic n-d
+    NdArgs q;
+    memset(&q, 0, sizeof(q));
+    q.nd = nd < 1 ? 1 : nd;
+    for (int d = 0; d < q.nd; d++) {
+        q.shape[d] = (uint32_t)p.shape[d];
+        for (int k = 0; k < NOPS; k++) q.stride[k][d] = p.stride[k][d];
+    }
+    bool vec = VEC > 1 && nd >= 1 && p.stride[0][last] == 1 && (p.shape[last] % VEC) == 0 && aligned_to(t, VEC * es[0]);
+    for (int k = 1; k < NOPS && vec; k++) {
+        vec = vec && (p.stride[k][last] == 0 || p.stride[k][last] == 1);
+        if (p.stride[k][last] == 1) vec = vec && aligned_to(p.ptr[k], VEC * es[k]);
+    }
+    for (int d = 0; d < last && vec; d++)
+        for (int k = 0; k < NOPS; k++)
+            if (p.stride[k][last] == 1) vec = vec && (p.stride[k][d] % VEC) == 0;
+    constexpr int UNROLL = 2;
+    if (vec) {
+        q.shape[last] = (uint32_t)(p.shape[last] / VEC);
+        for (int k = 0; k < NOPS; k++) {
+            q.vecload[k] = p.stride[k][last] == 1;
+            q.stride[k][last] = p.stride[k][last] * VEC;
+        }
+        const uint32_t nitems = (uint32_t)(p.total / VEC);
+        hipLaunchKernelGGL((map_nd_kernel<Op, VEC, UNROLL>), dim3(cdiv(nitems, kBlock * UNROLL)), dim3(kBlock), 0, stream, op, t, a, b, c, q, nitems);
+    } else {
+        const uint32_t nitems = (uint32_t)p.total;
+        hipLaunchKernelGGL((map_nd_kernel<Op, 1, UNROLL>), dim3(cdiv(nitems, kBlock * UNROLL)), dim3(kBlock), 0, stream, op, t, a, b, c, q, nitems);
+    }
+    DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
+
+}  // namespace dnh

@@ -1,0 +1,174 @@
+// dnh_reduce_last_axis, dnh_arg_reduce_last_axis, dnh_find_last_axis:
+// ITensorBackend SumLastAxis..CountTrueLastAxis, ArgMin/ArgMaxLastAxis, FindLastAxis (Tensor/Tensor/TensorBackend.fs:125-135).
+// Fold semantics follow Tensor/Tensor/Host/ScalarOps.fs:606-665: sum from zero, product from one, max from minValue<T>
+// with `if res > v then res else v`, min from maxValue<T>, all from true, any from false, countTrue into int64; an empty
+// axis yields the initial value.  Float sums and products are re-associated (tree order); everything else is order-independent.
+#include "reduce_kernels.h"
+#include "ops.h"
+
+using namespace dnh;
+
+namespace {
+
+template <class X> struct RSum {
+    using In = X; using State = X; using Out = X;
+    __device__ X init() const { return X(0); }
+    __device__ X step(X s, X v, int64_t) const { return OpAdd<X>{}(s, v); }
+    __device__ X combine(X a, X b) const { return OpAdd<X>{}(a, b); }
+    __device__ X extract(X s) const { return s; }
+};
+template <class X> struct RProd {
+    using In = X; using State = X; using Out = X;
+    __device__ X init() const { return X(1); }
+    __device__ X step(X s, X v, int64_t) const { return OpMul<X>{}(s, v); }
+    __device__ X combine(X a, X b) const { return OpMul<X>{}(a, b); }
+    __device__ X extract(X s) const { return s; }
+};
+template <class X> struct RMax {
+    using In = X; using State = X; using Out = X;
+    __device__ X init() const { return std::numeric_limits<X>::lowest(); }
+    __device__ X step(X s, X v, int64_t) const { return s > v ? s : v; }
+    __device__ X combine(X a, X b) const { return a > b ? a : b; }
+    __device__ X extract(X s) const { return s; }
+};
+template <class X> struct RMin {
+    using In = X; using State = X; using Out = X;
+    __device__ X init() const { return std::numeric_limits<X>::max(); }
+    __device__ X step(X s, X v, int64_t) const { return s < v ? s : v; }
+    __device__ X combine(X a, X b) const { return a < b ? a : b; }
+    __device__ X extract(X s) const { return s; }
+};
+struct RAll {
+    using In = uint8_t; using State = uint8_t; using Out = uint8_t;
+    __device__ uint8_t init() const { return 1; }
+    __device__ uint8_t step(uint8_t s, uint8_t v, int64_t) const { return (uint8_t)(s & (v != 0)); }
+    __device__ uint8_t combine(uint8_t a, uint8_t b) const { return (uint8_t)(a & b); }
+    __device__ uint8_t extract(uint8_t s) const { return s; }
+};
+struct RAny {
+    using In = uint8_t; using State = uint8_t; using Out = uint8_t;
+    __device__ uint8_t init() const { return 0; }
+    __device__ uint8_t step(uint8_t s, uint8_t v, int64_t) const { return (uint8_t)(s | (v != 0)); }
+    __device__ uint8_t combine(uint8_t a, uint8_t b) const { return (uint8_t)(a | b); }
+    __device__ uint8_t extract(uint8_t s) const { return s; }
+};
+struct RCountTrue {
+    using In = uint8_t; using State = int64_t; using Out = int64_t;
+    __device__ int64_t init() const { return 0; }
+    __device__ int64_t step(int64_t s, uint8_t v, int64_t) const { return s + (v != 0); }
+    __device__ int64_t combine(int64_t a, int64_t b) const { return a + b; }
+    __device__ int64_t extract(int64_t s) const { return s; }
+};
+
+template <class X> struct ArgState {
+    X val;
+    int64_t pos;
+};
+// State starts at (NotFound, minValue|maxValue) and is replaced only by a strictly better value, so a position is set
+// only together with a value better than the initial one; equal values therefore are either both unset or both set, and
+// taking the smaller position on a tie reproduces "first index wins" under any combine order.
+template <class X, bool MAX> struct RArg {
+    using In = X; using State = ArgState<X>; using Out = int64_t;
+    __device__ static bool better(X a, X b) { return MAX ? a > b : a < b; }
+    __device__ State init() const { return State{MAX ? std::numeric_limits<X>::lowest() : std::numeric_limits<X>::max(), DNH_NOT_FOUND}; }
+    __device__ State step(State s, X v, int64_t i) const { return better(v, s.val) ? State{v, i} : s; }
+    __device__ State combine(State a, State b) const {
+        const bool takeb = better(b.val, a.val) || (b.val == a.val && b.pos < a.pos);
+        return takeb ? b : a;
+    }
+    __device__ int64_t extract(State s) const { return s.pos; }
+};
+template <class X> struct RFind {
+    using In = X; using State = int64_t; using Out = int64_t;
+    X value;
+    __device__ int64_t init() const { return DNH_NOT_FOUND; }
+    __device__ int64_t step(int64_t s, X v, int64_t i) const { return (s == DNH_NOT_FOUND && v == value) ? i : s; }
+    __device__ int64_t combine(int64_t a, int64_t b) const {
+        if (a == DNH_NOT_FOUND) return b;
+        if (b == DNH_NOT_FOUND) return a;
+        return a < b ? a : b;
+    }
+    __device__ int64_t extract(int64_t s) const { return s; }
+};
+
+template <template <class> class RT>
+int32_t run_numeric(const DnhTensor* t, const DnhTensor* s, hipStream_t st, const char* what) {
+    switch (s->dtype) {
+        case DNH_U8: return launch_reduce(RT<uint8_t>{}, t, s, st, what);
+        case DNH_I8: return launch_reduce(RT<int8_t>{}, t, s, st, what);
+        case DNH_I32: return launch_reduce(RT<int32_t>{}, t, s, st, what);
+        case DNH_U32: return launch_reduce(RT<uint32_t>{}, t, s, st, what);
+        case DNH_I64: return launch_reduce(RT<int64_t>{}, t, s, st, what);
+        case DNH_U64: return launch_reduce(RT<uint64_t>{}, t, s, st, what);
+        case DNH_F32: return launch_reduce(RT<float>{}, t, s, st, what);
+        case DNH_F64: return launch_reduce(RT<double>{}, t, s, st, what);
+    }
+    return fail(DNH_ERR_NOT_SUPPORTED, "%s is not defined for %s", what, dtype_name(s->dtype));
+}
+
+template <bool MAX>
+int32_t run_arg(const DnhTensor* t, const DnhTensor* s, hipStream_t st, const char* what) {
+    switch (s->dtype) {
+        case DNH_U8: return launch_reduce(RArg<uint8_t, MAX>{}, t, s, st, what);
+        case DNH_I8: return launch_reduce(RArg<int8_t, MAX>{}, t, s, st, what);
+        case DNH_I32: return launch_reduce(RArg<int32_t, MAX>{}, t, s, st, what);
+        case DNH_U32: return launch_reduce(RArg<uint32_t, MAX>{}, t, s, st, what);
+        case DNH_I64: return launch_reduce(RArg<int64_t, MAX>{}, t, s, st, what);
+        case DNH_U64: return launch_reduce(RArg<uint64_t, MAX>{}, t, s, st, what);
+        case DNH_F32: return launch_reduce(RArg<float, MAX>{}, t, s, st, what);
+        case DNH_F64: return launch_reduce(RArg<double, MAX>{}, t, s, st, what);
+    }
+    return fail(DNH_ERR_NOT_SUPPORTED, "%s is not defined for %s", what, dtype_name(s->dtype));
+}
+
+}  // namespace
+
+extern "C" int32_t dnh_reduce_last_axis(int32_t op, const DnhTensor* t, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    DNH_TRY(check_tensor(t, "dnh_reduce_last_axis"));
+    DNH_TRY(check_tensor(src, "dnh_reduce_last_axis"));
+    hipStream_t st = (hipStream_t)stream;
+    if (op == DNH_ALL || op == DNH_ANY) {
+        if (src->dtype != DNH_BOOL || t->dtype != DNH_BOOL) return fail(DNH_ERR_INVALID_ARG, "All/Any need bool source and target");
+        return op == DNH_ALL ? launch_reduce(RAll{}, t, src, st, "AllLastAxis") : launch_reduce(RAny{}, t, src, st, "AnyLastAxis");
+    }
+    if (op == DNH_COUNT_TRUE) {
+        if (src->dtype != DNH_BOOL || t->dtype != DNH_I64) return fail(DNH_ERR_INVALID_ARG, "CountTrue needs a bool source and an int64 target");
+        return launch_reduce(RCountTrue{}, t, src, st, "CountTrueLastAxis");
+    }
+    if (t->dtype != src->dtype) return fail(DNH_ERR_INVALID_ARG, "dnh_reduce_last_axis: target is %s but source is %s", dtype_name(t->dtype), dtype_name(src->dtype));
+    switch (op) {
+        case DNH_SUM: return run_numeric<RSum>(t, src, st, "SumLastAxis");
+        case DNH_PRODUCT: return run_numeric<RProd>(t, src, st, "ProductLastAxis");
+        case DNH_MIN: return run_numeric<RMin>(t, src, st, "MinLastAxis");
+        case DNH_MAX: return run_numeric<RMax>(t, src, st, "MaxLastAxis");
+    }
+    return fail(DNH_ERR_INVALID_ARG, "dnh_reduce_last_axis: unknown op %d", op);
+}
+
+extern "C" int32_t dnh_arg_reduce_last_axis(int32_t op, const DnhTensor* t, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    DNH_TRY(check_tensor(t, "dnh_arg_reduce_last_axis"));
+    DNH_TRY(check_tensor(src, "dnh_arg_reduce_last_axis"));
+    if (t->dtype != DNH_I64) return fail(DNH_ERR_INVALID_ARG, "dnh_arg_reduce_last_axis: target must be int64");
+    hipStream_t st = (hipStream_t)stream;
+    if (op == DNH_ARG_MAX) return run_arg<true>(t, src, st, "ArgMaxLastAxis");
+    if (op == DNH_ARG_MIN) return run_arg<false>(t, src, st, "ArgMinLastAxis");
+    return fail(DNH_ERR_INVALID_ARG, "dnh_arg_reduce_last_axis: unknown op %d", op);
+}
+
+extern "C" int32_t dnh_find_last_axis(const void* value, const DnhTensor* t, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    DNH_TRY(check_tensor(t, "dnh_find_last_axis"));
+    DNH_TRY(check_tensor(src, "dnh_find_last_axis"));
+    if (!value) return fail(DNH_ERR_INVALID_ARG, "dnh_find_last_axis: null value");
+    if (t->dtype != DNH_I64) return fail(DNH_ERR_INVALID_ARG, "dnh_find_last_axis: target must be int64");
+    hipStream_t st = (hipStream_t)stream;
+#define CASE(DT, X) case DT: { X v; memcpy(&v, value, sizeof(X)); return launch_reduce(RFind<X>{v}, t, src, st, "FindLastAxis"); }
+    switch (src->dtype) {
+        CASE(DNH_BOOL, uint8_t) CASE(DNH_U8, uint8_t) CASE(DNH_I8, int8_t) CASE(DNH_I32, int32_t) CASE(DNH_U32, uint32_t)
+        CASE(DNH_I64, int64_t) CASE(DNH_U64, uint64_t) CASE(DNH_F32, float) CASE(DNH_F64, double)
+    }
+#undef CASE
+    return fail(DNH_ERR_NOT_SUPPORTED, "FindLastAxis on unknown dtype");
+}

@@ -1,0 +1,362 @@
+// Last-axis reduction kernels for gfx950.  A reducer R supplies
+//   In / State / Out, init(), step(State, In, int64 index), combine(State, State), extract(State).
+// Every combine below is commutative and associative (index-carrying states break value ties on the smaller index), so
+// any tree order yields the reference's sequential result for order-independent folds and the first-index rule of
+// ArgMin/ArgMax/Find (Tensor/Tensor/Host/ScalarOps.fs:638-665).
+//
+//   reduce_rows    : reduced axis has stride 1.  TPR threads (16, 64 = one wavefront, or 256 = the block) share a row,
+//                    16-byte loads, several in flight, wavefront shuffle tree + one LDS step for the block variant.
+//                    A long axis with few rows is split over gridDim.y into State partials (pass one of the two-pass tree).
+//   reduce_cols    : a kept dimension has stride 1 instead (the frontend's "reduce along the first axis" view,
+//                    Tensor.fs:4544-4567): lanes run along the kept dimension (coalesced), four wavefronts and
+//                    gridDim.y splits share the reduced axis, LDS combine, partials when split.
+//   reduce_rows<FROM_STATE> doubles as the finishing pass over partials.
+//   reduce_generic : one thread per output, for axes too short or layouts too irregular for the above.
+#pragma once
+
+#include "map_kernels.h"
+
+namespace dnh {
+
+struct OuterArgs {
+    int nd;
+    uint32_t shape[DNH_MAX_DIMS];
+    int64_t tstride[DNH_MAX_DIMS];
+    int64_t sstride[DNH_MAX_DIMS];
+};
+
+__device__ __forceinline__ void outer_offsets(const OuterArgs& o, uint32_t idx, int64_t& toff, int64_t& soff) {
+    toff = 0;
+    soff = 0;
+    for (int d = o.nd - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : idx / o.shape[d];
+        const uint32_t i = idx - q * o.shape[d];
+        idx = q;
+        toff += (int64_t)i * o.tstride[d];
+        soff += (int64_t)i * o.sstride[d];
+    }
+}
+
+template <class S>
+__device__ __forceinline__ S shfl_xor_any(const S& s, int mask) {
+    constexpr int W = (sizeof(S) + 3) / 4;
+    uint32_t w[W] = {};
+    __builtin_memcpy(w, &s, sizeof(S));
+#pragma unroll
+    for (int i = 0; i < W; i++) w[i] = (uint32_t)__shfl_xor((int)w[i], mask, 64);
+    S r;
+    __builtin_memcpy(&r, w, sizeof(S));
+    return r;
+}
+
+template <class R, int GROUP>
+__device__ __forceinline__ typename R::State group_reduce(const R& r, typename R::State s) {
+#pragma unroll
+    for (int m = (GROUP < 64 ? GROUP : 64) / 2; m >= 1; m >>= 1) s = r.combine(s, shfl_xor_any(s, m));
+    return s;
+}
+
+template <class R, int VEC, int TPR, bool FROM_STATE>
+__global__ __launch_bounds__(kBlock) void reduce_rows_kernel(R r, const void* src_, typename R::Out* out, typename R::State* partial,
+                                                             OuterArgs o, uint32_t rows, int64_t n, int64_t sr, int64_t chunk, uint32_t splits) {
+    using State = typename R::State;
+    using In = typename std::conditional<FROM_STATE, State, typename R::In>::type;
+    constexpr int RPB = kBlock / TPR;
+    constexpr int U = 4;
+    const In* src = (const In*)src_;
+    const uint32_t row = blockIdx.x * RPB + threadIdx.x / TPR;
+    const uint32_t lane = threadIdx.x % TPR;
+    const bool active = row < rows;
+    int64_t toff = 0, soff = 0;
+    if (active) {
+        outer_offsets(o, row, toff, soff);
+        if constexpr (FROM_STATE) soff = (int64_t)row * n;
+    }
+    const int64_t c0 = (int64_t)blockIdx.y * chunk;
+    const int64_t c1 = (c0 + chunk < n) ? c0 + chunk : n;
+    State st[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) st[e] = r.init();
+    if (active) {
+        const In* p = src + soff;
+        if constexpr (FROM_STATE) {
+            for (int64_t i = c0 + lane; i < c1; i += TPR) st[0] = r.combine(st[0], p[i]);
+        } else {
+            int64_t i = c0 + (int64_t)lane * VEC;
+            constexpr int64_t STEP = (int64_t)TPR * VEC;
+            for (; i + (U - 1) * STEP + VEC <= c1; i += U * STEP) {
+                Pack<In, VEC> v[U];
+#pragma unroll
+                for (int u = 0; u < U; u++) v[u] = load_pack<In, VEC>(p + (VEC == 1 ? (i + u * STEP) * sr : i + u * STEP));
+#pragma unroll
+                for (int u = 0; u < U; u++)
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) st[e] = r.step(st[e], v[u].v[e], i + u * STEP + e);
+            }
+            for (; i + VEC <= c1; i += STEP) {
+                Pack<In, VEC> v = load_pack<In, VEC>(p + (VEC == 1 ? i * sr : i));
+#pragma unroll
+                for (int e = 0; e < VEC; e++) st[e] = r.step(st[e], v.v[e], i + e);
+            }
+            if constexpr (VEC > 1) {
+                // the (c1 - c0) % VEC trailing elements of this chunk
+                const int64_t tail0 = c0 + ((c1 - c0) / VEC) * VEC;
+                const int64_t j = tail0 + lane;
+                if (j < c1) st[0] = r.step(st[0], p[j], j);
+            }
+        }
+    }
+    State s = st[0];
+#pragma unroll
+    for (int e = 1; e < VEC; e++) s = r.combine(s, st[e]);
+    s = group_reduce<R, TPR>(r, s);
+    if constexpr (TPR > 64) {
+        __shared__ State sh[TPR / 64];
+        const int wave = threadIdx.x / 64;
+        if ((threadIdx.x & 63) == 0) sh[wave] = s;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int w = 1; w < TPR / 64; w++) s = r.combine(s, sh[w]);
+        }
+    }
+    if (active && lane == 0) {
+        if (splits == 1) out[toff] = r.extract(s);
+        else partial[(int64_t)row * splits + blockIdx.y] = s;
+    }
+}
+
+template <class R, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(R r, const typename R::In* src, typename R::Out* out,
+                                                             typename R::State* partial, OuterArgs o, uint32_t col_tiles, uint32_t nc,
+                                                             int64_t tc_stride, int64_t n, int64_t sr, int64_t chunk, uint32_t splits) {
+    using State = typename R::State;
+    using In = typename R::In;
+    constexpr int NY = kBlock / 64;
+    constexpr int U = 4;
+    const uint32_t x = threadIdx.x & 63, y = threadIdx.x >> 6;
+    const uint32_t tile = blockIdx.x % col_tiles, other = blockIdx.x / col_tiles;
+    const uint32_t col0 = (tile * 64 + x) * VEC;
+    int64_t toff, soff;
+    outer_offsets(o, other, toff, soff);
+    const int64_t r0 = (int64_t)blockIdx.y * chunk;
+    const int64_t r1 = (r0 + chunk < n) ? r0 + chunk : n;
+    State st[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) st[e] = r.init();
+    const bool active = col0 < nc;
+    if (active) {
+        const In* p = src + soff + col0;
+        int64_t i = r0 + y;
+        for (; i + (U - 1) * NY < r1; i += U * NY) {
+            Pack<In, VEC> v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) v[u] = load_pack<In, VEC>(p + (i + u * NY) * sr);
+#pragma unroll
+            for (int u = 0; u < U; u++)
+#pragma unroll
+                for (int e = 0; e < VEC; e++) st[e] = r.step(st[e], v[u].v[e], i + u * NY);
+        }
+        for (; i < r1; i += NY) {
+            Pack<In, VEC> v = load_pack<In, VEC>(p + i * sr);
+#pragma unroll
+            for (int e = 0; e < VEC; e++) st[e] = r.step(st[e], v.v[e], i);
+        }
+    }
+    __shared__ State sh[NY - 1][64 * VEC];
+    if (y > 0) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) sh[y - 1][x * VEC + e] = st[e];
+    }
+    __syncthreads();
+    if (y == 0 && active) {
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            State s = st[e];
+#pragma unroll
+            for (int w = 0; w < NY - 1; w++) s = r.combine(s, sh[w][x * VEC + e]);
+            const uint32_t col = col0 + e;
+            if (splits == 1) out[toff + (int64_t)col * tc_stride] = r.extract(s);
+            else partial[((int64_t)other * nc + col) * splits + blockIdx.y] = s;
+        }
+    }
+}
+
+template <class R>
+__global__ __launch_bounds__(kBlock) void reduce_generic_kernel(R r, const typename R::In* src, typename R::Out* out, OuterArgs o,
+                                                                uint32_t nout, int64_t n, int64_t sr) {
+    const uint32_t idx = blockIdx.x * kBlock + threadIdx.x;
+    if (idx >= nout) return;
+    int64_t toff, soff;
+    outer_offsets(o, idx, toff, soff);
+    typename R::State s = r.init();
+    const typename R::In* p = src + soff;
+    for (int64_t i = 0; i < n; i++) s = r.step(s, p[i * sr], i);
+    out[toff] = r.extract(s);
+}
+
+// ---- host-side strategy --------------------------------------------------------------------------------------------------
+
+template <class R>
+int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStream_t stream, const char* what) {
+    using In = typename R::In;
+    using Out = typename R::Out;
+    using State = typename R::State;
+    constexpr int VEC = 16 / (int)sizeof(In);
+    DNH_TRY(check_tensor(t, what));
+    DNH_TRY(check_tensor(s, what));
+    if (s->ndims != t->ndims + 1) return fail(DNH_ERR_INVALID_ARG, "%s: source rank %d must be target rank %d + 1", what, s->ndims, t->ndims);
+    for (int d = 0; d < t->ndims; d++)
+        if (t->shape[d] != s->shape[d]) return fail(DNH_ERR_INVALID_ARG, "%s: target shape does not match the source's leading dimensions", what);
+    const int64_t n = s->shape[s->ndims - 1];
+    const int64_t sr = s->stride[s->ndims - 1];
+    const int64_t nout64 = nelems(t);
+    if (nout64 == 0) return DNH_OK;
+    if (nout64 > (int64_t)kMaxItems) return fail(DNH_ERR_NOT_SUPPORTED, "%s: more than 2^32 outputs", what);
+    const uint32_t nout = (uint32_t)nout64;
+    const In* src = (const In*)elem_ptr(s);
+    Out* out = (Out*)elem_ptr(t);
+
+    // collapse the kept dimensions jointly over target and source strides
+    OuterArgs o;
+    memset(&o, 0, sizeof(o));
+    {
+        int nd = 0;
+        for (int d = 0; d < t->ndims; d++) {
+            if (t->shape[d] == 1) continue;
+            if (nd > 0 && o.tstride[nd - 1] == t->stride[d] * t->shape[d] && o.sstride[nd - 1] == s->stride[d] * t->shape[d]) {
+                o.shape[nd - 1] *= (uint32_t)t->shape[d];
+                o.tstride[nd - 1] = t->stride[d];
+                o.sstride[nd - 1] = s->stride[d];
+                continue;
+            }
+            o.shape[nd] = (uint32_t)t->shape[d];
+            o.tstride[nd] = t->stride[d];
+            o.sstride[nd] = s->stride[d];
+            nd++;
+        }
+        o.nd = nd;
+    }
+    const int cus = device_cus();
+    const int64_t target_blocks = (int64_t)cus * 8;
+
+    // a kept dimension with source stride 1 (only of interest when the reduced axis itself is strided)
+    int dc = -1;
+    if (sr != 1)
+        for (int d = 0; d < o.nd; d++)
+            if (o.sstride[d] == 1 && o.shape[d] >= 32) dc = d;
+
+    if (!(dc >= 0 && n >= 8) && n >= 16) {
+        // rows
+        bool vec = VEC > 1 && sr == 1 && aligned_to(src, 16);
+        for (int d = 0; d < o.nd && vec; d++) vec = (o.sstride[d] % VEC) == 0;
+        const int v = vec ? VEC : 1;
+        int tpr = (n >= (int64_t)256 * v * 4) ? 256 : (n >= (int64_t)64 * v ? 64 : 16);
+        const int rpb = kBlock / tpr;
+        const int64_t row_blocks = (nout + rpb - 1) / rpb;
+        uint32_t splits = 1;
+        int64_t chunk = n;
+        if (tpr == 256 && row_blocks < target_blocks) {
+            const int64_t min_chunk = (int64_t)256 * v * 8;
+            int64_t want = (target_blocks + row_blocks - 1) / row_blocks;
+            int64_t maxs = (n + min_chunk - 1) / min_chunk;
+            int64_t sp = want < maxs ? want : maxs;
+            if (sp > 1) {
+                chunk = (n + sp - 1) / sp;
+                chunk = ((chunk + 256 * v - 1) / (256 * v)) * (256 * v);  // keeps every chunk start vector-aligned
+                splits = (uint32_t)((n + chunk - 1) / chunk);
+                if (splits <= 1) { splits = 1; chunk = n; }
+            }
+        }
+        State* partial = nullptr;
+        if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial));
+        const dim3 grid((unsigned)row_blocks, splits);
+#define DNH_ROWS(V, TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, V, TPR, false>), grid, dim3(kBlock), 0, stream, r, (const void*)src, out, partial, o, nout, n, sr, chunk, splits)
+        if (vec) {
+            if (tpr == 256) DNH_ROWS(VEC, 256); else if (tpr == 64) DNH_ROWS(VEC, 64); else DNH_ROWS(VEC, 16);
+        } else {
+            if (tpr == 256) DNH_ROWS(1, 256); else if (tpr == 64) DNH_ROWS(1, 64); else DNH_ROWS(1, 16);
+        }
+#undef DNH_ROWS
+        DNH_LAUNCH_CHECK();
+        if (splits > 1) {
+            // finishing pass: rows of `splits` State partials
+            if (splits > 64) {
+                hipLaunchKernelGGL((reduce_rows_kernel<R, 1, 256, true>), dim3(nout), dim3(kBlock), 0, stream, r, (const void*)partial, out,
+                                   (State*)nullptr, o, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u);
+            } else {
+                hipLaunchKernelGGL((reduce_rows_kernel<R, 1, 16, true>), dim3(cdiv(nout, 16)), dim3(kBlock), 0, stream, r, (const void*)partial, out,
+                                   (State*)nullptr, o, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u);
+            }
+            DNH_LAUNCH_CHECK();
+        }
+        return DNH_OK;
+    }
+
+    // columns
+    if (dc >= 0 && n >= 8) {
+        const uint32_t nc = o.shape[dc];
+        const int64_t tc_stride = o.tstride[dc];
+        OuterArgs oo;  // the other kept dimensions
+        memset(&oo, 0, sizeof(oo));
+        uint32_t others = 1;
+        for (int d = 0; d < o.nd; d++) {
+            if (d == dc) continue;
+            oo.shape[oo.nd] = o.shape[d];
+            oo.tstride[oo.nd] = o.tstride[d];
+            oo.sstride[oo.nd] = o.sstride[d];
+            others *= o.shape[d];
+            oo.nd++;
+        }
+        bool vec = VEC > 1 && aligned_to(src, 16) && (nc % VEC) == 0 && (sr % VEC) == 0;
+        for (int d = 0; d < oo.nd && vec; d++) vec = (oo.sstride[d] % VEC) == 0;
+        const int v = vec ? VEC : 1;
+        const uint32_t col_tiles = cdiv(nc, 64 * v);
+        const int64_t base_blocks = (int64_t)col_tiles * others;
+        uint32_t splits = 1;
+        int64_t chunk = n;
+        if (base_blocks < target_blocks) {
+            const int64_t min_chunk = 64;
+            int64_t want = (target_blocks + base_blocks - 1) / base_blocks;
+            int64_t maxs = (n + min_chunk - 1) / min_chunk;
+            int64_t sp = want < maxs ? want : maxs;
+            if (sp > 1) {
+                chunk = (n + sp - 1) / sp;
+                splits = (uint32_t)((n + chunk - 1) / chunk);
+                if (splits <= 1) { splits = 1; chunk = n; }
+            }
+        }
+        if (base_blocks <= 0x7FFFFFFF && splits <= 65535) {
+            State* partial = nullptr;
+            if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial));
+            const dim3 grid((unsigned)base_blocks, splits);
+            if (vec)
+                hipLaunchKernelGGL((reduce_cols_kernel<R, VEC>), grid, dim3(kBlock), 0, stream, r, src, out, partial, oo, col_tiles, nc, tc_stride, n, sr, chunk, splits);
+            else
+                hipLaunchKernelGGL((reduce_cols_kernel<R, 1>), grid, dim3(kBlock), 0, stream, r, src, out, partial, oo, col_tiles, nc, tc_stride, n, sr, chunk, splits);
+            DNH_LAUNCH_CHECK();
+            if (splits > 1) {
+                // partials are laid out [others][nc][splits]; enumerate outputs in that order for the finishing pass
+                OuterArgs fo = oo;
+                fo.shape[fo.nd] = nc;
+                fo.tstride[fo.nd] = tc_stride;
+                fo.sstride[fo.nd] = 0;
+                fo.nd++;
+                if (splits > 64)
+                    hipLaunchKernelGGL((reduce_rows_kernel<R, 1, 256, true>), dim3(nout), dim3(kBlock), 0, stream, r, (const void*)partial, out,
+                                       (State*)nullptr, fo, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u);
+                else
+                    hipLaunchKernelGGL((reduce_rows_kernel<R, 1, 16, true>), dim3(cdiv(nout, 16)), dim3(kBlock), 0, stream, r, (const void*)partial, out,
+                                       (State*)nullptr, fo, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u);
+                DNH_LAUNCH_CHECK();
+            }
+            return DNH_OK;
+        }
+    }
+
+    hipLaunchKernelGGL((reduce_generic_kernel<R>), dim3(cdiv(nout, kBlock)), dim3(kBlock), 0, stream, r, src, out, o, nout, n, sr);
+    DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
+
+}  // namespace dnh

@@ -1,0 +1,253 @@
+// Device, memory, stream and error plumbing of libtensor_hip — the part of the C ABI the reference obtains from the
+// CUDA driver through ManagedCuda (Tensor/Tensor/Cuda/CudaUtils.fs:36-60 context, Cuda/CudaBackend.fs:54-93 storage,
+// :206-270 transfers, Cuda/CudaRegMem.fs pinned memory, Cuda/CudaCfg.fs:16-27 stream).
+#include "common.h"
+
+#include <map>
+#include <mutex>
+
+namespace dnh {
+
+namespace {
+std::mutex g_mu;
+bool g_init = false;
+int g_device = 0;
+int g_cus = 256;
+int32_t* g_error_flag = nullptr;
+
+struct Workspace {
+    void* ptr = nullptr;
+    size_t bytes = 0;
+};
+std::map<hipStream_t, Workspace> g_ws;
+}  // namespace
+
+std::string& last_error() {
+    thread_local std::string e;
+    return e;
+}
+
+static int32_t init_locked(int device) {
+    if (g_init && device == g_device) return DNH_OK;
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count == 0) return fail(DNH_ERR_HIP, "no HIP device available (%s)", hipGetErrorString(e));
+    if (device < 0 || device >= count) return fail(DNH_ERR_INVALID_ARG, "device %d out of range (0..%d)", device, count - 1);
+    DNH_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    DNH_HIP(hipGetDeviceProperties(&prop, device));
+    g_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    if (!g_error_flag) {
+        DNH_HIP(hipMalloc((void**)&g_error_flag, sizeof(int32_t)));
+        DNH_HIP(hipMemset(g_error_flag, 0, sizeof(int32_t)));
+    }
+    g_device = device;
+    g_init = true;
+    return DNH_OK;
+}
+
+int32_t ensure_init() {
+    std::lock_guard<std::mutex> lock(g_mu);
+    if (g_init) {
+        // HIP's current device is per host thread; make the calling thread use ours.
+        DNH_HIP(hipSetDevice(g_device));
+        return DNH_OK;
+    }
+    return init_locked(0);
+}
+
+int device_cus() { return g_cus; }
+int32_t* error_flag_ptr() { return g_error_flag; }
+
+int32_t workspace(hipStream_t stream, size_t bytes, void** out) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    Workspace& w = g_ws[stream];
+    if (w.bytes < bytes) {
+        if (w.ptr) {
+            // work that still reads the old buffer is ordered before the free by synchronising the stream
+            DNH_HIP(hipStreamSynchronize(stream));
+            DNH_HIP(hipFree(w.ptr));
+            w.ptr = nullptr;
+            w.bytes = 0;
+        }
+        size_t want = bytes < (size_t)(4 << 20) ? (size_t)(4 << 20) : bytes + bytes / 2;
+        DNH_HIP(hipMalloc(&w.ptr, want));
+        w.bytes = want;
+    }
+    *out = w.ptr;
+    return DNH_OK;
+}
+
+static void drop_workspace(hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    auto it = g_ws.find(stream);
+    if (it != g_ws.end()) {
+        if (it->second.ptr) (void)hipFree(it->second.ptr);
+        g_ws.erase(it);
+    }
+}
+
+}  // namespace dnh
+
+using namespace dnh;
+
+extern "C" {
+
+int32_t dnh_init(int32_t device) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    return init_locked(device);
+}
+
+int32_t dnh_device_info(DnhDeviceInfo* info) {
+    if (!info) return fail(DNH_ERR_INVALID_ARG, "dnh_device_info: null argument");
+    DNH_TRY(ensure_init());
+    hipDeviceProp_t prop;
+    DNH_HIP(hipGetDeviceProperties(&prop, g_device));
+    memset(info, 0, sizeof(*info));
+    info->device = g_device;
+    info->compute_units = prop.multiProcessorCount;
+    info->wavefront_size = prop.warpSize;
+    info->max_threads_per_block = prop.maxThreadsPerBlock;
+    info->lds_bytes_per_block = (int64_t)prop.sharedMemPerBlock;
+    info->total_memory_bytes = (int64_t)prop.totalGlobalMem;
+    info->l2_bytes = (int64_t)prop.l2CacheSize;
+    info->clock_khz = prop.clockRate;
+    info->memory_clock_khz = prop.memoryClockRate;
+    strncpy(info->name, prop.name, sizeof(info->name) - 1);
+    strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
+    return DNH_OK;
+}
+
+int32_t dnh_last_error(char* buf, size_t n) {
+    if (!buf || n == 0) return DNH_ERR_INVALID_ARG;
+    const std::string& e = last_error();
+    size_t m = e.size() < n - 1 ? e.size() : n - 1;
+    memcpy(buf, e.data(), m);
+    buf[m] = 0;
+    return DNH_OK;
+}
+
+int32_t dnh_async_error(void* stream, int32_t* code) {
+    if (!code) return fail(DNH_ERR_INVALID_ARG, "dnh_async_error: null argument");
+    DNH_TRY(ensure_init());
+    int32_t flag = 0;
+    DNH_HIP(hipStreamSynchronize((hipStream_t)stream));
+    DNH_HIP(hipMemcpy(&flag, g_error_flag, sizeof(flag), hipMemcpyDeviceToHost));
+    if (flag) DNH_HIP(hipMemset(g_error_flag, 0, sizeof(flag)));
+    *code = flag ? DNH_ERR_INDEX_OUT_OF_RANGE : DNH_OK;
+    if (flag) last_error() = "an index tensor held a position outside the indexed tensor's shape";
+    return DNH_OK;
+}
+
+int32_t dnh_alloc(size_t bytes, void** out) {
+    if (!out) return fail(DNH_ERR_INVALID_ARG, "dnh_alloc: null argument");
+    DNH_TRY(ensure_init());
+    *out = nullptr;
+    DNH_HIP(hipMalloc(out, bytes ? bytes : 1));
+    return DNH_OK;
+}
+
+int32_t dnh_free(void* ptr) {
+    if (!ptr) return DNH_OK;
+    DNH_TRY(ensure_init());
+    DNH_HIP(hipFree(ptr));  // hipFree waits for outstanding work that may still use the buffer
+    return DNH_OK;
+}
+
+int32_t dnh_host_alloc(size_t bytes, void** out) {
+    if (!out) return fail(DNH_ERR_INVALID_ARG, "dnh_host_alloc: null argument");
+    DNH_TRY(ensure_init());
+    *out = nullptr;
+    DNH_HIP(hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault));
+    return DNH_OK;
+}
+
+int32_t dnh_host_free(void* ptr) {
+    if (!ptr) return DNH_OK;
+    DNH_HIP(hipHostFree(ptr));
+    return DNH_OK;
+}
+
+int32_t dnh_memset(void* dst, int32_t byte_value, size_t bytes, void* stream) {
+    DNH_TRY(ensure_init());
+    if (bytes == 0) return DNH_OK;
+    DNH_HIP(hipMemsetAsync(dst, byte_value, bytes, (hipStream_t)stream));
+    return DNH_OK;
+}
+
+static int32_t copy_impl(void* dst, const void* src, size_t bytes, void* stream, int32_t sync, hipMemcpyKind kind) {
+    DNH_TRY(ensure_init());
+    if (bytes == 0) return DNH_OK;
+    if (!dst || !src) return fail(DNH_ERR_INVALID_ARG, "memcpy: null pointer");
+    DNH_HIP(hipMemcpyAsync(dst, src, bytes, kind, (hipStream_t)stream));
+    if (sync) DNH_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return DNH_OK;
+}
+
+int32_t dnh_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream, int32_t sync) {
+    return copy_impl(dst, src, bytes, stream, sync, hipMemcpyHostToDevice);
+}
+int32_t dnh_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream, int32_t sync) {
+    return copy_impl(dst, src, bytes, stream, sync, hipMemcpyDeviceToHost);
+}
+int32_t dnh_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream, int32_t sync) {
+    return copy_impl(dst, src, bytes, stream, sync, hipMemcpyDeviceToDevice);
+}
+
+int32_t dnh_stream_create(void** stream) {
+    if (!stream) return fail(DNH_ERR_INVALID_ARG, "dnh_stream_create: null argument");
+    DNH_TRY(ensure_init());
+    hipStream_t s;
+    DNH_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *stream = (void*)s;
+    return DNH_OK;
+}
+
+int32_t dnh_stream_destroy(void* stream) {
+    if (!stream) return DNH_OK;
+    DNH_HIP(hipStreamSynchronize((hipStream_t)stream));
+    drop_workspace((hipStream_t)stream);
+    DNH_HIP(hipStreamDestroy((hipStream_t)stream));
+    return DNH_OK;
+}
+
+int32_t dnh_stream_sync(void* stream) {
+    DNH_TRY(ensure_init());
+    DNH_HIP(hipStreamSynchronize((hipStream_t)stream));
+    return DNH_OK;
+}
+
+int32_t dnh_device_sync(void) {
+    DNH_TRY(ensure_init());
+    DNH_HIP(hipDeviceSynchronize());
+    return DNH_OK;
+}
+
+int32_t dnh_event_create(void** event) {
+    if (!event) return fail(DNH_ERR_INVALID_ARG, "dnh_event_create: null argument");
+    DNH_TRY(ensure_init());
+    hipEvent_t e;
+    DNH_HIP(hipEventCreate(&e));
+    *event = (void*)e;
+    return DNH_OK;
+}
+int32_t dnh_event_destroy(void* event) {
+    if (!event) return DNH_OK;
+    DNH_HIP(hipEventDestroy((hipEvent_t)event));
+    return DNH_OK;
+}
+int32_t dnh_event_record(void* event, void* stream) {
+    DNH_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
+    return DNH_OK;
+}
+int32_t dnh_event_sync(void* event) {
+    DNH_HIP(hipEventSynchronize((hipEvent_t)event));
+    return DNH_OK;
+}
+int32_t dnh_event_elapsed_ms(void* start, void* stop, float* ms) {
+    if (!ms) return fail(DNH_ERR_INVALID_ARG, "dnh_event_elapsed_ms: null argument");
+    DNH_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return DNH_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,217 @@
+/*
+ * tensor_hip.h — C ABI of libtensor_hip.so, the MI355X (gfx950) tensor backend that a Deep.Net
+ * `TensorHipBackend<'T>` binds through P/Invoke (cdecl, blittable arguments only).
+ *
+ * Every entry point replaces one member (or a family of members) of the reference plugin interface
+ * `ITensorBackend<'T>` (Tensor/Tensor/TensorBackend.fs:64-146) or one facility the reference's CUDA
+ * storage/device objects obtain from the CUDA driver (Tensor/Tensor/Cuda/CudaBackend.fs,
+ * Tensor/Tensor/Cuda/CudaUtils.fs).  The citation beside each declaration names what it replaces.
+ *
+ * Conventions
+ *  - every function returns a DnhStatus (0 = OK); a human-readable message for the calling thread's
+ *    last failure is available from dnh_last_error();
+ *  - tensors are passed as pointers to DnhTensor descriptors, which the library copies before it returns;
+ *    `base` is a DEVICE pointer to element 0 of the storage, `offset` and `stride` are in ELEMENTS and
+ *    may be zero (broadcast) or negative, exactly as in TensorLayout (Tensor/Tensor/TensorLayout.fs:12-24);
+ *  - operands arrive already broadcast to the target's shape by the frontend
+ *    (Tensor/Tensor/Tensor.fs:4520-4540); the library checks shapes and dtypes and reports
+ *    DNH_ERR_INVALID_ARG on a mismatch;
+ *  - `stream` is a hipStream_t passed as void* (NULL = the default stream); all ops are asynchronous with
+ *    respect to the host unless stated otherwise;
+ *  - all entry points may be called from any thread.
+ */
+#ifndef TENSOR_HIP_H
+#define TENSOR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define DNH_MAX_DIMS 8
+
+typedef enum DnhStatus {
+    DNH_OK = 0,
+    DNH_ERR_INVALID_ARG = 1,      /* -> ArgumentException / InvalidOperationException          */
+    DNH_ERR_NOT_SUPPORTED = 2,    /* -> NotSupportedException (CudaBackend.fs:486-492)          */
+    DNH_ERR_OUT_OF_MEMORY = 3,    /* -> OutOfCudaMemoryException analogue (CudaUtils.fs:183-210) */
+    DNH_ERR_HIP = 4,              /* -> CudaException analogue                                  */
+    DNH_ERR_INDEX_OUT_OF_RANGE = 5, /* -> IndexOutOfRangeException (Host/FastAccess.fs:51-61)   */
+    DNH_ERR_NOT_INITIALIZED = 6
+} DnhStatus;
+
+/* Element types: the set the reference marshals to kernels (Cuda/NativeTensor.fs:22-34). bool is one byte 0/1. */
+typedef enum DnhDType {
+    DNH_BOOL = 0,
+    DNH_U8 = 1,
+    DNH_I8 = 2,
+    DNH_I32 = 3,
+    DNH_U32 = 4,
+    DNH_I64 = 5,
+    DNH_U64 = 6,
+    DNH_F32 = 7,
+    DNH_F64 = 8,
+    DNH_DTYPE_COUNT = 9
+} DnhDType;
+
+/* Replaces the by-value kernel argument struct Tensor<T,N> (Cuda/Kernels/Tensor.cuh:7-16,
+ * Cuda/NativeTensor.fs:96-112): one rank-agnostic, blittable descriptor. */
+typedef struct DnhTensor {
+    void*   base;                  /* device pointer to element 0 of the storage                 */
+    int64_t offset;                /* TensorLayout.Offset (elements)                             */
+    int32_t ndims;                 /* 0..DNH_MAX_DIMS                                            */
+    int32_t dtype;                 /* DnhDType                                                   */
+    int64_t shape[DNH_MAX_DIMS];   /* TensorLayout.Shape                                         */
+    int64_t stride[DNH_MAX_DIMS];  /* TensorLayout.Stride (elements)                             */
+} DnhTensor;
+
+typedef struct DnhDeviceInfo {
+    int32_t device;
+    int32_t compute_units;
+    int32_t wavefront_size;
+    int32_t max_threads_per_block;
+    int64_t lds_bytes_per_block;
+    int64_t total_memory_bytes;
+    int64_t l2_bytes;
+    int32_t clock_khz;
+    int32_t memory_clock_khz;
+    char    name[128];
+    char    arch[64];
+} DnhDeviceInfo;
+
+/* Unary element ops: ITensorBackend UnaryPlus..Truncate (TensorBackend.fs:74-94), Negate (:113);
+ * scalar semantics Host/ScalarOps.fs:381-493, ScalarPrimitives.fs:54-150, Sgn.fs:11-15.
+ * Round is ties-to-even (F# `round`), unlike the reference CUDA kernel (Cuda/Kernels/Elemwise.cuh:128). */
+typedef enum DnhUnaryOp {
+    DNH_UNARY_PLUS = 0, DNH_UNARY_MINUS, DNH_ABS, DNH_SGN, DNH_LOG, DNH_LOG10, DNH_EXP, DNH_SIN, DNH_COS,
+    DNH_TAN, DNH_ASIN, DNH_ACOS, DNH_ATAN, DNH_SINH, DNH_COSH, DNH_TANH, DNH_SQRT, DNH_CEILING, DNH_FLOOR,
+    DNH_ROUND, DNH_TRUNCATE, DNH_NEGATE, DNH_UNARY_COUNT
+} DnhUnaryOp;
+
+/* Binary element ops: ITensorBackend Add..MinElemwise (TensorBackend.fs:97-104), And/Or/Xor (:114-116);
+ * Host/ScalarOps.fs:495-575.  Max/Min are `if a>b then a else b` / `if a<b then a else b`. */
+typedef enum DnhBinaryOp {
+    DNH_ADD = 0, DNH_SUBTRACT, DNH_MULTIPLY, DNH_DIVIDE, DNH_MODULO, DNH_POWER, DNH_MAX_ELEMWISE,
+    DNH_MIN_ELEMWISE, DNH_AND, DNH_OR, DNH_XOR, DNH_BINARY_COUNT
+} DnhBinaryOp;
+
+/* Comparisons into a bool target: ITensorBackend Equal..GreaterOrEqual (TensorBackend.fs:106-111);
+ * Host/ScalarOps.fs:535-563. */
+typedef enum DnhCompareOp {
+    DNH_EQUAL = 0, DNH_NOT_EQUAL, DNH_LESS, DNH_LESS_OR_EQUAL, DNH_GREATER, DNH_GREATER_OR_EQUAL,
+    DNH_COMPARE_COUNT
+} DnhCompareOp;
+
+/* Last-axis folds: ITensorBackend SumLastAxis..CountTrueLastAxis (TensorBackend.fs:125-131);
+ * Host/ScalarOps.fs:299-361 (ApplyAxisFold), :606-636. */
+typedef enum DnhReduceOp {
+    DNH_SUM = 0, DNH_PRODUCT, DNH_MIN, DNH_MAX, DNH_ALL, DNH_ANY, DNH_COUNT_TRUE, DNH_REDUCE_COUNT
+} DnhReduceOp;
+
+/* Index-valued last-axis folds: ArgMinLastAxis / ArgMaxLastAxis (TensorBackend.fs:133-134);
+ * Host/ScalarOps.fs:638-654. */
+typedef enum DnhArgReduceOp { DNH_ARG_MIN = 0, DNH_ARG_MAX = 1 } DnhArgReduceOp;
+
+/* "value was not found": SpecialIdx.NotFound = Int64.MinValue + 4 (Tensor/Tensor/TensorRng.fs:24). */
+#define DNH_NOT_FOUND ((int64_t)(-9223372036854775807LL - 1LL + 4LL))
+
+/* ---------------------------------------------------------------------------------------------------
+ * Device, errors                                     (replaces Cuda/CudaUtils.fs:36-60 context creation)
+ * ------------------------------------------------------------------------------------------------- */
+int32_t dnh_init(int32_t device);
+int32_t dnh_device_info(DnhDeviceInfo* info);
+/* Copies the calling thread's last error message (NUL terminated, truncated to n). */
+int32_t dnh_last_error(char* buf, size_t n);
+/* Reads and clears the device-side index error flag set by gather/scatter kernels on `stream`
+ * (synchronises the stream).  *code = DNH_OK or DNH_ERR_INDEX_OUT_OF_RANGE.
+ * Replaces the error word + `Cfg.Stacktrace` read-back of Cuda/CudaKernels.fs:323-342, 385-398. */
+int32_t dnh_async_error(void* stream, int32_t* code);
+
+/* ---------------------------------------------------------------------------------------------------
+ * Memory and streams        (replaces TensorCudaStorage / CudaDeviceVariable, Cuda/CudaBackend.fs:54-93,
+ *                            transfers :206-270, pinned host memory Cuda/CudaRegMem.fs, stream Cuda/CudaCfg.fs:16-27)
+ * ------------------------------------------------------------------------------------------------- */
+int32_t dnh_alloc(size_t bytes, void** out);          /* at least one byte is allocated (CudaBackend.fs:56-58) */
+int32_t dnh_free(void* ptr);                          /* waits for in-flight work; callable from any thread    */
+int32_t dnh_host_alloc(size_t bytes, void** out);     /* pinned host memory for transfers                      */
+int32_t dnh_host_free(void* ptr);
+int32_t dnh_memset(void* dst, int32_t byte_value, size_t bytes, void* stream);
+int32_t dnh_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream, int32_t sync);
+int32_t dnh_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream, int32_t sync);
+int32_t dnh_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream, int32_t sync);
+int32_t dnh_stream_create(void** stream);
+int32_t dnh_stream_destroy(void* stream);
+int32_t dnh_stream_sync(void* stream);
+int32_t dnh_device_sync(void);
+/* Events, for timing kernels on the stream they run on. */
+int32_t dnh_event_create(void** event);
+int32_t dnh_event_destroy(void* event);
+int32_t dnh_event_record(void* event, void* stream);
+int32_t dnh_event_sync(void* event);
+int32_t dnh_event_elapsed_ms(void* start, void* stop, float* ms);
+
+/* ---------------------------------------------------------------------------------------------------
+ * Element-wise ops
+ * ------------------------------------------------------------------------------------------------- */
+/* ITensorBackend.FillConst (TensorBackend.fs:71; Host/ScalarOps.fs:363-365). `value` points to one host element of t's dtype. */
+int32_t dnh_fill_const(const DnhTensor* t, const void* value, void* stream);
+/* ITensorBackend.FillIncrementing (TensorBackend.fs:72; Host/ScalarOps.fs:367-370): t[pos] = start + incr * T(pos[0]). */
+int32_t dnh_fill_incrementing(const DnhTensor* t, const void* start, const void* incr, void* stream);
+/* ITensorBackend.Copy (TensorBackend.fs:67; Host/HostBackend.fs:196-208). Same dtype, any layouts. */
+int32_t dnh_copy(const DnhTensor* t, const DnhTensor* src, void* stream);
+/* ITensorBackend.Convert (TensorBackend.fs:69; Host/ScalarOps.fs:376-379): C# explicit numeric conversion. */
+int32_t dnh_convert(const DnhTensor* t, const DnhTensor* src, void* stream);
+/* Unary ops, DnhUnaryOp. */
+int32_t dnh_unary(int32_t op, const DnhTensor* t, const DnhTensor* a, void* stream);
+/* ITensorBackend.IsFinite (TensorBackend.fs:95; ScalarPrimitives.fs:181-188): bool target; true for every integer. */
+int32_t dnh_is_finite(const DnhTensor* t_bool, const DnhTensor* a, void* stream);
+/* Binary ops, DnhBinaryOp (And/Or/Xor take bool operands). */
+int32_t dnh_binary(int32_t op, const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream);
+/* Comparisons, DnhCompareOp, into a bool target. */
+int32_t dnh_compare(int32_t op, const DnhTensor* t_bool, const DnhTensor* a, const DnhTensor* b, void* stream);
+/* ITensorBackend.IfThenElse (TensorBackend.fs:118; Host/ScalarOps.fs:577-581). */
+int32_t dnh_if_then_else(const DnhTensor* t, const DnhTensor* cond_bool, const DnhTensor* if_true,
+                         const DnhTensor* if_false, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------
+ * Reductions along the LAST axis of `src` (src.ndims == t.ndims + 1, t.shape == src.shape[0..n-2]);
+ * the frontend permutes the reduced axis to the last position as a view (Tensor.fs:4544-4567), so the
+ * strides of `src` are arbitrary and select the kernel strategy.
+ * ------------------------------------------------------------------------------------------------- */
+int32_t dnh_reduce_last_axis(int32_t op, const DnhTensor* t, const DnhTensor* src, void* stream);
+int32_t dnh_arg_reduce_last_axis(int32_t op, const DnhTensor* t_i64, const DnhTensor* src, void* stream);
+/* ITensorBackend.FindLastAxis (TensorBackend.fs:135; Host/ScalarOps.fs:656-665): first index equal to *value, else DNH_NOT_FOUND. */
+int32_t dnh_find_last_axis(const void* value, const DnhTensor* t_i64, const DnhTensor* src, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------
+ * Indexing
+ * ------------------------------------------------------------------------------------------------- */
+/* ITensorBackend.Gather (TensorBackend.fs:119; Host/ScalarOps.fs:583-591).  idx has src->ndims entries, each NULL
+ * (identity on that dimension) or an int64 tensor already broadcast to t's shape.  An out-of-range index sets the
+ * stream's error flag (dnh_async_error) and leaves the target element unwritten; it never faults the device. */
+int32_t dnh_gather(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, void* stream);
+/* ITensorBackend.Scatter (TensorBackend.fs:120; Host/ScalarOps.fs:593-604): t[idx[s]] += src[s]; the frontend
+ * zero-fills t first (Tensor.fs:2159).  idx has t->ndims entries broadcast to src's shape. */
+int32_t dnh_scatter(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, void* stream);
+/* ITensorBackend.CountTrue is dnh_reduce_last_axis(DNH_COUNT_TRUE).
+ * ITensorBackend.MaskedGet (TensorBackend.fs:121; Host/ScalarOps.fs:667-681): masks has src->ndims entries, each NULL
+ * or a rank-1 bool tensor of length src->shape[d]; selected elements are written to t in row-major order. */
+int32_t dnh_masked_get(const DnhTensor* t, const DnhTensor* src, const DnhTensor* const* masks, int32_t n_masks, void* stream);
+/* ITensorBackend.MaskedSet (TensorBackend.fs:122; Host/ScalarOps.fs:683-697). */
+int32_t dnh_masked_set(const DnhTensor* t, const DnhTensor* const* masks, int32_t n_masks, const DnhTensor* src, void* stream);
+/* ITensorBackend.TrueIndices (TensorBackend.fs:123; Host/ScalarOps.fs:699-707): t is [nTrue; src.ndims] int64. */
+int32_t dnh_true_indices(const DnhTensor* t_i64, const DnhTensor* src_bool, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------
+ * Dot: ITensorBackend VecVecDot / MatVecDot / MatMatDot / BatchedMatMatDot (TensorBackend.fs:137-140;
+ * Host/HostBackend.fs:463-546).  The ranks of (t, a, b) select the variant exactly as Tensor.FillDot does
+ * (Tensor.fs:2714-2730): (0,1,1) (1,2,1) (2,2,2) or (n,n,n) with n>2.  fp32 and fp64.
+ * ------------------------------------------------------------------------------------------------- */
+int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TENSOR_HIP_H */

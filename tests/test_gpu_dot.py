@@ -1,0 +1,105 @@
+"""GPU parity: dot (vec.vec, mat.vec, mat.mat, batched) through the C ABI.
+The reference's fp32/fp64 dot runs in MKL, whose summation order cannot be recovered, so the contract is the K-term
+bound: with u = unit roundoff, S_ij = sum_k |a_ik||b_kj|, |gpu - oracle| <= (2K + 64) * u * S_ij and likewise against the fp64 product."""
+import numpy as np
+import pytest
+
+from util import both
+
+pytestmark = pytest.mark.gpu
+
+
+def check_dot(ref, got, a, b):
+    u = np.finfo(a.dtype).eps / 2
+    K = a.shape[-1]
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    if b.ndim == 1:
+        exact = a64 @ b64
+        S = np.abs(a64) @ np.abs(b64)
+    else:
+        exact = np.matmul(a64, b64)
+        S = np.matmul(np.abs(a64), np.abs(b64))
+    bound = (2 * K + 64) * u * S + np.finfo(a.dtype).tiny
+    assert got.shape == exact.shape
+    assert np.all(np.abs(got.astype(np.float64) - ref.astype(np.float64)) <= bound)
+    assert np.all(np.abs(got.astype(np.float64) - exact) <= bound)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("m,k,n", [(5, 3, 3), (128, 16, 128), (128, 512, 128), (256, 64, 384), (130, 70, 50), (1, 1, 1), (33, 1000, 7)])
+def test_matmat(H, G, rng, dt, m, k, n):
+    a = rng.standard_normal((m, k)).astype(dt)
+    b = rng.standard_normal((k, n)).astype(dt)
+    ref, got = both(H, G, lambda a, b: a @ b, a, b)
+    check_dot(ref, got, a, b)
+
+
+def test_doc_vector(H, G):
+    # Guide-Operations.md:129-148
+    h = 3.0 * np.arange(5.0)[:, None] + np.arange(3.0)[None, :]
+    i = 0.1 + np.eye(3)
+    ref, got = both(H, G, lambda a, b: a @ b, h, i)
+    exp = np.array([[0.3, 1.3, 2.3], [4.2, 5.2, 6.2], [8.1, 9.1, 10.1], [12.0, 13.0, 14.0], [15.9, 16.9, 17.9]])
+    assert np.allclose(got, exp, rtol=1e-14)
+    assert np.allclose(ref, exp, rtol=1e-14)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_vecvec_matvec(H, G, rng, dt):
+    a = rng.standard_normal((77, 300)).astype(dt)
+    x = rng.standard_normal(300).astype(dt)
+    y = rng.standard_normal(300).astype(dt)
+    ref, got = both(H, G, lambda a, x: a @ x, a, x)
+    check_dot(ref, got, a, x)
+    ref, got = both(H, G, lambda x, y: x @ y, x, y)
+    check_dot(ref.reshape(1), got.reshape(1), x[None, :], y)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_batched_equals_loop_and_broadcast(H, G, rng, dt):
+    # Tensor.Test/BaseTests.fs:84-96: a batched product equals the loop of 2-d products
+    a = rng.standard_normal((3, 4, 128, 48)).astype(dt)
+    b = rng.standard_normal((3, 4, 48, 130)).astype(dt)
+    ref, got = both(H, G, lambda a, b: a @ b, a, b)
+    check_dot(ref, got, a, b)
+    ta, tb = G.ofNumpy(a), G.ofNumpy(b)
+    for i in range(3):
+        for j in range(4):
+            single = G.toNumpy(ta[i, j] @ tb[i, j])
+            assert np.array_equal(single, got[i, j])
+    # broadcast batch dimension (stride 0) and transposed operand views
+    b1 = rng.standard_normal((1, 4, 48, 130)).astype(dt)
+    ref, got = both(H, G, lambda a, b: a @ b, a, b1)
+    check_dot(ref, got, a, np.broadcast_to(b1, (3, 4, 48, 130)))
+    at = np.ascontiguousarray(np.swapaxes(a, -1, -2))
+    ref, got = both(H, G, lambda a, b: a.T @ b, at, b)
+    check_dot(ref, got, a, b)
+    # (AB)^T = B^T A^T through transposed views on both sides and a transposed target
+    def f(a, b):
+        t = type(a).new([3, 4, 130, 128], a.Dev, a.DataType)
+        t.FillDot(b.T, a.T)
+        return t
+    ref2, got2 = both(H, G, f, a, b)
+    check_dot(np.swapaxes(ref2, -1, -2), np.swapaxes(got2, -1, -2), a, b)
+
+
+def test_config5_block_small(H, G, rng):
+    """batched matmul -> tanh -> row softmax (max, subtract, exp, sum, divide), the fifth benchmark configuration."""
+    a = (rng.standard_normal((4, 128, 128)) / np.sqrt(128)).astype(np.float32)
+    b = (rng.standard_normal((4, 128, 128)) / np.sqrt(128)).astype(np.float32)
+
+    def block(a, b):
+        t = (a @ b).tanh()
+        mx = t.maxAxis(2)
+        e = (t - mx[:, :, None]).exp()
+        sm = e.sumAxis(2)
+        return e / sm[:, :, None]
+    ref, got = both(H, G, block, a, b)
+    assert np.allclose(got, ref, rtol=2e-4, atol=1e-7)
+    assert np.allclose(got.sum(axis=2), 1.0, atol=1e-5)
+
+
+def test_non_float_dot_not_supported(G):
+    a = G.ofNumpy(np.ones((4, 4), np.int32))
+    with pytest.raises(NotImplementedError):
+        a @ a

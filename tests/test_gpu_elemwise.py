@@ -1,0 +1,233 @@
+"""GPU parity: element-wise map / map2 / map3 through the C ABI against the CPU oracle on identical seeded inputs.
+Bar: bit-exact for integer/bool work and for the exactly rounded fp ops (+ - * / sqrt abs neg min max rounding);
+1e-6 relative for transcendentals (the oracle is double libm rounded to T; the kernels use correctly-implemented
+single-precision routines, no fast-math)."""
+import numpy as np
+import pytest
+
+from util import both, assert_exact, assert_rel
+
+pytestmark = pytest.mark.gpu
+
+NUM = [np.uint8, np.int8, np.int32, np.uint32, np.int64, np.uint64, np.float32, np.float64]
+
+
+def rand(rng, dt, shape, lo=-50, hi=50):
+    dt = np.dtype(dt)
+    if dt.kind == "f":
+        return (rng.random(shape) * (hi - lo) + lo).astype(dt)
+    if dt.kind == "u":
+        return rng.integers(0, min(hi * 2, np.iinfo(dt).max), size=shape).astype(dt)
+    if dt.kind == "b":
+        return rng.random(shape) < 0.5
+    return rng.integers(max(lo, np.iinfo(dt).min), min(hi, np.iinfo(dt).max), size=shape).astype(dt)
+
+
+@pytest.mark.parametrize("dt", NUM)
+@pytest.mark.parametrize("op", ["add", "sub", "mul", "div", "mod", "max", "min"])
+def test_binary_exact(H, G, rng, dt, op):
+    a = rand(rng, dt, (37, 129))
+    b = rand(rng, dt, (37, 129))
+    if op in ("div", "mod"):
+        b[b == 0] = 3
+    f = {"add": lambda x, y: x + y, "sub": lambda x, y: x - y, "mul": lambda x, y: x * y, "div": lambda x, y: x / y,
+         "mod": lambda x, y: x % y, "max": lambda x, y: type(x).maxElemwise(x, y), "min": lambda x, y: type(x).minElemwise(x, y)}[op]
+    ref, got = both(H, G, f, a, b)
+    assert_exact(ref, got)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("fn,lo,hi", [("log", 0.01, 50), ("log10", 0.01, 50), ("exp", -20, 20), ("sin", -20, 20), ("cos", -20, 20),
+                                      ("tan", -1.5, 1.5), ("asin", -1, 1), ("acos", -1, 1), ("atan", -50, 50), ("sinh", -10, 10),
+                                      ("cosh", -10, 10), ("tanh", -5, 5)])
+def test_transcendental_rel(H, G, rng, dt, fn, lo, hi):
+    a = rand(rng, dt, (1000, 65), lo, hi)
+    ref, got = both(H, G, lambda x: getattr(x, fn)(), a)
+    assert_rel(ref, got, 1e-6)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("fn", ["sqrt", "ceiling", "floor", "round", "truncate", "abs", "sgn", "__neg__", "__pos__"])
+def test_unary_exact_fp(H, G, rng, dt, fn):
+    a = rand(rng, dt, (513, 33), 0 if fn == "sqrt" else -50, 50)
+    a.flat[:8] = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 0.0, -0.0] if fn != "sqrt" else [0.5, 1.5, 2.5, 0.25, 4, 9, 0.0, 2.0]
+    ref, got = both(H, G, lambda x: getattr(x, fn)(), a)
+    assert_exact(ref, got)
+
+
+def test_special_values_fp(H, G):
+    for dt in (np.float32, np.float64):
+        a = np.array([np.inf, -np.inf, np.nan, 0.0, -0.0, 1.0, -1.0, 1e-40, 3e38], dtype=dt)
+        for fn in ["tanh", "exp", "atan", "sqrt", "abs", "sgn", "floor", "round"]:
+            with np.errstate(all="ignore"):
+                ref, got = both(H, G, lambda x: getattr(x, fn)(), a)
+            assert_rel(ref, got, 1e-6)
+        ref, got = both(H, G, lambda x: x.isFinite(), a)
+        assert_exact(ref, got)
+
+
+@pytest.mark.parametrize("dt", [np.int8, np.int32, np.int64])
+def test_unary_int(H, G, rng, dt):
+    a = rand(rng, dt, (100, 17))
+    for fn in ["__neg__", "abs", "__pos__"] + (["sgn"] if dt != np.int8 else []):
+        ref, got = both(H, G, lambda x: getattr(x, fn)(), a)
+        assert_exact(ref, got)
+
+
+def test_unsupported_raise(G, rng):
+    a = G.ofNumpy(rand(rng, np.uint32, (8,)))
+    with pytest.raises(NotImplementedError):
+        -a
+    with pytest.raises(NotImplementedError):
+        G.ofNumpy(rand(rng, np.int32, (8,))).tanh()
+    with pytest.raises(NotImplementedError):
+        G.ofNumpy(rand(rng, np.int32, (8,))) ** G.ofNumpy(rand(rng, np.int32, (8,)))
+
+
+def test_integer_wraparound(H, G):
+    a = np.array([2 ** 31 - 1, -2 ** 31, 123456789, -5], dtype=np.int32)
+    b = np.array([1, -1, 987654321, 3], dtype=np.int32)
+    for f in (lambda x, y: x + y, lambda x, y: x - y, lambda x, y: x * y):
+        ref, got = both(H, G, f, a, b)
+        assert_exact(ref, got)
+    # truncation toward zero
+    ref, got = both(H, G, lambda x, y: x / y, np.array([-7, 7, -7, 7], np.int32), np.array([2, -2, -2, 2], np.int32))
+    assert_exact(ref, got)
+    assert got.tolist() == [-3, -3, 3, 3]
+    ref, got = both(H, G, lambda x, y: x % y, np.array([-7, 7, -7, 7], np.int32), np.array([2, -2, -2, 2], np.int32))
+    assert got.tolist() == [-1, 1, -1, 1]
+
+
+@pytest.mark.parametrize("dt", [np.bool_] + NUM)
+def test_compare(H, G, rng, dt):
+    a = rand(rng, dt, (63, 70), -3, 3)
+    b = rand(rng, dt, (63, 70), -3, 3)
+    for f in (lambda x, y: x == y, lambda x, y: x != y, lambda x, y: x < y, lambda x, y: x <= y, lambda x, y: x > y, lambda x, y: x >= y):
+        ref, got = both(H, G, f, a, b)
+        assert_exact(ref, got)
+
+
+def test_logic(H, G, rng):
+    a = rand(rng, np.bool_, (1000,))
+    b = rand(rng, np.bool_, (1000,))
+    for f in (lambda x, y: x & y, lambda x, y: x | y, lambda x, y: x ^ y, lambda x, y: ~x):
+        ref, got = both(H, G, f, a, b)
+        assert_exact(ref, got)
+
+
+@pytest.mark.parametrize("dt", [np.bool_, np.int8, np.int32, np.float32, np.int64, np.float64])
+def test_if_then_else(H, G, rng, dt):
+    c = rand(rng, np.bool_, (33, 65))
+    a = rand(rng, dt, (33, 65))
+    b = rand(rng, dt, (33, 65))
+    ref, got = both(H, G, lambda c, a, b: type(a).ifThenElse(c, a, b), c, a, b)
+    assert_exact(ref, got)
+    assert_exact(np.where(c, a, b), got)
+
+
+def test_scalar_broadcast_and_power(H, G, rng):
+    a = rand(rng, np.float32, (4097,), 0.1, 5)
+    ref, got = both(H, G, lambda x: x * 2.5 + 1.0, a)
+    assert_exact(ref, got)
+    ref, got = both(H, G, lambda x: x ** 1.7, a)
+    assert_rel(ref, got, 1e-6)
+    ai = rand(rng, np.int32, (100000,), -1000, 1000)
+    ref, got = both(H, G, lambda x: x > 0, ai)
+    assert_exact(ref, got)
+    assert_exact(ai > 0, got)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64, np.int32, np.uint8])
+def test_strided_and_broadcast_views(H, G, rng, dt):
+    x = rand(rng, dt, (6, 20, 70))
+    v = rand(rng, dt, (70,))
+    w = rand(rng, dt, (20, 1))
+
+    # permuted view + broadcast vector, as the frontend builds them
+    def f(x, v, w):
+        xp = x.permuteAxes([2, 0, 1])          # shape [20, 70, 6]
+        return xp + v[None, :, None] + w[:, :, None]
+    ref, got = both(H, G, f, x, v, w)
+    assert_exact(ref, got)
+    exp = np.transpose(x, (1, 2, 0)) + v[None, :, None] + w[:, :, None]
+    assert_exact(exp.astype(dt), got)
+
+    # slices with offsets, transposes, reversed axes, copies into non-contiguous targets
+    def g(x, v, w):
+        s = x[1:5, 3:17, 5:64]
+        return (s.T.reverseAxis(0) - s.T).Copy()
+    ref, got = both(H, G, g, x, v, w)
+    assert_exact(ref, got)
+
+    def h(x, v, w):
+        t = type(x).new([70, 20], x.Dev, x.DataType).T     # column-major target of shape [20, 70]
+        t.FillAdd(x[2], x[3])
+        return t
+    ref, got = both(H, G, h, x, v, w)
+    assert_exact(ref, got)
+
+
+def test_large_transpose_copy_and_add(H, G, rng):
+    x = rng.standard_normal((16, 96, 200)).astype(np.float32)
+    v = rng.random(200).astype(np.float32)
+
+    def f(x, v):
+        xp = x.permuteAxes([2, 0, 1])              # [96, 200, 16], strides [200, 1, 19200]
+        return xp + v[None, :, None], xp.Copy()
+    (r1, r2), (g1, g2) = both(H, G, f, x, v)
+    assert_exact(r1, g1)
+    assert_exact(r2, g2)
+    assert_exact(np.transpose(x, (1, 2, 0)).copy(), g2)
+    # fp64 uses the 32x32 tile variant
+    xd = x.astype(np.float64)
+    ref, got = both(H, G, lambda x: x.permuteAxes([2, 0, 1]).Copy(), xd)
+    assert_exact(ref, got)
+
+
+def test_in_place(H, G):
+    # the documentation's f3.FillMultiply f3 e example, Guide-Operations.md:103-115
+    def f(f3, d, e):
+        f3.FillMultiply(d, e)
+        f3.FillMultiply(f3, e)
+        return f3
+    ref, got = both(H, G, f, np.array([-1.0, -1.0, 29.0, 40.0]), np.arange(4.0), 10.0 * np.arange(4.0))
+    assert_exact(ref, got)
+    assert got.tolist() == [0.0, 100.0, 800.0, 2700.0]
+
+
+@pytest.mark.parametrize("src", [np.bool_] + NUM)
+@pytest.mark.parametrize("dst", [np.bool_] + NUM)
+def test_convert(H, G, rng, src, dst):
+    a = rand(rng, src, (257,), 0, 100)
+    ref, got = both(H, G, lambda x: x.convert(dst), a)
+    assert_exact(ref, got)
+    if np.dtype(dst) != np.bool_:
+        assert_exact(a.astype(dst), got)
+
+
+def test_fill_and_counting(H, G):
+    for dt in NUM:
+        ref, got = both(H, G, lambda x: type(x).filled([5, 7], 3, x.Dev, x.DataType), np.zeros(1, dt))
+        assert_exact(ref, got)
+        ref, got = both(H, G, lambda x: type(x).counting(1000, x.Dev, x.DataType), np.zeros(1, dt))
+        assert_exact(ref, got)
+    got = G.toNumpy(G.zeros([3, 0, 4], np.float32))
+    assert got.shape == (3, 0, 4)
+
+
+def test_empty_and_scalar(H, G):
+    ref, got = both(H, G, lambda a, b: a + b, np.zeros((0, 5), np.float32), np.zeros((0, 5), np.float32))
+    assert got.shape == (0, 5)
+    ref, got = both(H, G, lambda a, b: a * b, np.array(3.0, np.float64), np.array(4.0, np.float64))
+    assert got == 12.0 and ref == 12.0
+
+
+def test_config1_chain_small(H, G, rng):
+    """y = tanh(a*b + c); exp(-y*y) — the element-wise chain of the first benchmark configuration, six backend calls."""
+    a, b, c = (rng.uniform(-1, 1, (256, 512)).astype(np.float32) for _ in range(3))
+
+    def chain(a, b, c):
+        y = (a * b + c).tanh()
+        return (-(y * y)).exp()
+    ref, got = both(H, G, chain, a, b, c)
+    assert_rel(ref, got, 1e-6)

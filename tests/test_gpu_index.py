@@ -1,0 +1,174 @@
+"""GPU parity: gather / scatter / masked get / masked set / trueIdx through the C ABI — all bit-exact against the oracle
+and against NumPy's own indexing."""
+import numpy as np
+import pytest
+
+from util import both, assert_exact
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dt", [np.int32, np.float32, np.int64, np.float64, np.uint8, np.bool_])
+def test_gather_1d(H, G, rng, dt):
+    src = (rng.integers(0, 2, 100000) > 0) if dt == np.bool_ else rng.integers(-1000, 1000, 100000).astype(dt)
+    idx = rng.integers(0, src.size, 30011).astype(np.int64)
+    ref, got = both(H, G, lambda s, i: type(s).gather([i], s), src, idx)
+    assert_exact(ref, got)
+    assert_exact(src[idx], got)
+
+
+def test_gather_nd_with_none_and_broadcast(H, G, rng):
+    src = rng.standard_normal((30, 40, 50)).astype(np.float32)
+    i0 = rng.integers(0, 30, (40, 1)).astype(np.int64)
+    i2 = rng.integers(0, 50, (1, 7)).astype(np.int64)
+    # target shape [40, 7]; dimension 1 of src maps identically from target dimension 1?  No: identity needs d < target rank
+    ref, got = both(H, G, lambda s, a, b: type(s).gather([a, None, b], s), src, i0, rng.integers(0, 50, (40, 40)).astype(np.int64))
+    assert_exact(ref, got)
+    # documentation vectors (Guide-Index.md:87-105)
+    s = np.array([[0.0, 0.1, 0.2, 0.3], [1.0, 1.1, 1.2, 1.3], [2.0, 2.1, 2.2, 2.3]])
+    g = G.toNumpy(type(G.ofNumpy(s)).gather([G.ofNumpy(np.array([1, 2, 0, 0])), G.ofNumpy(np.array([3, 1, 0, 3]))], G.ofNumpy(s)))
+    assert g.tolist() == [1.3, 2.1, 0.0, 0.3]
+    g2 = G.toNumpy(type(G.ofNumpy(s)).gather([None, G.ofNumpy(np.array([3, 1, 0]))], G.ofNumpy(s)))
+    assert g2.tolist() == [0.3, 1.1, 2.0]
+    _ = i2
+
+
+def test_gather_out_of_range_raises(H, G):
+    s = np.arange(10, dtype=np.int32)
+    for bad in ([3, 10], [-1, 2]):
+        with pytest.raises(IndexError):
+            type(G.ofNumpy(s)).gather([G.ofNumpy(np.array(bad, dtype=np.int64))], G.ofNumpy(s))
+        with pytest.raises(IndexError):
+            type(H.ofNumpy(s)).gather([H.ofNumpy(np.array(bad, dtype=np.int64))], H.ofNumpy(s))
+    # the flag is cleared by the read: a following valid gather succeeds
+    ok = type(G.ofNumpy(s)).gather([G.ofNumpy(np.array([9, 0], dtype=np.int64))], G.ofNumpy(s))
+    assert G.toNumpy(ok).tolist() == [9, 0]
+
+
+@pytest.mark.parametrize("dt", [np.int32, np.int64, np.uint32, np.uint64, np.uint8, np.int8])
+def test_scatter_int_with_duplicates(H, G, rng, dt):
+    src = rng.integers(0, 100, 50000).astype(dt)
+    idx = rng.integers(0, 777, 50000).astype(np.int64)          # heavy duplication: sums, wrapping for narrow types
+    ref, got = both(H, G, lambda s, i: type(s).scatter([i], [1000], s), src, idx)
+    assert_exact(ref, got)
+    exp = np.zeros(1000, dtype=dt)
+    np.add.at(exp, idx, src)
+    assert_exact(exp, got)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_scatter_fp_unique(H, G, rng, dt):
+    src = rng.standard_normal(40000).astype(dt)
+    idx = rng.permutation(100000)[:40000].astype(np.int64)
+    ref, got = both(H, G, lambda s, i: type(s).scatter([i], [100000], s), src, idx)
+    assert_exact(ref, got)
+
+
+def test_scatter_doc_vector(H, G):
+    # Guide-Index.md:118-133: first row summed into [0,3]; rows 1 and 2 swapped; row 3 stays zero
+    src = np.array([[0.0, 0.1, 0.2, 0.3], [1.0, 1.1, 1.2, 1.3], [2.0, 2.1, 2.2, 2.3]])
+    i0 = np.array([[0, 0, 0, 0], [2, 2, 2, 2], [1, 1, 1, 1]], dtype=np.int64)
+    i1 = np.array([[3, 3, 3, 3], [0, 1, 2, 3], [0, 1, 2, 3]], dtype=np.int64)
+    ref, got = both(H, G, lambda s, a, b: type(s).scatter([a, b], [4, 4], s), src, i0, i1)
+    exp = np.array([[0, 0, 0, 0.6], [2.0, 2.1, 2.2, 2.3], [1.0, 1.1, 1.2, 1.3], [0, 0, 0, 0]])
+    assert np.allclose(got, exp, rtol=0, atol=1e-15)
+    assert np.allclose(ref, exp, rtol=0, atol=1e-15)
+    with pytest.raises(IndexError):
+        type(G.ofNumpy(src)).scatter([G.ofNumpy(i0), G.ofNumpy(i1 + 1)], [4, 4], G.ofNumpy(src))
+
+
+@pytest.mark.parametrize("n", [0, 1, 15, 16, 17, 4096, 4097, 100003])
+def test_masked_get_1d(H, G, rng, n):
+    a = rng.integers(-1000, 1000, n).astype(np.int32)
+    m = a > 0
+    ref, got = both(H, G, lambda a, m: a.M(m), a, m)
+    assert_exact(ref, got)
+    assert_exact(a[m], got)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64, np.uint8, np.bool_])
+def test_masked_get_set_nd(H, G, rng, dt):
+    a = (rng.random((37, 41)) < 0.5) if dt == np.bool_ else rng.integers(0, 100, (37, 41)).astype(dt)
+    m = rng.random((37, 41)) < 0.3
+    ref, got = both(H, G, lambda a, m: a.M(m), a, m)
+    assert_exact(ref, got)
+    assert_exact(a[m], got)
+    # per-dimension masks and NoMask (Guide-Logic.md:97-100)
+    m0 = rng.random(37) < 0.5
+    m1 = rng.random(41) < 0.5
+    for f, exp in ((lambda a, x, y: a.M(x, None), a[m0, :]), (lambda a, x, y: a.M(None, y), a[:, m1]),
+                   (lambda a, x, y: a.M(x, y), a[np.ix_(m0, m1)])):
+        ref, got = both(H, G, f, a, m0, m1)
+        assert_exact(ref, got)
+        assert_exact(exp, got)
+    # masked set, also on a transposed (non-reshapeable) target
+    k = int(m.sum())
+    v = (rng.random(k) < 0.5) if dt == np.bool_ else rng.integers(100, 200, k).astype(dt)
+
+    def setm(a, m, v):
+        a.setM([m], v)
+        return a
+    ref, got = both(H, G, setm, a, m, v)
+    assert_exact(ref, got)
+    exp = a.copy()
+    exp[m] = v
+    assert_exact(exp, got)
+
+    def setm_t(a, m, v):
+        at = a.T
+        at.setM([m.T.Copy()], v)
+        return a
+    ref, got = both(H, G, setm_t, a, m, v[: int(m.T.sum())])
+    assert_exact(ref, got)
+
+
+def test_mask_doc_vectors(H, G):
+    a = np.array([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]])
+    m = np.array([[True, True, False], [False, False, True]])
+    t = G.ofNumpy(a)
+    assert G.toNumpy(t.M(G.ofNumpy(m))).tolist() == [1.0, 2.0, 6.0]                       # Guide-Logic.md:85-91
+    assert G.toNumpy(t.M(G.ofNumpy(np.array([True, False])), None)).tolist() == [[1.0, 2.0, 3.0]]   # :97-100
+    t.setM([G.ofNumpy(m)], G.ofNumpy(np.array([8.0, 9.0, 0.0])))
+    assert G.toNumpy(t).tolist() == [[8.0, 9.0, 3.0], [4.0, 5.0, 0.0]]                    # :109-114
+
+
+@pytest.mark.parametrize("shape", [(2, 4), (50,), (7, 11, 13), (3, 0), (100, 100)])
+def test_true_idx(H, G, rng, shape):
+    m = rng.random(shape) < 0.4
+    ref, got = both(H, G, lambda m: m.trueIdx(), m)
+    assert_exact(ref, got)
+    assert_exact(np.argwhere(m).astype(np.int64).reshape(-1, len(shape)), got)
+    # on a permuted view
+    if len(shape) == 3:
+        ref, got = both(H, G, lambda m: m.permuteAxes([1, 2, 0]).trueIdx(), m)
+        assert_exact(ref, got)
+
+
+def test_true_idx_doc_vector(G):
+    a = np.array([[True, False, True, False], [False, True, True, False]])
+    assert G.toNumpy(G.ofNumpy(a).trueIdx()).tolist() == [[0, 0], [0, 2], [1, 1], [1, 2]]   # Guide-Logic.md:46-53
+
+
+def test_config4_sequence_small(H, G, rng):
+    """compare -> mask -> ifThenElse / countTrue / maskedGet / gather / scatter on int32, the fourth benchmark configuration."""
+    n, mcount = 1 << 16, 1 << 14
+    a = rng.integers(-1000, 1001, n).astype(np.int32)
+    b = rng.integers(-1000, 1001, n).astype(np.int32)
+    idx = rng.integers(0, n, mcount).astype(np.int64)
+    idxu = rng.permutation(n)[:mcount].astype(np.int64)
+
+    def seq(a, b, idx, idxu):
+        T = type(a)
+        m = a > 0
+        r = T.ifThenElse(m, a, b)
+        k = m.countTrue()
+        g = a.M(m)
+        h = T.gather([idx], a)
+        s = T.scatter([idxu], [n], h)
+        return m, r, k, g, h, s
+    ref, got = both(H, G, seq, a, b, idx, idxu)
+    for r, g in zip(ref, got):
+        if isinstance(r, int):
+            assert r == g == int((a > 0).sum())
+        else:
+            assert_exact(r, g)

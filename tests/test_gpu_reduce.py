@@ -1,0 +1,159 @@
+"""GPU parity: axis reductions through the C ABI against the CPU oracle.
+Order-independent folds (max/min/all/any/countTrue, integer sums/products) and ArgMin/ArgMax/Find are bit-exact.
+Float sums/products are re-associated on the GPU; contract (u = unit roundoff of T, S = sum of |x| over the reduced
+elements, n their count):  |gpu - ref| <= (n + c + d) * u * S  with c + d <= 64 (per-lane chunk + tree depth bound)."""
+import numpy as np
+import pytest
+
+from util import both, assert_exact
+
+pytestmark = pytest.mark.gpu
+
+NOT_FOUND = -(2 ** 63) + 4
+
+
+def sum_bound_ok(ref, got, x, axis):
+    u = np.finfo(x.dtype).eps / 2
+    S = np.sum(np.abs(x.astype(np.float64)), axis=axis)
+    n = x.shape[axis] if axis is not None else x.size
+    bound = (n + 64) * u * S + np.finfo(x.dtype).tiny
+    exact = np.sum(x.astype(np.float64), axis=axis)
+    err = np.abs(got.astype(np.float64) - ref.astype(np.float64))
+    assert np.all(err <= bound), f"worst {np.max(err / np.maximum(bound, 1e-300))} of bound"
+    # the tree is expected to be at least as close to the exact sum as the sequential fold's own bound
+    assert np.all(np.abs(got.astype(np.float64) - exact) <= bound)
+
+
+SHAPES = [(7, 5), (64, 1000), (3, 4099), (1000, 33), (5, 17, 300), (2, 40000), (1, 70000)]
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_sum_max_min_fp_all_axes(H, G, rng, dt, shape):
+    x = rng.standard_normal(shape).astype(dt)
+    for ax in range(len(shape)):
+        ref, got = both(H, G, lambda t: t.sumAxis(ax), x)
+        sum_bound_ok(ref, got, x, ax)
+        for name in ("maxAxis", "minAxis", "argMaxAxis", "argMinAxis"):
+            ref, got = both(H, G, lambda t: getattr(t, name)(ax), x)
+            assert_exact(ref, got)
+        assert_exact(np.argmax(x, axis=ax).astype(np.int64), G.toNumpy(G.ofNumpy(x).argMaxAxis(ax)))
+        assert_exact(np.max(x, axis=ax), G.toNumpy(G.ofNumpy(x).maxAxis(ax)))
+
+
+@pytest.mark.parametrize("dt", [np.int32, np.int64, np.uint8, np.int8, np.uint32, np.uint64])
+def test_int_folds_exact(H, G, rng, dt):
+    x = rng.integers(0, 100, size=(33, 1030)).astype(dt)
+    for ax in (0, 1):
+        for name in ("sumAxis", "productAxis", "maxAxis", "minAxis", "argMaxAxis", "argMinAxis"):
+            ref, got = both(H, G, lambda t: getattr(t, name)(ax), x)
+            assert_exact(ref, got)
+
+
+def test_product_fp(H, G, rng):
+    x = rng.uniform(0.9, 1.1, (50, 700)).astype(np.float32)
+    for ax in (0, 1):
+        ref, got = both(H, G, lambda t: t.productAxis(ax), x)
+        assert np.allclose(ref, got, rtol=x.shape[ax] * 2 ** -23, atol=0)
+
+
+def test_full_reductions(H, G, rng):
+    x = rng.standard_normal((300, 1111)).astype(np.float32)
+    ref, got = both(H, G, lambda t: t.sumTensor(), x)
+    sum_bound_ok(ref, got, x, None)
+    for f in (lambda t: t.maxTensor(), lambda t: t.minTensor()):
+        ref, got = both(H, G, f, x)
+        assert_exact(ref, got)
+    t = G.ofNumpy(x)
+    assert t.argMax() == list(np.unravel_index(np.argmax(x), x.shape))
+    assert t.argMin() == list(np.unravel_index(np.argmin(x), x.shape))
+    # a permuted view flattens through a copy (ITensor.fs:306-316)
+    ref, got = both(H, G, lambda t: t.T.maxTensor(), x)
+    assert_exact(ref, got)
+
+
+def test_argmax_ties_and_notfound(H, G):
+    x = np.array([[1, 5, 5, 2, 5], [7, 7, 7, 7, 7], [-np.inf] * 5, [np.nan] * 5, [np.nan, 3, np.nan, 3, 1]], dtype=np.float32)
+    ref, got = both(H, G, lambda t: t.argMaxAxis(1), x)
+    assert_exact(ref, got)
+    assert got.tolist() == [1, 0, NOT_FOUND, NOT_FOUND, 1]
+    ref, got = both(H, G, lambda t: t.argMinAxis(1), x)
+    assert_exact(ref, got)
+    # planted ties far apart in a long row: the lowest index must win whatever lane/block sees it
+    y = np.zeros((4, 100000), dtype=np.float32)
+    y[0, [99999, 512, 70000]] = 9
+    y[1, [65536, 65537]] = 3
+    y[2, 99999] = 1
+    for ax_view in (lambda t: t.argMaxAxis(1), lambda t: t.T.Copy().argMaxAxis(0)):
+        ref, got = both(H, G, ax_view, y)
+        assert_exact(ref, got)
+        assert got.tolist() == [512, 65536, 99999, 0]
+    # integer rows that never exceed the initial value
+    z = np.full((2, 10), np.iinfo(np.int32).min, dtype=np.int32)
+    z[1, 7] = 0
+    ref, got = both(H, G, lambda t: t.argMaxAxis(1), z)
+    assert got.tolist() == [NOT_FOUND, 7]
+    assert_exact(ref, got)
+
+
+def test_max_of_neg_inf_is_min_value(H, G):
+    # the fold starts at Single.MinValue, so a row of -inf yields -FLT_MAX (ScalarOps.fs:620-623)
+    x = np.full((3, 100), -np.inf, dtype=np.float32)
+    ref, got = both(H, G, lambda t: t.maxAxis(1), x)
+    assert_exact(ref, got)
+    assert got[0] == np.finfo(np.float32).min
+
+
+def test_empty_axis_yields_initial_value(H, G):
+    x = np.zeros((4, 0), dtype=np.float32)
+    for name, val in (("sumAxis", 0.0), ("productAxis", 1.0), ("maxAxis", np.finfo(np.float32).min), ("minAxis", np.finfo(np.float32).max)):
+        ref, got = both(H, G, lambda t: getattr(t, name)(1), x)
+        assert_exact(ref, got)
+        assert got.tolist() == [val] * 4
+    ref, got = both(H, G, lambda t: t.argMaxAxis(1), x)
+    assert got.tolist() == [NOT_FOUND] * 4
+    b = np.zeros((3, 0), dtype=np.bool_)
+    assert G.toNumpy(G.ofNumpy(b).allAxis(1)).tolist() == [True] * 3
+    assert G.toNumpy(G.ofNumpy(b).anyAxis(1)).tolist() == [False] * 3
+    assert G.toNumpy(G.ofNumpy(b).countTrueAxis(1)).tolist() == [0] * 3
+
+
+@pytest.mark.parametrize("shape", [(9, 1000), (100, 100), (2, 3, 4097), (1, 300000)])
+def test_bool_folds(H, G, rng, shape):
+    m = rng.random(shape) < 0.5
+    m2 = np.ones(shape, dtype=np.bool_)
+    m2.flat[m2.size // 2] = False
+    for x in (m, m2, np.zeros(shape, np.bool_)):
+        for ax in range(len(shape)):
+            for name in ("allAxis", "anyAxis", "countTrueAxis"):
+                ref, got = both(H, G, lambda t: getattr(t, name)(ax), x)
+                assert_exact(ref, got)
+        assert G.ofNumpy(x).countTrue() == int(np.count_nonzero(x))
+        assert G.ofNumpy(x).all() == bool(x.all()) and G.ofNumpy(x).any() == bool(x.any())
+
+
+def test_find(H, G, rng):
+    x = rng.integers(0, 50, size=(40, 5000)).astype(np.int32)
+    for ax in (0, 1):
+        ref, got = both(H, G, lambda t: t.findAxis(7, ax), x)
+        assert_exact(ref, got)
+    ref, got = both(H, G, lambda t: t.findAxis(1000, 1), x)
+    assert (got == NOT_FOUND).all()
+    assert_exact(ref, got)
+    a = np.array([[1.0, 2.0, 3.0, 4.0], [5.0, 6.0, 7.0, 3.0]])
+    assert G.toNumpy(G.ofNumpy(a).findAxis(3.0, 1)).tolist() == [2, 3]          # Guide-Index.md:52-57
+    assert G.ofNumpy(a).tryFind(3.0) == [0, 2]                                   # Guide-Index.md:44-49
+
+
+def test_strided_reduce_axis(H, G, rng):
+    x = rng.standard_normal((50, 60, 70)).astype(np.float32)
+    # reduce over a middle axis of a sliced, permuted view
+    def f(t):
+        v = t[5:45, :, 3:60].permuteAxes([1, 2, 0])
+        return v.maxAxis(0), v.maxAxis(1), v.maxAxis(2), v.argMaxAxis(1)
+    ref, got = both(H, G, f, x)
+    for r, g in zip(ref, got):
+        assert_exact(r, g)
+    # a single strided column reduced to a scalar
+    ref, got = both(H, G, lambda t: t[:, 7, 9].maxAxis(0), x)
+    assert_exact(ref, got)
