@@ -1,0 +1,231 @@
+"""Per-configuration timings of the HIP backend (used by `bench.py --all`): the five synthetic workloads of the
+benchmark definition, one line per backend call with its algorithmic bytes (or FLOPs), HIP-event time and fraction of
+the roofline that bounds it.  Inputs come from seed 123; an op whose working set is below ~600 MB is launched over
+several independent buffer sets in rotation so that the 256 MB Infinity Cache cannot serve re-reads."""
+import ctypes as C
+import math
+
+import numpy as np
+
+HBM_PEAK_GBS = 8000.0
+FP32_MFMA_PEAK_TFLOPS = 157.3
+
+
+class Timer:
+    def __init__(self):
+        from deepnet_amd import native
+        self.native = native
+        self.lib = native.load()
+        self.stream = C.c_void_p(0)
+        self.e0, self.e1 = C.c_void_p(), C.c_void_p()
+        native.check(self.lib.dnh_event_create(C.byref(self.e0)))
+        native.check(self.lib.dnh_event_create(C.byref(self.e1)))
+
+    def issue(self, call):
+        entry, args = call
+        self.native.check(getattr(self.lib, "dnh_" + entry)(*args, self.stream))
+
+    def time(self, sets, reps=20, warm=3):
+        """sets: list of call lists (one list of (entry, args) per buffer set).  Returns average ms per pass over one set."""
+        lib, check = self.lib, self.native.check
+        for i in range(warm):
+            for call in sets[i % len(sets)]:
+                self.issue(call)
+        check(lib.dnh_device_sync())
+        check(lib.dnh_event_record(self.e0, self.stream))
+        for i in range(reps):
+            for call in sets[i % len(sets)]:
+                self.issue(call)
+        check(lib.dnh_event_record(self.e1, self.stream))
+        check(lib.dnh_event_sync(self.e1))
+        ms = C.c_float()
+        check(lib.dnh_event_elapsed_ms(self.e0, self.e1, C.byref(ms)))
+        return ms.value / reps
+
+
+def nsets_for(nbytes):
+    return max(1, min(40, math.ceil(600e6 / max(nbytes, 1))))
+
+
+def report(log, cfg, name, ms, nbytes=None, flops=None):
+    if flops:
+        tf = flops / (ms * 1e-3) / 1e12
+        log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {tf:8.2f} TFLOP/s  {100 * tf / FP32_MFMA_PEAK_TFLOPS:5.1f}% of fp32 MFMA peak")
+        return {"cfg": cfg, "op": name, "ms": ms, "TFLOPs": tf, "frac": tf / FP32_MFMA_PEAK_TFLOPS}
+    gb = nbytes / (ms * 1e-3) / 1e9
+    log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {gb:8.1f} GB/s  {100 * gb / HBM_PEAK_GBS:5.1f}% of HBM peak  ({nbytes / 1e6:.1f} MB)")
+    return {"cfg": cfg, "op": name, "ms": ms, "GBps": gb, "frac": gb / HBM_PEAK_GBS}
+
+
+def run_all(log, which=(1, 2, 3, 4, 5)):
+    from deepnet_amd import abi, hip as G
+    from deepnet_amd.backend import CAbiTensorBackend
+    from deepnet_amd.tensor import Tensor
+    T = Timer()
+    rng = np.random.default_rng(123)
+    keep = []
+    results = []
+
+    def D(t):
+        d = CAbiTensorBackend._desc(t)
+        keep.append((t, d))
+        return C.byref(d)
+
+    def new(shape, dt):
+        return Tensor.new(shape, G.Dev, dt)
+
+    def timed(cfg, name, nbytes, build, flops=None, reps=20):
+        ns = nsets_for(nbytes)
+        sets = [build(i) for i in range(ns)]
+        ms = T.time(sets, reps=max(reps, ns))
+        results.append(report(log, cfg, name, ms, nbytes, flops))
+        keep.clear()
+
+    f32 = np.float32
+    if 1 in which:
+        n = 4096
+        N = n * n
+        base = [rng.uniform(-1, 1, (n, n)).astype(f32) for _ in range(3)]
+
+        def chain_set(i):
+            a, b, c = (G.ofNumpy(x) for x in base)
+            t1, t2, y, t3, t4, out = (new([n, n], f32) for _ in range(6))
+            return [("binary", (abi.DNH_MULTIPLY, D(t1), D(a), D(b))), ("binary", (abi.DNH_ADD, D(t2), D(t1), D(c))),
+                    ("unary", (abi.DNH_TANH, D(y), D(t2))), ("binary", (abi.DNH_MULTIPLY, D(t3), D(y), D(y))),
+                    ("unary", (abi.DNH_UNARY_MINUS, D(t4), D(t3))), ("unary", (abi.DNH_EXP, D(out), D(t4)))]
+        names = [("Multiply a*b", 3), ("Add t1+c", 3), ("Tanh", 2), ("Multiply y*y", 2), ("UnaryMinus", 2), ("Exp", 2)]
+        sets = [chain_set(i) for i in range(4)]
+        for k, (nm, mult) in enumerate(names):
+            ms = T.time([[s[k]] for s in sets], reps=20)
+            results.append(report(log, 1, nm + " 4096x4096", ms, mult * N * 4))
+        ms = T.time(sets, reps=12)
+        results.append(report(log, 1, "chain of 6 calls (eager)", ms, 14 * N * 4))
+        keep.clear()
+        del sets
+
+    if 2 in which:
+        x = G.ofNumpy(rng.standard_normal((256, 512, 1024), dtype=f32))
+        v = G.ofNumpy(rng.random(1024, dtype=f32))
+        N = 256 * 512 * 1024
+        xp = x.permuteAxes([2, 0, 1])                       # shape [512, 1024, 256], strides [1024, 1, 524288]
+        vb = v[None, :, None].broadcastTo(xp.Shape)         # strides [0, 1, 0]
+        y = new(xp.Shape, f32)
+        timed(2, "Add permuted x + broadcast v", 2 * N * 4 + 4096, lambda i: [("binary", (abi.DNH_ADD, D(y), D(xp), D(vb)))], reps=10)
+        timed(2, "Copy permuted x -> contiguous", 2 * N * 4, lambda i: [("copy", (D(y), D(xp)))], reps=10)
+        # the NumPy reading of "axes (2,0,1)": shape [1024, 256, 512], strides [1, 524288, 1024]
+        xq = x.permuteAxes([1, 2, 0])
+        vq = v[:, None, None].broadcastTo(xq.Shape)
+        yq = new(xq.Shape, f32)
+        timed(2, "Add (NumPy-convention permute)", 2 * N * 4 + 4096, lambda i: [("binary", (abi.DNH_ADD, D(yq), D(xq), D(vq)))], reps=10)
+        del x, v, xp, vb, y, xq, vq, yq
+
+    if 3 in which:
+        n = 8192
+        N = n * n
+        for dt, s in ((np.float32, 4), (np.float64, 8)):
+            a = G.ofNumpy(rng.standard_normal((n, n)).astype(dt) if dt == np.float32 else rng.uniform(-1, 1, (n, n)))
+            b = G.ofNumpy(G.toNumpy(a) * dt(0.5))
+            srcs = [a, b]
+            vec = new([n], dt)
+            ivec = new([n], np.int64)
+            sc = new([], dt)
+            nm = np.dtype(dt).name
+            for label, view in (("last axis", lambda t: t), ("first axis", lambda t: t.permuteAxes([1, 0]))):
+                timed(3, f"Sum {label} {nm}", N * s + n * s, lambda i: [("reduce_last_axis", (abi.DNH_SUM, D(vec), D(view(srcs[i % 2]))))])
+                timed(3, f"Max {label} {nm}", N * s + n * s, lambda i: [("reduce_last_axis", (abi.DNH_MAX, D(vec), D(view(srcs[i % 2]))))])
+                timed(3, f"ArgMax {label} {nm}", N * s + n * 8, lambda i: [("arg_reduce_last_axis", (abi.DNH_ARG_MAX, D(ivec), D(view(srcs[i % 2]))))])
+            timed(3, f"Sum full {nm}", N * s + s, lambda i: [("reduce_last_axis", (abi.DNH_SUM, D(sc), D(srcs[i % 2].flatten())))])
+            del a, b, srcs
+
+    if 4 in which:
+        N, M = 1 << 24, 1 << 22
+        ha = rng.integers(-1000, 1001, N).astype(np.int32)
+        hb = rng.integers(-1000, 1001, N).astype(np.int32)
+        hidx = rng.integers(0, N, M).astype(np.int64)
+        hidxu = rng.permutation(N)[:M].astype(np.int64)
+        K = int((ha > 0).sum())
+        zero = G.scalar(0, np.int32)
+
+        def mk():
+            a, b = G.ofNumpy(ha), G.ofNumpy(hb)
+            m = new([N], np.bool_)
+            m.Backend.Greater(m, a, zero.broadcastTo([N]))
+            return a, b, m
+        timed(4, "Greater int32 > 0 -> bool", N * 4 + N + 4,
+              lambda i: (lambda a, b, m: [("compare", (abi.DNH_GREATER, D(m), D(a), D(zero.broadcastTo([N]))))])(*mk()))
+        timed(4, "IfThenElse bool,int32,int32", N + 3 * N * 4,
+              lambda i: (lambda a, b, m: [("if_then_else", (D(new([N], np.int32)), D(m), D(a), D(b)))])(*mk()))
+        cnt = new([], np.int64)
+        timed(4, "CountTrue bool[16Mi]", N + 8,
+              lambda i: (lambda a, b, m: [("reduce_last_axis", (abi.DNH_COUNT_TRUE, D(cnt), D(m)))])(*mk()))
+
+        def mget(i):
+            a, b, m = mk()
+            arr = (C.POINTER(abi.DnhTensor) * 1)()
+            dm = CAbiTensorBackend._desc(m)
+            keep.append((m, dm, arr))
+            arr[0] = C.pointer(dm)
+            return [("masked_get", (D(new([K], np.int32)), D(a), arr, 1))]
+        timed(4, "MaskedGet int32 by bool mask", 2 * N + N * 4 + K * 4, mget)
+
+        def gat(i):
+            a = G.ofNumpy(ha)
+            idx = G.ofNumpy(hidx)
+            arr = (C.POINTER(abi.DnhTensor) * 1)()
+            di = CAbiTensorBackend._desc(idx)
+            keep.append((idx, di, arr))
+            arr[0] = C.pointer(di)
+            return [("gather", (D(new([M], np.int32)), arr, 1, D(a)))]
+        timed(4, "Gather 4Mi int64 idx from 16Mi", M * 8 + M * 4 + M * 4, gat)
+
+        def sca(i):
+            src = G.ofNumpy(ha[:M])
+            idx = G.ofNumpy(hidxu)
+            t = new([N], np.int32)
+            arr = (C.POINTER(abi.DnhTensor) * 1)()
+            di = CAbiTensorBackend._desc(idx)
+            z = np.zeros(1, np.int32)
+            keep.append((idx, di, arr, z))
+            arr[0] = C.pointer(di)
+            return [("fill_const", (D(t), z.ctypes.data_as(C.c_void_p))), ("scatter", (D(t), arr, 1, D(src)))]
+        timed(4, "FillConst 0 + Scatter (unique idx)", N * 4 + M * 8 + M * 4 + M * 4, sca)
+
+    if 5 in which:
+        Bn, n = 64, 512
+        N = Bn * n * n
+        R = Bn * n
+        sd = 1.0 / math.sqrt(512.0)
+        ha = (rng.standard_normal((Bn, n, n)) * sd).astype(f32)
+        hb = (rng.standard_normal((Bn, n, n)) * sd).astype(f32)
+
+        def mk5():
+            return G.ofNumpy(ha), G.ofNumpy(hb), new([Bn, n, n], f32)
+        timed(5, "BatchedMatMatDot 64x512^3 fp32", 3 * N * 4, lambda i: (lambda a, b, c: [("dot", (D(c), D(a), D(b)))])(*mk5()),
+              flops=2.0 * Bn * n ** 3)
+        timed(5, "Tanh [64,512,512]", 2 * N * 4, lambda i: (lambda a, b, c: [("unary", (abi.DNH_TANH, D(c), D(a)))])(*mk5()))
+        timed(5, "MaxAxis 2 (rows of 512)", N * 4 + R * 4,
+              lambda i: (lambda a, b, c: [("reduce_last_axis", (abi.DNH_MAX, D(new([Bn, n], f32)), D(a)))])(*mk5()))
+
+        def sub5(i):
+            a, b, c = mk5()
+            mx = new([Bn, n], f32)
+            mx.Backend.MaxLastAxis(mx, a)
+            return [("binary", (abi.DNH_SUBTRACT, D(c), D(a), D(mx[:, :, None].broadcastTo([Bn, n, n]))))]
+        timed(5, "Subtract t - rowmax (broadcast)", 2 * N * 4 + R * 4, sub5)
+        timed(5, "Exp [64,512,512]", 2 * N * 4, lambda i: (lambda a, b, c: [("unary", (abi.DNH_EXP, D(c), D(a)))])(*mk5()))
+        timed(5, "SumAxis 2 (rows of 512)", N * 4 + R * 4,
+              lambda i: (lambda a, b, c: [("reduce_last_axis", (abi.DNH_SUM, D(new([Bn, n], f32)), D(a)))])(*mk5()))
+
+        def div5(i):
+            a, b, c = mk5()
+            sm = new([Bn, n], f32)
+            sm.Backend.SumLastAxis(sm, a)
+            return [("binary", (abi.DNH_DIVIDE, D(c), D(a), D(sm[:, :, None].broadcastTo([Bn, n, n]))))]
+        timed(5, "Divide e / rowsum (broadcast)", 2 * N * 4 + R * 4, div5)
+    return results
+
+
+if __name__ == "__main__":
+    import sys
+    which = tuple(int(x) for x in sys.argv[1:]) or (1, 2, 3, 4, 5)
+    run_all(lambda *a: print(*a, flush=True), which)
