@@ -181,26 +181,50 @@ struct TrArgs {
     uint32_t na, nb, tiles_a, tiles_b;
     int64_t sa[kMaxOperands], sb[kMaxOperands];   // element strides along A and B
     int staged[kMaxOperands];                     // source k goes through LDS
+    uint32_t lds_off[kMaxOperands];               // byte offset of source k's tile in dynamic LDS (staged sources only)
 };
 
-template <class Op, int TILE>
+// Direct (not LDS-staged) operand fetch of the transposing kernel for VEC consecutive positions tx.. along B at row r along A:
+// one vector when the operand runs along B, one scalar when it is broadcast along B, element by element otherwise.
+template <class X, int VEC>
+__device__ __forceinline__ Pack<X, VEC> tr_direct(const X* g, uint32_t r, uint32_t tx, int64_t sa, int64_t sb) {
+    const X* q = g + (int64_t)r * sa + (int64_t)tx * sb;
+    if (sb == 0) return splat_pack<X, VEC>(*q);
+    if (sb == 1 && VEC > 1 && (((uintptr_t)q) % (VEC * sizeof(X))) == 0) return load_pack<X, VEC>(q);
+    Pack<X, VEC> v;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) v.v[e] = q[(int64_t)e * sb];
+    return v;
+}
+
+template <class Op, int TILE, int VEC>
 __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t, const typename Op::A* a, const typename Op::B* b,
                                                         const typename Op::C* c, TrArgs p) {
     using T = typename Op::T;
     using A = typename Op::A;
     using B = typename Op::B;
     using C = typename Op::C;
-    constexpr int ROWS = kBlock / TILE;  // rows of the tile covered per pass
-    __shared__ A la[Op::NSRC >= 1 ? TILE : 1][TILE + 1];
-    __shared__ B lb[Op::NSRC >= 2 ? TILE : 1][TILE + 1];
-    __shared__ C lc[Op::NSRC >= 3 ? TILE : 1][TILE + 1];
+    constexpr int TV = TILE / VEC;       // threads per tile row (each handles VEC consecutive elements)
+    constexpr int ROWS = kBlock / TV;    // tile rows covered per pass
+    constexpr int ITER = TILE / ROWS;    // passes
+    // only staged sources own an LDS tile ([TILE][TILE+1] elements each), so occupancy is not spent on unused tiles
+    extern __shared__ __align__(16) unsigned char tr_lds[];
+    typedef A (*TileA)[TILE + 1];
+    typedef B (*TileB)[TILE + 1];
+    typedef C (*TileC)[TILE + 1];
+    TileA la = (TileA)(tr_lds + p.lds_off[1]);
+    TileB lb = (TileB)(tr_lds + p.lds_off[2]);
+    TileC lc = (TileC)(tr_lds + p.lds_off[3]);
 
     uint32_t bid = blockIdx.x;
     const uint32_t tb = bid % p.tiles_b;
     bid /= p.tiles_b;
     const uint32_t ta = bid % p.tiles_a;
     bid /= p.tiles_a;
-    int64_t off[kMaxOperands] = {0, 0, 0, 0};
+    const uint32_t a0 = ta * TILE, b0 = tb * TILE;
+    int64_t off[kMaxOperands];
+#pragma unroll
+    for (int k = 0; k <= Op::NSRC; k++) off[k] = (int64_t)a0 * p.sa[k] + (int64_t)b0 * p.sb[k];
     for (int d = p.nouter - 1; d >= 0; d--) {
         const uint32_t q = (d == 0) ? 0u : bid / p.oshape[d];
         const uint32_t idx = bid - q * p.oshape[d];
@@ -208,42 +232,80 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
 #pragma unroll
         for (int k = 0; k <= Op::NSRC; k++) off[k] += (int64_t)idx * p.ostride[k][d];
     }
-    const uint32_t a0 = ta * TILE, b0 = tb * TILE;
-    const uint32_t tx = threadIdx.x % TILE, ty = threadIdx.x / TILE;
+    t += off[0];
+    if constexpr (Op::NSRC >= 1) a += off[1];
+    if constexpr (Op::NSRC >= 2) b += off[2];
+    if constexpr (Op::NSRC >= 3) c += off[3];
+    const uint32_t tx = (threadIdx.x % TV) * VEC, ty = threadIdx.x / TV;
+    const uint32_t la_n = p.na - a0 < (uint32_t)TILE ? p.na - a0 : TILE;   // valid extent of this tile along A and B
+    const uint32_t lb_n = p.nb - b0 < (uint32_t)TILE ? p.nb - b0 : TILE;
 
-    // stage: lanes run along A (the staged sources' unit-stride dimension); LDS tile is [b][a]
-    {
-        const uint32_t ia = a0 + tx;
-        if (ia < p.na) {
-            for (uint32_t r = ty; r < TILE; r += ROWS) {
-                const uint32_t ib = b0 + r;
-                if (ib < p.nb) {
-                    if constexpr (Op::NSRC >= 1)
-                        if (p.staged[1]) la[r][tx] = a[off[1] + (int64_t)ia * p.sa[1] + (int64_t)ib * p.sb[1]];
-                    if constexpr (Op::NSRC >= 2)
-                        if (p.staged[2]) lb[r][tx] = b[off[2] + (int64_t)ia * p.sa[2] + (int64_t)ib * p.sb[2]];
-                    if constexpr (Op::NSRC >= 3)
-                        if (p.staged[3]) lc[r][tx] = c[off[3] + (int64_t)ia * p.sa[3] + (int64_t)ib * p.sb[3]];
-                }
+    // stage: lanes run along A (the staged sources' unit-stride dimension); the LDS tile is [b][a]
+    if (tx < la_n) {
+#pragma unroll
+        for (int it = 0; it < ITER; it++) {
+            const uint32_t r = ty + it * ROWS;
+            if (r < lb_n) {
+                if constexpr (Op::NSRC >= 1)
+                    if (p.staged[1]) {
+                        const Pack<A, VEC> v = load_pack<A, VEC>(a + (int64_t)r * p.sb[1] + tx);
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) la[r][tx + e] = v.v[e];
+                    }
+                if constexpr (Op::NSRC >= 2)
+                    if (p.staged[2]) {
+                        const Pack<B, VEC> v = load_pack<B, VEC>(b + (int64_t)r * p.sb[2] + tx);
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) lb[r][tx + e] = v.v[e];
+                    }
+                if constexpr (Op::NSRC >= 3)
+                    if (p.staged[3]) {
+                        const Pack<C, VEC> v = load_pack<C, VEC>(c + (int64_t)r * p.sb[3] + tx);
+#pragma unroll
+                        for (int e = 0; e < VEC; e++) lc[r][tx + e] = v.v[e];
+                    }
+            }
+        }
+    }
+    // Operands that are not staged are read in the store pattern (lanes along B).  All of these loads are issued before
+    // the first store: on this architecture loads and stores retire through one in-order counter, so a load placed
+    // after a store would wait for that store to complete.
+    Pack<A, VEC> da[ITER];
+    Pack<B, VEC> db[ITER];
+    Pack<C, VEC> dc[ITER];
+    if (tx < lb_n) {
+#pragma unroll
+        for (int it = 0; it < ITER; it++) {
+            const uint32_t r = ty + it * ROWS;
+            if (r < la_n) {
+                if constexpr (Op::NSRC >= 1)
+                    if (!p.staged[1]) da[it] = tr_direct<A, VEC>(a, r, tx, p.sa[1], p.sb[1]);
+                if constexpr (Op::NSRC >= 2)
+                    if (!p.staged[2]) db[it] = tr_direct<B, VEC>(b, r, tx, p.sa[2], p.sb[2]);
+                if constexpr (Op::NSRC >= 3)
+                    if (!p.staged[3]) dc[it] = tr_direct<C, VEC>(c, r, tx, p.sa[3], p.sb[3]);
             }
         }
     }
     __syncthreads();
-    // compute + store: lanes run along B (the target's unit-stride dimension)
-    {
-        const uint32_t ib = b0 + tx;
-        if (ib < p.nb) {
-            for (uint32_t r = ty; r < TILE; r += ROWS) {
-                const uint32_t ia = a0 + r;
-                if (ia < p.na) {
+    // compute + store: lanes run along B (the target's unit-stride dimension), VEC consecutive elements per thread
+    if (tx < lb_n) {
+#pragma unroll
+        for (int it = 0; it < ITER; it++) {
+            const uint32_t r = ty + it * ROWS;
+            if (r < la_n) {
+                Pack<T, VEC> res;
+#pragma unroll
+                for (int e = 0; e < VEC; e++) {
                     A xa = A();
                     B xb = B();
                     C xc = C();
-                    if constexpr (Op::NSRC >= 1) xa = p.staged[1] ? la[tx][r] : a[off[1] + (int64_t)ia * p.sa[1] + (int64_t)ib * p.sb[1]];
-                    if constexpr (Op::NSRC >= 2) xb = p.staged[2] ? lb[tx][r] : b[off[2] + (int64_t)ia * p.sa[2] + (int64_t)ib * p.sb[2]];
-                    if constexpr (Op::NSRC >= 3) xc = p.staged[3] ? lc[tx][r] : c[off[3] + (int64_t)ia * p.sa[3] + (int64_t)ib * p.sb[3]];
-                    t[off[0] + (int64_t)ia * p.sa[0] + (int64_t)ib * p.sb[0]] = apply_op(op, xa, xb, xc);
+                    if constexpr (Op::NSRC >= 1) xa = p.staged[1] ? la[tx + e][r] : da[it].v[e];
+                    if constexpr (Op::NSRC >= 2) xb = p.staged[2] ? lb[tx + e][r] : db[it].v[e];
+                    if constexpr (Op::NSRC >= 3) xc = p.staged[3] ? lc[tx + e][r] : dc[it].v[e];
+                    res.v[e] = apply_op(op, xa, xb, xc);
                 }
+                store_pack<T, VEC>(t + (int64_t)r * p.sa[0] + tx, res);
             }
         }
     }
@@ -292,7 +354,8 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
         for (int k = 1; k < NOPS; k++)
             if (p.stride[k][0] == 1) al = al && aligned_to(p.ptr[k], VEC * es[k]);
         if (al) {
-            constexpr int UNROLL = 4;
+            // one 16-byte vector per thread: measured fastest on MI355X (more per-thread unrolling lowers achieved bandwidth)
+            constexpr int UNROLL = 1;
             const int64_t nvec = p.total / VEC;
             const unsigned blocks = nvec ? cdiv(nvec, (int64_t)kBlock * UNROLL) : 1;
             hipLaunchKernelGGL((map_flat_kernel<Op, VEC, UNROLL>), dim3(blocks), dim3(kBlock), 0, stream, op, t, a, b, c,
@@ -348,9 +411,24 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 q.sb[k] = p.stride[k][last];
                 q.staged[k] = (k >= 1 && p.stride[k][dA] == 1 && p.stride[k][last] != 0 && p.stride[k][last] != 1) ? 1 : 0;
             }
+            uint32_t lds_bytes = 0;
+            for (int k = 1; k < NOPS; k++) {
+                if (!q.staged[k]) continue;
+                q.lds_off[k] = lds_bytes;
+                lds_bytes += (uint32_t)((TILE * (TILE + 1) * es[k] + 15) / 16 * 16);
+            }
             const int64_t blocks = (int64_t)q.tiles_a * q.tiles_b * outer;
+            // vector path: every tile row a whole number of aligned vectors for the target and every staged source
+            bool vec = VEC > 1 && (q.na % VEC) == 0 && (q.nb % VEC) == 0 && aligned_to(t, VEC * es[0]) && (q.sa[0] % VEC) == 0;
+            for (int d = 0; d < q.nouter && vec; d++) vec = (q.ostride[0][d] % VEC) == 0;
+            for (int k = 1; k < NOPS && vec; k++) {
+                if (!q.staged[k]) continue;
+                vec = aligned_to(p.ptr[k], VEC * es[k]) && (q.sb[k] % VEC) == 0;
+                for (int d = 0; d < q.nouter && vec; d++) vec = (q.ostride[k][d] % VEC) == 0;
+            }
             if (blocks <= 0x7FFFFFFF) {
-                hipLaunchKernelGGL((map_tr_kernel<Op, TILE>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, op, t, a, b, c, q);
+                if (vec) hipLaunchKernelGGL((map_tr_kernel<Op, TILE, (VEC < TILE ? VEC : 1)>), dim3((unsigned)blocks), dim3(kBlock), lds_bytes, stream, op, t, a, b, c, q);
+                else hipLaunchKernelGGL((map_tr_kernel<Op, TILE, 1>), dim3((unsigned)blocks), dim3(kBlock), lds_bytes, stream, op, t, a, b, c, q);
                 DNH_LAUNCH_CHECK();
                 return DNH_OK;
             }
@@ -373,7 +451,7 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
     for (int d = 0; d < last && vec; d++)
         for (int k = 0; k < NOPS; k++)
             if (p.stride[k][last] == 1) vec = vec && (p.stride[k][d] % VEC) == 0;
-    constexpr int UNROLL = 2;
+    constexpr int UNROLL = 1;
     if (vec) {
         q.shape[last] = (uint32_t)(p.shape[last] / VEC);
         for (int k = 0; k < NOPS; k++) {

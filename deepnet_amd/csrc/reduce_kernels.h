@@ -126,17 +126,17 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(R r, const void* sr
     }
 }
 
-template <class R, int VEC>
+template <class R, int VEC, int WX>
 __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(R r, const typename R::In* src, typename R::Out* out,
                                                              typename R::State* partial, OuterArgs o, uint32_t col_tiles, uint32_t nc,
                                                              int64_t tc_stride, int64_t n, int64_t sr, int64_t chunk, uint32_t splits) {
     using State = typename R::State;
     using In = typename R::In;
-    constexpr int NY = kBlock / 64;
-    constexpr int U = 4;
-    const uint32_t x = threadIdx.x & 63, y = threadIdx.x >> 6;
+    constexpr int NY = kBlock / WX;
+    constexpr int U = 2;
+    const uint32_t x = threadIdx.x % WX, y = threadIdx.x / WX;
     const uint32_t tile = blockIdx.x % col_tiles, other = blockIdx.x / col_tiles;
-    const uint32_t col0 = (tile * 64 + x) * VEC;
+    const uint32_t col0 = (tile * WX + x) * VEC;
     int64_t toff, soff;
     outer_offsets(o, other, toff, soff);
     const int64_t r0 = (int64_t)blockIdx.y * chunk;
@@ -163,18 +163,24 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(R r, const typename
             for (int e = 0; e < VEC; e++) st[e] = r.step(st[e], v.v[e], i);
         }
     }
-    __shared__ State sh[NY - 1][64 * VEC];
-    if (y > 0) {
+    if constexpr (NY > 1) {
+        __shared__ State sh[NY - 1][WX * VEC];
+        if (y > 0) {
 #pragma unroll
-        for (int e = 0; e < VEC; e++) sh[y - 1][x * VEC + e] = st[e];
+            for (int e = 0; e < VEC; e++) sh[y - 1][x * VEC + e] = st[e];
+        }
+        __syncthreads();
+        if (y == 0) {
+#pragma unroll
+            for (int e = 0; e < VEC; e++)
+#pragma unroll
+                for (int w = 0; w < NY - 1; w++) st[e] = r.combine(st[e], sh[w][x * VEC + e]);
+        }
     }
-    __syncthreads();
     if (y == 0 && active) {
 #pragma unroll
         for (int e = 0; e < VEC; e++) {
             State s = st[e];
-#pragma unroll
-            for (int w = 0; w < NY - 1; w++) s = r.combine(s, sh[w][x * VEC + e]);
             const uint32_t col = col0 + e;
             if (splits == 1) out[toff + (int64_t)col * tc_stride] = r.extract(s);
             else partial[((int64_t)other * nc + col) * splits + blockIdx.y] = s;
@@ -196,6 +202,21 @@ __global__ __launch_bounds__(kBlock) void reduce_generic_kernel(R r, const typen
 }
 
 // ---- host-side strategy --------------------------------------------------------------------------------------------------
+
+// Finishing pass of the two-pass tree: `nout` rows of `splits` State partials each.
+template <class R>
+int32_t launch_finish(const R& r, typename R::State* partial, typename R::Out* out, const OuterArgs& o, uint32_t nout, uint32_t splits,
+                      hipStream_t stream) {
+    using State = typename R::State;
+#define DNH_FIN(TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, 1, TPR, true>), dim3(cdiv(nout, kBlock / TPR)), dim3(kBlock), 0, stream, r, \
+                                        (const void*)partial, out, (State*)nullptr, o, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u)
+    if (splits > 512) DNH_FIN(256);
+    else if (splits > 32) DNH_FIN(64);
+    else DNH_FIN(16);
+#undef DNH_FIN
+    DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
 
 template <class R>
 int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStream_t stream, const char* what) {
@@ -281,14 +302,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         DNH_LAUNCH_CHECK();
         if (splits > 1) {
             // finishing pass: rows of `splits` State partials
-            if (splits > 64) {
-                hipLaunchKernelGGL((reduce_rows_kernel<R, 1, 256, true>), dim3(nout), dim3(kBlock), 0, stream, r, (const void*)partial, out,
-                                   (State*)nullptr, o, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u);
-            } else {
-                hipLaunchKernelGGL((reduce_rows_kernel<R, 1, 16, true>), dim3(cdiv(nout, 16)), dim3(kBlock), 0, stream, r, (const void*)partial, out,
-                                   (State*)nullptr, o, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u);
-            }
-            DNH_LAUNCH_CHECK();
+            DNH_TRY(launch_finish(r, partial, out, o, nout, splits, stream));
         }
         return DNH_OK;
     }
@@ -311,29 +325,39 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         bool vec = VEC > 1 && aligned_to(src, 16) && (nc % VEC) == 0 && (sr % VEC) == 0;
         for (int d = 0; d < oo.nd && vec; d++) vec = (oo.sstride[d] % VEC) == 0;
         const int v = vec ? VEC : 1;
-        const uint32_t col_tiles = cdiv(nc, 64 * v);
-        const int64_t base_blocks = (int64_t)col_tiles * others;
-        uint32_t splits = 1;
-        int64_t chunk = n;
-        if (base_blocks < target_blocks) {
-            const int64_t min_chunk = 64;
-            int64_t want = (target_blocks + base_blocks - 1) / base_blocks;
-            int64_t maxs = (n + min_chunk - 1) / min_chunk;
-            int64_t sp = want < maxs ? want : maxs;
-            if (sp > 1) {
-                chunk = (n + sp - 1) / sp;
-                splits = (uint32_t)((n + chunk - 1) / chunk);
-                if (splits <= 1) { splits = 1; chunk = n; }
+        // Lanes along the kept dimension: the whole block when that still yields about four blocks per CU (4 KB contiguous per
+        // row visit, no LDS step), else 64 lanes x 4 wavefronts sharing the reduced axis.  A block never takes fewer rows than
+        // keeps the State partials (written and re-read once) near 1/64 of the source traffic.
+        const int64_t min_rows = 64 * (int64_t)((sizeof(State) + sizeof(In) - 1) / sizeof(In));
+        int wx = 256;
+        uint32_t col_tiles = 1, splits = 1;
+        int64_t base_blocks = 1, chunk = n;
+        for (;;) {
+            col_tiles = cdiv(nc, wx * v);
+            base_blocks = (int64_t)col_tiles * others;
+            const int64_t maxs = (n + min_rows - 1) / min_rows;
+            if (wx == 64 || (nc >= (uint32_t)(256 * v) && base_blocks * maxs >= (int64_t)cus * 4)) {
+                const int64_t want = ((int64_t)cus * 4 + base_blocks - 1) / base_blocks;
+                const int64_t sp = want < maxs ? want : maxs;
+                splits = 1;
+                chunk = n;
+                if (sp > 1) {
+                    chunk = (n + sp - 1) / sp;
+                    splits = (uint32_t)((n + chunk - 1) / chunk);
+                    if (splits <= 1) { splits = 1; chunk = n; }
+                }
+                break;
             }
+            wx = 64;
         }
         if (base_blocks <= 0x7FFFFFFF && splits <= 65535) {
             State* partial = nullptr;
             if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial));
             const dim3 grid((unsigned)base_blocks, splits);
-            if (vec)
-                hipLaunchKernelGGL((reduce_cols_kernel<R, VEC>), grid, dim3(kBlock), 0, stream, r, src, out, partial, oo, col_tiles, nc, tc_stride, n, sr, chunk, splits);
-            else
-                hipLaunchKernelGGL((reduce_cols_kernel<R, 1>), grid, dim3(kBlock), 0, stream, r, src, out, partial, oo, col_tiles, nc, tc_stride, n, sr, chunk, splits);
+#define DNH_COLS(V, W) hipLaunchKernelGGL((reduce_cols_kernel<R, V, W>), grid, dim3(kBlock), 0, stream, r, src, out, partial, oo, col_tiles, nc, tc_stride, n, sr, chunk, splits)
+            if (vec) { if (wx == 256) DNH_COLS(VEC, 256); else DNH_COLS(VEC, 64); }
+            else { if (wx == 256) DNH_COLS(1, 256); else DNH_COLS(1, 64); }
+#undef DNH_COLS
             DNH_LAUNCH_CHECK();
             if (splits > 1) {
                 // partials are laid out [others][nc][splits]; enumerate outputs in that order for the finishing pass
@@ -342,13 +366,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
                 fo.tstride[fo.nd] = tc_stride;
                 fo.sstride[fo.nd] = 0;
                 fo.nd++;
-                if (splits > 64)
-                    hipLaunchKernelGGL((reduce_rows_kernel<R, 1, 256, true>), dim3(nout), dim3(kBlock), 0, stream, r, (const void*)partial, out,
-                                       (State*)nullptr, fo, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u);
-                else
-                    hipLaunchKernelGGL((reduce_rows_kernel<R, 1, 16, true>), dim3(cdiv(nout, 16)), dim3(kBlock), 0, stream, r, (const void*)partial, out,
-                                       (State*)nullptr, fo, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u);
-                DNH_LAUNCH_CHECK();
+                DNH_TRY(launch_finish(r, partial, out, fo, nout, splits, stream));
             }
             return DNH_OK;
         }
