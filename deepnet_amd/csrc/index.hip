@@ -259,6 +259,150 @@ __global__ __launch_bounds__(kBlock) void compact_move_kernel(MaskArgs m, W* ful
     }
 }
 
+// ---- contiguous 1-d fast path ------------------------------------------------------------------------------------------------
+// Rank-1 unit-stride data and mask (the `a.M(mask)` form after the frontend's reshape/flatten, Tensor.fs:3044-3052): a block
+// covers kFastJ * 256 vectors of VEC elements; thread t owns vector t of each of the kFastJ segments, so mask bytes and data
+// are read with fully coalesced vector loads and no index arithmetic.  Ranks follow the element order (segment, thread,
+// element): the per-segment counts of a thread are packed into one 64-bit word (16 bits each) and scanned together.
+constexpr int kFastJ = 4;
+
+template <int VEC>
+__device__ __forceinline__ uint32_t mask_flags(const uint8_t* m) {
+    const Pack<uint8_t, VEC> v = load_pack<uint8_t, VEC>(m);
+    uint32_t f = 0;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) f |= (uint32_t)(v.v[e] != 0) << e;
+    return f;
+}
+
+__device__ __forceinline__ uint64_t block_exclusive_scan64(uint64_t c, uint64_t* total) {
+    __shared__ uint64_t wave_sum[kBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint64_t inc = c;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t lo = (uint32_t)__shfl_up((int)(uint32_t)inc, d, 64);
+        const uint32_t hi = (uint32_t)__shfl_up((int)(uint32_t)(inc >> 32), d, 64);
+        if (lane >= d) inc += ((uint64_t)hi << 32) | lo;
+    }
+    if (lane == 63) wave_sum[wave] = inc;
+    __syncthreads();
+    uint64_t base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; w++) {
+        if (w < wave) base += wave_sum[w];
+        tot += wave_sum[w];
+    }
+    *total = tot;
+    return base + inc - c;
+}
+
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void compact_count_fast_kernel(const uint8_t* mask, uint32_t nvec, uint32_t* counts) {
+    uint32_t c = 0;
+#pragma unroll
+    for (int j = 0; j < kFastJ; j++) {
+        const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+        if (v < nvec) c += __popc(mask_flags<VEC>(mask + (size_t)v * VEC));
+    }
+    uint32_t total;
+    block_exclusive_scan(c, &total);
+    if (threadIdx.x == 0) counts[blockIdx.x] = total;
+}
+
+// SET = false: out[k] = full[i] (MaskedGet);  SET = true: full[i] = out[k] (MaskedSet)
+// Sum of counts[0..n): the exclusive prefix a block needs, computed by the block itself from the (L2-resident) per-block
+// counts so that no separate scan launch sits between the count and move passes.
+__device__ __forceinline__ uint32_t block_sum_before(const uint32_t* counts, uint32_t n) {
+    __shared__ uint32_t part[kBlock / 64];
+    uint32_t s = 0;
+    for (uint32_t i = threadIdx.x; i < n; i += kBlock) s += counts[i];
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) s += (uint32_t)__shfl_xor((int)s, m, 64);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
+    __syncthreads();
+    uint32_t tot = 0;
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; w++) tot += part[w];
+    return tot;
+}
+
+template <class W, bool SET, bool PREFIXED>
+__global__ __launch_bounds__(kBlock) void compact_move_fast_kernel(const uint8_t* mask, W* full, W* out, uint32_t nvec, uint32_t nout,
+                                                                   const uint32_t* block_base) {
+    constexpr int VEC = 16 / (int)sizeof(W);
+    uint32_t flags[kFastJ];
+    Pack<W, VEC> data[kFastJ];
+    uint64_t packed = 0;
+#pragma unroll
+    for (int j = 0; j < kFastJ; j++) {
+        const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+        flags[j] = 0;
+        if (v < nvec) {
+            flags[j] = mask_flags<VEC>(mask + (size_t)v * VEC);
+            if constexpr (!SET) data[j] = load_pack<W, VEC>(full + (size_t)v * VEC);
+        }
+        packed |= (uint64_t)__popc(flags[j]) << (16 * j);
+    }
+    uint64_t total;
+    const uint64_t pre = block_exclusive_scan64(packed, &total);
+    uint32_t seg_base = PREFIXED ? block_base[blockIdx.x] : block_sum_before(block_base, blockIdx.x);
+#pragma unroll
+    for (int j = 0; j < kFastJ; j++) {
+        uint32_t k = seg_base + (uint32_t)((pre >> (16 * j)) & 0xFFFF);
+        seg_base += (uint32_t)((total >> (16 * j)) & 0xFFFF);
+        const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) {
+            if (flags[j] & (1u << e)) {
+                if (k < nout) {
+                    if constexpr (SET) full[(size_t)v * VEC + e] = out[k];
+                    else out[k] = data[j].v[e];
+                }
+                k++;
+            }
+        }
+    }
+}
+
+template <class W, bool SET>
+int32_t run_compaction_fast(const uint8_t* mask, void* full, void* out, int64_t n, int64_t nout64, hipStream_t stream) {
+    constexpr int VEC = 16 / (int)sizeof(W);
+    const uint32_t nvec = (uint32_t)(n / VEC);
+    const uint32_t nout = (uint32_t)(nout64 > (int64_t)kMaxItems ? kMaxItems : nout64);
+    const uint32_t nb = cdiv(nvec, kFastJ * kBlock);
+    uint32_t* counts;
+    DNH_TRY(workspace(stream, sizeof(uint32_t) * (size_t)nb, (void**)&counts));
+    hipLaunchKernelGGL(compact_count_fast_kernel<VEC>, dim3(nb), dim3(kBlock), 0, stream, mask, nvec, counts);
+    DNH_LAUNCH_CHECK();
+    if (nb <= 8192) {
+        // few blocks: each block sums the counts before it (at most 32 KB of L2 reads) instead of waiting for a scan launch
+        hipLaunchKernelGGL((compact_move_fast_kernel<W, SET, false>), dim3(nb), dim3(kBlock), 0, stream, mask, (W*)full, (W*)out, nvec, nout, counts);
+    } else {
+        hipLaunchKernelGGL(compact_scan_kernel, dim3(1), dim3(kBlock), 0, stream, counts, nb);
+        DNH_LAUNCH_CHECK();
+        hipLaunchKernelGGL((compact_move_fast_kernel<W, SET, true>), dim3(nb), dim3(kBlock), 0, stream, mask, (W*)full, (W*)out, nvec, nout, counts);
+    }
+    DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
+
+// The fast path applies to one unit-stride dimension whose length is a whole number of 16-byte vectors, 16-byte aligned data.
+template <bool SET>
+bool try_compaction_fast(const MaskArgs& m, void* full, void* out, const Lay& olay, int esize, int64_t n, int64_t nout, hipStream_t stream, int32_t* status) {
+    if (m.whole || m.full.nd != 1 || !m.mask[0] || m.mask_stride[0] != 1 || m.full.stride[0] != 1) return false;
+    if (olay.nd != 1 || olay.stride[0] != 1) return false;
+    if (n > (int64_t)kMaxItems || n == 0 || nout == 0) return false;
+    const int vec = 16 / esize;
+    if ((n % vec) != 0 || !aligned_to(full, 16) || !aligned_to(m.mask[0], vec)) return false;
+    switch (esize) {
+        case 1: *status = run_compaction_fast<uint8_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
+        case 4: *status = run_compaction_fast<uint32_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
+        case 8: *status = run_compaction_fast<uint64_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
+    }
+    return false;
+}
+
 template <int MODE>
 int32_t run_compaction(const MaskArgs& m, void* full, void* out, const Lay& olay, int esize, int64_t n64, int64_t nout64, hipStream_t stream) {
     if (n64 == 0 || nout64 == 0) return DNH_OK;
@@ -347,6 +491,8 @@ extern "C" int32_t dnh_masked_get(const DnhTensor* t, const DnhTensor* src, cons
     if (t->dtype != src->dtype) return fail(DNH_ERR_INVALID_ARG, "dnh_masked_get: dtypes differ");
     MaskArgs m;
     DNH_TRY(make_mask_args(&m, src, masks, n_masks, "dnh_masked_get"));
+    int32_t st = DNH_OK;
+    if (try_compaction_fast<false>(m, elem_ptr(src), elem_ptr(t), lay_of(t), dtype_size(t->dtype), nelems(src), nelems(t), (hipStream_t)stream, &st)) return st;
     return run_compaction<kMaskedGet>(m, elem_ptr(src), elem_ptr(t), lay_of(t), dtype_size(t->dtype), nelems(src), nelems(t), (hipStream_t)stream);
 }
 
@@ -357,6 +503,8 @@ extern "C" int32_t dnh_masked_set(const DnhTensor* t, const DnhTensor* const* ma
     if (t->dtype != src->dtype) return fail(DNH_ERR_INVALID_ARG, "dnh_masked_set: dtypes differ");
     MaskArgs m;
     DNH_TRY(make_mask_args(&m, t, masks, n_masks, "dnh_masked_set"));
+    int32_t st = DNH_OK;
+    if (try_compaction_fast<true>(m, elem_ptr(t), elem_ptr(src), lay_of(src), dtype_size(t->dtype), nelems(t), nelems(src), (hipStream_t)stream, &st)) return st;
     return run_compaction<kMaskedSet>(m, elem_ptr(t), elem_ptr(src), lay_of(src), dtype_size(t->dtype), nelems(t), nelems(src), (hipStream_t)stream);
 }
 

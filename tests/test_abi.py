@@ -1,0 +1,81 @@
+"""CPU: the C-ABI library loads, exports every symbol include/tensor_hip.h declares, its descriptor layout matches the header
+as compiled by gcc, and — with no GPU in the machine — the product path fails loudly instead of falling back."""
+import ctypes as C
+import os
+import re
+import subprocess
+import tempfile
+
+import numpy as np
+import pytest
+
+from deepnet_amd import abi, native
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "tensor_hip.h")
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    return sorted(set(re.findall(r"^int32_t\s+(dnh_\w+)\s*\(", text, flags=re.M)))
+
+
+def test_library_exports_every_declared_symbol():
+    lib = native.load()
+    names = declared_symbols()
+    assert len(names) >= 39
+    for n in names:
+        assert hasattr(lib, n), f"libtensor_hip.so lacks {n}"
+    assert sorted(abi.EXPORTED_SYMBOLS) == names, "deepnet_amd/abi.py and include/tensor_hip.h disagree"
+
+
+def test_descriptor_layout_matches_the_header():
+    src = r'''
+#include <stdio.h>
+#include <stddef.h>
+#include "tensor_hip.h"
+int main(void) {
+  printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(DnhTensor), offsetof(DnhTensor, base), offsetof(DnhTensor, offset),
+         offsetof(DnhTensor, ndims), offsetof(DnhTensor, dtype), offsetof(DnhTensor, shape), offsetof(DnhTensor, stride), sizeof(DnhDeviceInfo));
+  printf("%d %d %d %d %d %lld\n", DNH_F64, DNH_NEGATE, DNH_XOR, DNH_GREATER_OR_EQUAL, DNH_COUNT_TRUE, (long long)DNH_NOT_FOUND);
+  return 0; }'''
+    with tempfile.TemporaryDirectory() as d:
+        c = os.path.join(d, "t.c")
+        open(c, "w").write(src)
+        exe = os.path.join(d, "t")
+        subprocess.check_call(["gcc", "-std=c99", "-I", os.path.join(ROOT, "include"), c, "-o", exe])
+        out = subprocess.check_output([exe]).decode().split()
+    vals = [int(x) for x in out]
+    T = abi.DnhTensor
+    assert vals[:8] == [C.sizeof(T), T.base.offset, T.offset.offset, T.ndims.offset, T.dtype.offset, T.shape.offset, T.stride.offset,
+                        C.sizeof(abi.DnhDeviceInfo)]
+    assert vals[8:] == [abi.DNH_F64, abi.DNH_NEGATE, abi.DNH_XOR, abi.DNH_GREATER_OR_EQUAL, abi.DNH_COUNT_TRUE, abi.NOT_FOUND]
+
+
+def test_oracle_exports_the_same_operator_set():
+    from oracle import hostref
+    lib = hostref.load()
+    for name in abi.OP_SIGNATURES:
+        assert hasattr(lib, "href_" + name)
+
+
+def _have_gpu():
+    return os.path.exists("/dev/kfd") and os.access("/dev/kfd", os.R_OK | os.W_OK)
+
+
+@pytest.mark.skipif(_have_gpu(), reason="a GPU is present; this test pins the no-GPU failure mode")
+def test_product_path_fails_loudly_without_a_gpu():
+    from deepnet_amd import hip
+    with pytest.raises(native.HipError):
+        hip.ofNumpy(np.zeros(4, np.float32))
+    assert "HIP" in native.last_error() or "hip" in native.last_error()
+    # argument validation happens before any device work and reports through the same channel
+    lib = native.load()
+    assert lib.dnh_last_error(None, 0) == abi.DNH_ERR_INVALID_ARG
+
+
+def test_status_codes_map_to_reference_exception_kinds():
+    assert native._EXC[abi.DNH_ERR_INVALID_ARG] is ValueError
+    assert native._EXC[abi.DNH_ERR_NOT_SUPPORTED] is NotImplementedError
+    assert native._EXC[abi.DNH_ERR_INDEX_OUT_OF_RANGE] is IndexError
+    assert native._EXC[abi.DNH_ERR_OUT_OF_MEMORY] is MemoryError
