@@ -1,0 +1,264 @@
+namespace Tensor.Hip
+
+// TensorHipStorage / TensorHipBackend / TensorHipDevice: the HIP counterpart of Tensor/Tensor/Cuda/CudaBackend.fs behind the
+// unchanged plugin interfaces of Tensor/Tensor/TensorBackend.fs.  Every ITensorBackend member is one call into
+// libtensor_hip.so; nothing is computed on the managed side.  Source only (no .NET SDK on this repository's build machine).
+
+open System
+open System.Runtime.InteropServices
+open Tensor
+open Tensor.Utils
+open Tensor.Backend
+
+/// Thread-local options (mirror of Tensor.Cuda.Cfg, Cuda/CudaCfg.fs:14-60).
+module Cfg =
+    [<ThreadStatic; DefaultValue>]
+    val mutable private stream: nativeint
+    [<ThreadStatic; DefaultValue>]
+    val mutable private noIndexCheck: bool
+    /// hipStream_t all operations of this thread are issued on (IntPtr.Zero = default stream)
+    let Stream with get () = stream and set v = stream <- v
+    /// read the device index-error flag after every Gather/Scatter so a bad index raises at the faulting call (default true)
+    let Stacktrace with get () = not noIndexCheck and set v = noIndexCheck <- not v
+
+module internal Desc =
+    let dtypeOf (t: Type) =
+        if   t = typeof<bool>   then DType.Bool elif t = typeof<byte>   then DType.U8  elif t = typeof<sbyte>  then DType.I8
+        elif t = typeof<int32>  then DType.I32  elif t = typeof<uint32> then DType.U32 elif t = typeof<int64>  then DType.I64
+        elif t = typeof<uint64> then DType.U64  elif t = typeof<single> then DType.F32 elif t = typeof<double> then DType.F64
+        else raise (NotSupportedException (sprintf "element type %s is not supported by the HIP backend" t.Name))
+
+    let make (basePtr: nativeint) (dataType: Type) (layout: TensorLayout) =
+        if layout.NDims > 8 then raise (NotSupportedException "the HIP backend supports at most 8 dimensions")
+        let mutable d = DnhTensor()
+        d.Base <- basePtr
+        d.Offset <- layout.Offset
+        d.NDims <- layout.NDims
+        d.DType <- int (dtypeOf dataType)
+        d.Shape <- Array.zeroCreate 8
+        d.Stride <- Array.zeroCreate 8
+        layout.Shape |> List.iteri (fun i s -> d.Shape.[i] <- s)
+        layout.Stride |> List.iteri (fun i s -> d.Stride.[i] <- s)
+        d
+
+/// Device memory owned by one tensor storage (CudaBackend.fs:54-93).
+type TensorHipStorage<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> ValueType> (nElems: int64) =
+    let bytes = unativeint (max nElems 1L) * unativeint sizeof<'T>
+    let mutable ptr = IntPtr.Zero
+    do Native.check (Native.dnh_alloc (bytes, &ptr))
+
+    member this.Ptr = ptr
+    member this.NElems = nElems
+    override this.Finalize () = if ptr <> IntPtr.Zero then Native.dnh_free ptr |> ignore
+
+    interface ITensorStorage<'T> with
+        member this.Backend layout = TensorHipBackend<'T> (layout, this) :> ITensorBackend<_>
+        member this.Dev = TensorHipDevice.Instance :> ITensorDevice
+
+and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> ValueType>
+        (layout: TensorLayout, storage: TensorHipStorage<'T>) =
+
+    static let desc (t: ITensorFrontend<'A>) =
+        let st = t.Storage :?> TensorHipStorage<'A>
+        Desc.make st.Ptr typeof<'A> t.Layout
+
+    static let unary op (trgt: ITensorFrontend<'R>) (a: ITensorFrontend<'A>) =
+        let mutable t, a = desc trgt, desc a
+        Native.check (Native.dnh_unary (op, &t, &a, Cfg.Stream))
+    static let binary op (trgt: ITensorFrontend<'R>) (a: ITensorFrontend<'A>) (b: ITensorFrontend<'A>) =
+        let mutable t, a, b = desc trgt, desc a, desc b
+        Native.check (Native.dnh_binary (op, &t, &a, &b, Cfg.Stream))
+    static let compare op (trgt: ITensorFrontend<bool>) (a: ITensorFrontend<'A>) (b: ITensorFrontend<'A>) =
+        let mutable t, a, b = desc trgt, desc a, desc b
+        Native.check (Native.dnh_compare (op, &t, &a, &b, Cfg.Stream))
+    static let reduce op (trgt: ITensorFrontend<'R>) (src: ITensorFrontend<'A>) =
+        let mutable t, s = desc trgt, desc src
+        Native.check (Native.dnh_reduce_last_axis (op, &t, &s, Cfg.Stream))
+    static let argReduce op (trgt: ITensorFrontend<int64>) (src: ITensorFrontend<'A>) =
+        let mutable t, s = desc trgt, desc src
+        Native.check (Native.dnh_arg_reduce_last_axis (op, &t, &s, Cfg.Stream))
+    static let dot (trgt: ITensorFrontend<'T>) (a: ITensorFrontend<'T>) (b: ITensorFrontend<'T>) =
+        let mutable t, a, b = desc trgt, desc a, desc b
+        Native.check (Native.dnh_dot (&t, &a, &b, Cfg.Stream))
+
+    /// pins optional descriptors and calls f with the array of their addresses (IntPtr.Zero for None)
+    static let withDescs (ts: ITensorFrontend<'A> option list) (f: nativeint[] -> unit) =
+        let descs = ts |> List.map (Option.map desc)
+        let handles = descs |> List.map (Option.map (fun d -> GCHandle.Alloc (box d, GCHandleType.Pinned)))
+        try f (handles |> List.map (function Some h -> h.AddrOfPinnedObject () | None -> IntPtr.Zero) |> Array.ofList)
+        finally handles |> List.iter (Option.iter (fun h -> h.Free ()))
+
+    static let checkIndexError () =
+        if Cfg.Stacktrace then
+            let mutable code = 0
+            Native.check (Native.dnh_async_error (Cfg.Stream, &code))
+            Native.check code
+
+    let itemAddr (idx: int64[]) = storage.Ptr + nativeint (TensorLayout.addr (List.ofArray idx) layout) * nativeint sizeof<'T>
+
+    interface ITensorBackend<'T> with
+        member this.Item
+            with get idx =                                              // CudaBackend.fs:77-87: synchronous 1-element copy
+                let v = [| Unchecked.defaultof<'T> |]
+                let h = GCHandle.Alloc (v, GCHandleType.Pinned)
+                try Native.check (Native.dnh_memcpy_d2h (h.AddrOfPinnedObject (), itemAddr idx, unativeint sizeof<'T>, Cfg.Stream, 1))
+                finally h.Free ()
+                v.[0]
+            and set idx value =
+                let v = [| value |]
+                let h = GCHandle.Alloc (v, GCHandleType.Pinned)
+                try Native.check (Native.dnh_memcpy_h2d (itemAddr idx, h.AddrOfPinnedObject (), unativeint sizeof<'T>, Cfg.Stream, 1))
+                finally h.Free ()
+
+        member this.Copy (trgt, src) =
+            let mutable t, s = desc trgt, desc src
+            Native.check (Native.dnh_copy (&t, &s, Cfg.Stream))
+        member this.Convert (trgt: ITensorFrontend<'T>, src: ITensorFrontend<'S>) =
+            let mutable t, s = desc trgt, desc src
+            Native.check (Native.dnh_convert (&t, &s, Cfg.Stream))
+        member this.Transfer (trgt, src) = HipTransfer.transfer (trgt, src)   // host <-> device, as CudaBackend.fs:206-270
+        member this.FillConst (value, trgt) =
+            let mutable t = desc trgt
+            let h = GCHandle.Alloc ([| value |], GCHandleType.Pinned)
+            try Native.check (Native.dnh_fill_const (&t, h.AddrOfPinnedObject (), Cfg.Stream)) finally h.Free ()
+        member this.FillIncrementing (start, incr, trgt) =
+            let mutable t = desc trgt
+            let h = GCHandle.Alloc ([| start; incr |], GCHandleType.Pinned)
+            try
+                let p = h.AddrOfPinnedObject ()
+                Native.check (Native.dnh_fill_incrementing (&t, p, p + nativeint sizeof<'T>, Cfg.Stream))
+            finally h.Free ()
+
+        member this.UnaryPlus (t, a) = unary 0 t a
+        member this.UnaryMinus (t, a) = unary 1 t a
+        member this.Abs (t, a) = unary 2 t a
+        member this.Sgn (t, a) = unary 3 t a
+        member this.Log (t, a) = unary 4 t a
+        member this.Log10 (t, a) = unary 5 t a
+        member this.Exp (t, a) = unary 6 t a
+        member this.Sin (t, a) = unary 7 t a
+        member this.Cos (t, a) = unary 8 t a
+        member this.Tan (t, a) = unary 9 t a
+        member this.Asin (t, a) = unary 10 t a
+        member this.Acos (t, a) = unary 11 t a
+        member this.Atan (t, a) = unary 12 t a
+        member this.Sinh (t, a) = unary 13 t a
+        member this.Cosh (t, a) = unary 14 t a
+        member this.Tanh (t, a) = unary 15 t a
+        member this.Sqrt (t, a) = unary 16 t a
+        member this.Ceiling (t, a) = unary 17 t a
+        member this.Floor (t, a) = unary 18 t a
+        member this.Round (t, a) = unary 19 t a
+        member this.Truncate (t, a) = unary 20 t a
+        member this.Negate (t, a) = unary 21 t a
+        member this.IsFinite (trgt, a) =
+            let mutable t, a = desc trgt, desc a
+            Native.check (Native.dnh_is_finite (&t, &a, Cfg.Stream))
+
+        member this.Add (t, a, b) = binary 0 t a b
+        member this.Subtract (t, a, b) = binary 1 t a b
+        member this.Multiply (t, a, b) = binary 2 t a b
+        member this.Divide (t, a, b) = binary 3 t a b
+        member this.Modulo (t, a, b) = binary 4 t a b
+        member this.Power (t, a, b) = binary 5 t a b
+        member this.MaxElemwise (t, a, b) = binary 6 t a b
+        member this.MinElemwise (t, a, b) = binary 7 t a b
+        member this.And (t, a, b) = binary 8 t a b
+        member this.Or (t, a, b) = binary 9 t a b
+        member this.Xor (t, a, b) = binary 10 t a b
+
+        member this.Equal (t, a, b) = compare 0 t a b
+        member this.NotEqual (t, a, b) = compare 1 t a b
+        member this.Less (t, a, b) = compare 2 t a b
+        member this.LessOrEqual (t, a, b) = compare 3 t a b
+        member this.Greater (t, a, b) = compare 4 t a b
+        member this.GreaterOrEqual (t, a, b) = compare 5 t a b
+
+        member this.IfThenElse (trgt, cond, ifTrue, ifFalse) =
+            let mutable t, c, a, b = desc trgt, desc cond, desc ifTrue, desc ifFalse
+            Native.check (Native.dnh_if_then_else (&t, &c, &a, &b, Cfg.Stream))
+
+        member this.Gather (trgt, srcIdxs, src) =
+            let mutable t, s = desc trgt, desc src
+            withDescs srcIdxs (fun p -> Native.check (Native.dnh_gather (&t, p, p.Length, &s, Cfg.Stream)))
+            checkIndexError ()
+        member this.Scatter (trgt, trgtIdxs, src) =
+            let mutable t, s = desc trgt, desc src
+            withDescs trgtIdxs (fun p -> Native.check (Native.dnh_scatter (&t, p, p.Length, &s, Cfg.Stream)))
+            checkIndexError ()
+        member this.MaskedGet (trgt, src, masks) =
+            let mutable t, s = desc trgt, desc src
+            withDescs (List.ofArray masks) (fun p -> Native.check (Native.dnh_masked_get (&t, &s, p, p.Length, Cfg.Stream)))
+        member this.MaskedSet (trgt, masks, src) =
+            let mutable t, s = desc trgt, desc src
+            withDescs (List.ofArray masks) (fun p -> Native.check (Native.dnh_masked_set (&t, p, p.Length, &s, Cfg.Stream)))
+        member this.TrueIndices (trgt, src) =
+            let mutable t, s = desc trgt, desc src
+            Native.check (Native.dnh_true_indices (&t, &s, Cfg.Stream))
+
+        member this.SumLastAxis (t, s) = reduce 0 t s
+        member this.ProductLastAxis (t, s) = reduce 1 t s
+        member this.MinLastAxis (t, s) = reduce 2 t s
+        member this.MaxLastAxis (t, s) = reduce 3 t s
+        member this.AllLastAxis (t, s) = reduce 4 t s
+        member this.AnyLastAxis (t, s) = reduce 5 t s
+        member this.CountTrueLastAxis (t, s) = reduce 6 t s
+        member this.ArgMinLastAxis (t, s) = argReduce 0 t s
+        member this.ArgMaxLastAxis (t, s) = argReduce 1 t s
+        member this.FindLastAxis (value, trgt, src) =
+            let mutable t, s = desc trgt, desc src
+            let h = GCHandle.Alloc ([| value |], GCHandleType.Pinned)
+            try Native.check (Native.dnh_find_last_axis (h.AddrOfPinnedObject (), &t, &s, Cfg.Stream)) finally h.Free ()
+
+        member this.VecVecDot (t, a, b) = dot t a b
+        member this.MatVecDot (t, a, b) = dot t a b
+        member this.MatMatDot (t, a, b) = dot t a b
+        member this.BatchedMatMatDot (t, a, b) = dot t a b
+
+        // not on the accelerated path; the CUDA backend leaves SVD and the eigen-decomposition unsupported too (CudaBackend.fs:486-492)
+        member this.BatchedInvert (trgt, src) = raise (NotSupportedException "BatchedInvert is not supported by the HIP backend")
+        member this.BatchedSVD (trgtS, trgtUV, src) = raise (NotSupportedException "BatchedSVD is not supported by the HIP backend")
+        member this.SymmetricEigenDecomposition (part, eigVals, eigVecs, src) =
+            raise (NotSupportedException "SymmetricEigenDecomposition is not supported by the HIP backend")
+
+/// Host <-> device copies: the source is made row-major first, a non-row-major target goes through a device temporary
+/// (CudaBackend.fs:206-270).  Returns false for pairs this backend does not handle so the frontend can try the other side
+/// (Tensor.fs:704-711).
+and internal HipTransfer =
+    static member transfer (trgt: ITensorFrontend<'T>, src: ITensorFrontend<'T>) : bool =
+        match box trgt.Storage, box src.Storage with
+        | (:? TensorHipStorage<'T> as ts), (:? Tensor.Host.TensorHostStorage<'T> as hs) ->
+            let src = if TensorLayout.isC src.Layout then src else src.Copy (order=RowMajor)
+            let hs = src.Storage :?> Tensor.Host.TensorHostStorage<'T>
+            use pin = hs.Pin ()
+            let bytes = unativeint (src.NElems * int64 sizeof<'T>)
+            let hostPtr = pin.Ptr + nativeint (src.Layout.Offset * int64 sizeof<'T>)
+            if TensorLayout.isC trgt.Layout then
+                let dst = ts.Ptr + nativeint (trgt.Layout.Offset * int64 sizeof<'T>)
+                Native.check (Native.dnh_memcpy_h2d (dst, hostPtr, bytes, Cfg.Stream, 1))
+            else
+                let tmp = trgt.Copy (order=RowMajor)
+                let tmpSt = tmp.Storage :?> TensorHipStorage<'T>
+                Native.check (Native.dnh_memcpy_h2d (tmpSt.Ptr, hostPtr, bytes, Cfg.Stream, 1))
+                trgt.CopyFrom tmp
+            true
+        | (:? Tensor.Host.TensorHostStorage<'T> as hs), (:? TensorHipStorage<'T>) ->
+            let src = if TensorLayout.isC src.Layout then src else src.Copy (order=RowMajor)
+            let ss = src.Storage :?> TensorHipStorage<'T>
+            let tmpHost = if TensorLayout.isC trgt.Layout then trgt else trgt.Copy (order=RowMajor)
+            let ths = tmpHost.Storage :?> Tensor.Host.TensorHostStorage<'T>
+            use pin = ths.Pin ()
+            let bytes = unativeint (src.NElems * int64 sizeof<'T>)
+            let srcPtr = ss.Ptr + nativeint (src.Layout.Offset * int64 sizeof<'T>)
+            Native.check (Native.dnh_memcpy_d2h (pin.Ptr + nativeint (tmpHost.Layout.Offset * int64 sizeof<'T>), srcPtr, bytes, Cfg.Stream, 1))
+            if not (obj.ReferenceEquals (tmpHost, trgt)) then trgt.CopyFrom tmpHost
+            true
+        | _ -> false
+
+/// The device (CudaBackend.fs:497-507): new storage is uninitialised, so Zeroed = false and `zeros` launches FillConst.
+and TensorHipDevice private () =
+    inherit BaseTensorDevice ()
+    static member Instance = TensorHipDevice ()
+    override this.Id = "Hip"
+    override this.Create nElems = TensorHipStorage<'T> nElems :> ITensorStorage<'T>
+    override this.Zeroed = false

@@ -1,0 +1,80 @@
+namespace Tensor.Hip
+
+// P/Invoke surface of libtensor_hip.so (include/tensor_hip.h).  Source only: this repository's build machine has no
+// .NET SDK, so these files are compiled where Deep.Net is (add them to Tensor/Tensor/Tensor.fsproj after the Cuda/ group
+// and ship libtensor_hip.so under runtimes/linux-x64/native, the location Tensor/Tensor/NativeLib.fs:146-161 probes).
+
+open System
+open System.Runtime.InteropServices
+
+/// DnhStatus
+type internal Status =
+    | OK = 0
+    | InvalidArg = 1
+    | NotSupported = 2
+    | OutOfMemory = 3
+    | Hip = 4
+    | IndexOutOfRange = 5
+    | NotInitialized = 6
+
+/// DnhDType — the element types the reference marshals to kernels (Cuda/NativeTensor.fs:22-34).
+type internal DType =
+    | Bool = 0 | U8 = 1 | I8 = 2 | I32 = 3 | U32 = 4 | I64 = 5 | U64 = 6 | F32 = 7 | F64 = 8
+
+/// DnhTensor: blittable descriptor passed by reference (replaces the Reflection.Emit structs of Cuda/NativeTensor.fs:96-208).
+[<Struct; StructLayout(LayoutKind.Sequential)>]
+type internal DnhTensor =
+    val mutable Base:   nativeint
+    val mutable Offset: int64
+    val mutable NDims:  int32
+    val mutable DType:  int32
+    [<MarshalAs(UnmanagedType.ByValArray, SizeConst=8)>]
+    val mutable Shape:  int64[]
+    [<MarshalAs(UnmanagedType.ByValArray, SizeConst=8)>]
+    val mutable Stride: int64[]
+
+module internal Native =
+    [<Literal>]
+    let Lib = "tensor_hip"
+    let private cc = CallingConvention.Cdecl
+
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_init (int device)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_last_error (byte[] buf, unativeint n)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_async_error (nativeint stream, int& code)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_alloc (unativeint bytes, nativeint& ptr)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_free (nativeint ptr)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_memcpy_h2d (nativeint dst, nativeint src, unativeint bytes, nativeint stream, int sync)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_memcpy_d2h (nativeint dst, nativeint src, unativeint bytes, nativeint stream, int sync)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_stream_sync (nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_fill_const (DnhTensor& t, nativeint value, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_fill_incrementing (DnhTensor& t, nativeint start, nativeint incr, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_copy (DnhTensor& t, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_convert (DnhTensor& t, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_unary (int op, DnhTensor& t, DnhTensor& a, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_is_finite (DnhTensor& t, DnhTensor& a, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_binary (int op, DnhTensor& t, DnhTensor& a, DnhTensor& b, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_compare (int op, DnhTensor& t, DnhTensor& a, DnhTensor& b, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_if_then_else (DnhTensor& t, DnhTensor& c, DnhTensor& a, DnhTensor& b, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_reduce_last_axis (int op, DnhTensor& t, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_arg_reduce_last_axis (int op, DnhTensor& t, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_find_last_axis (nativeint value, DnhTensor& t, DnhTensor& src, nativeint stream)
+    // index tensors and masks: arrays of pointers to pinned descriptors, IntPtr.Zero where the reference passes None
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_gather (DnhTensor& t, nativeint[] idx, int nIdx, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_scatter (DnhTensor& t, nativeint[] idx, int nIdx, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_masked_get (DnhTensor& t, DnhTensor& src, nativeint[] masks, int nMasks, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_masked_set (DnhTensor& t, nativeint[] masks, int nMasks, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_true_indices (DnhTensor& t, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_dot (DnhTensor& t, DnhTensor& a, DnhTensor& b, nativeint stream)
+
+    /// Maps a status to the exception type the reference's backends raise for the same condition.
+    let check (status: int) =
+        if status <> 0 then
+            let buf = Array.zeroCreate<byte> 1024
+            dnh_last_error (buf, unativeint buf.Length) |> ignore
+            let msg = System.Text.Encoding.UTF8.GetString(buf).TrimEnd('\000')
+            match enum<Status> status with
+            | Status.InvalidArg -> raise (InvalidOperationException msg)
+            | Status.NotSupported -> raise (NotSupportedException msg)
+            | Status.OutOfMemory -> raise (OutOfMemoryException msg)
+            | Status.IndexOutOfRange -> raise (IndexOutOfRangeException msg)
+            | _ -> failwithf "HIP tensor backend error %d: %s" status msg
