@@ -57,7 +57,7 @@ def report(log, cfg, name, ms, nbytes=None, flops=None):
     return {"cfg": cfg, "op": name, "ms": ms, "GBps": gb, "frac": gb / HBM_PEAK_GBS}
 
 
-def run_all(log, which=(1, 2, 3, 4, 5)):
+def run_all(log, which=(1, 2, 3, 4, 5, 6)):
     from deepnet_amd import abi, hip as G
     from deepnet_amd.backend import CAbiTensorBackend
     from deepnet_amd.tensor import Tensor
@@ -222,10 +222,24 @@ def run_all(log, which=(1, 2, 3, 4, 5)):
             sm.Backend.SumLastAxis(sm, a)
             return [("binary", (abi.DNH_DIVIDE, D(c), D(a), D(sm[:, :, None].broadcastTo([Bn, n, n]))))]
         timed(5, "Divide e / rowsum (broadcast)", 2 * N * 4 + R * 4, div5)
+    if 6 in which:
+        # the vector forms of dot (not one of the five configurations; bandwidth-bound)
+        n = 8192
+        for dt, sz in ((np.float32, 4), (np.float64, 8)):
+            nm = np.dtype(dt).name
+            mats = [G.ofNumpy(rng.standard_normal((n, n)).astype(dt)) for _ in range(3)]
+            x = G.ofNumpy(rng.standard_normal(n).astype(dt))
+            y = new([n], dt)
+            timed(6, f"MatVecDot 8192x8192 {nm}", n * n * sz + 2 * n * sz, lambda i: [("dot", (D(y), D(mats[i % 3]), D(x)))])
+            timed(6, f"MatVecDot transposed view {nm}", n * n * sz + 2 * n * sz, lambda i: [("dot", (D(y), D(mats[i % 3].T), D(x)))])
+            u, v = (G.ofNumpy(rng.standard_normal(1 << 26).astype(dt)) for _ in range(2))
+            r = new([], dt)
+            timed(6, f"VecVecDot 64Mi {nm}", 2 * (1 << 26) * sz, lambda i: [("dot", (D(r), D(u), D(v)))])
+            del mats, u, v
     return results
 
 
 if __name__ == "__main__":
     import sys
-    which = tuple(int(x) for x in sys.argv[1:]) or (1, 2, 3, 4, 5)
+    which = tuple(int(x) for x in sys.argv[1:]) or (1, 2, 3, 4, 5, 6)
     run_all(lambda *a: print(*a, flush=True), which)

@@ -247,6 +247,171 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
     return DNH_OK;
 }
 
+// ---- vector forms -------------------------------------------------------------------------------------------------------------
+// VecVecDot and MatVecDot are bandwidth-bound reductions, not tile problems: y[m] = sum_k A[m,k] * x[k].
+//   gemv_rows : A's k dimension has stride 1 — TPR threads share a row, 16-byte loads of A and x, shuffle tree; a long K with few
+//               rows (the vector-vector case is M = 1) is split over gridDim.y into partials.
+//   gemv_cols : A's m dimension has stride 1 (a transposed view) — one lane per m, coalesced along m, K split over gridDim.y.
+// Partials are summed by gemv_finish in index order (deterministic, no float atomics).
+
+template <class T, int VEC, int TPR>
+__global__ __launch_bounds__(kBlock) void gemv_rows_kernel(T* y, T* partial, const T* a, const T* x, uint32_t M, int64_t K, int64_t sam,
+                                                           int64_t sak, int64_t sxk, int64_t sym, int64_t chunk, uint32_t splits) {
+    constexpr int RPB = kBlock / TPR;
+    const uint32_t m = blockIdx.x * RPB + threadIdx.x / TPR;
+    const uint32_t lane = threadIdx.x % TPR;
+    const int64_t k0 = (int64_t)blockIdx.y * chunk;
+    const int64_t k1 = (k0 + chunk < K) ? k0 + chunk : K;
+    T acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) acc[e] = T(0);
+    if (m < M) {
+        const T* row = a + (int64_t)m * sam;
+        if constexpr (VEC > 1) {
+            int64_t k = k0 + (int64_t)lane * VEC;
+            for (; k + VEC <= k1; k += (int64_t)TPR * VEC) {
+                const Pack<T, VEC> va = load_pack<T, VEC>(row + k);
+                const Pack<T, VEC> vx = *(const Pack<T, VEC>*)(x + k);
+#pragma unroll
+                for (int e = 0; e < VEC; e++) acc[e] += va.v[e] * vx.v[e];
+            }
+            const int64_t t0 = k0 + ((k1 - k0) / VEC) * VEC + lane;
+            if (t0 < k1) acc[0] += row[t0] * x[t0];
+        } else {
+            for (int64_t k = k0 + lane; k < k1; k += TPR) acc[0] += row[k * sak] * x[k * sxk];
+        }
+    }
+    T s = acc[0];
+#pragma unroll
+    for (int e = 1; e < VEC; e++) s += acc[e];
+#pragma unroll
+    for (int w = (TPR < 64 ? TPR : 64) / 2; w >= 1; w >>= 1) s += __shfl_xor(s, w, 64);
+    if constexpr (TPR > 64) {
+        __shared__ T sh[TPR / 64];
+        if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = s;
+        __syncthreads();
+        if (threadIdx.x == 0)
+#pragma unroll
+            for (int w = 1; w < TPR / 64; w++) s += sh[w];
+    }
+    if (m < M && lane == 0) {
+        if (splits == 1) y[(int64_t)m * sym] = s;
+        else partial[(int64_t)m * splits + blockIdx.y] = s;
+    }
+}
+
+template <class T, int VEC>
+__global__ __launch_bounds__(kBlock) void gemv_cols_kernel(T* y, T* partial, const T* a, const T* x, uint32_t M, int64_t K, int64_t sak,
+                                                           int64_t sxk, int64_t sym, int64_t chunk, uint32_t splits) {
+    const uint32_t m = (blockIdx.x * kBlock + threadIdx.x) * VEC;
+    if (m >= M) return;
+    const int64_t k0 = (int64_t)blockIdx.y * chunk;
+    const int64_t k1 = (k0 + chunk < K) ? k0 + chunk : K;
+    T acc[VEC];
+#pragma unroll
+    for (int e = 0; e < VEC; e++) acc[e] = T(0);
+    const T* p = a + m;
+    int64_t k = k0;
+    for (; k + 1 < k1; k += 2) {
+        const Pack<T, VEC> v0 = load_pack<T, VEC>(p + k * sak);
+        const Pack<T, VEC> v1 = load_pack<T, VEC>(p + (k + 1) * sak);
+        const T x0 = x[k * sxk], x1 = x[(k + 1) * sxk];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] += v0.v[e] * x0;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] += v1.v[e] * x1;
+    }
+    if (k < k1) {
+        const Pack<T, VEC> v0 = load_pack<T, VEC>(p + k * sak);
+        const T x0 = x[k * sxk];
+#pragma unroll
+        for (int e = 0; e < VEC; e++) acc[e] += v0.v[e] * x0;
+    }
+#pragma unroll
+    for (int e = 0; e < VEC; e++) {
+        if (splits == 1) y[(int64_t)(m + e) * sym] = acc[e];
+        else partial[(int64_t)(m + e) * splits + blockIdx.y] = acc[e];
+    }
+}
+
+template <class T>
+__global__ __launch_bounds__(kBlock) void gemv_finish_kernel(T* y, const T* partial, uint32_t M, uint32_t splits, int64_t sym) {
+    const uint32_t m = blockIdx.x;
+    T s = T(0);
+    for (uint32_t i = threadIdx.x; i < splits; i += kBlock) s += partial[(int64_t)m * splits + i];
+#pragma unroll
+    for (int w = 32; w >= 1; w >>= 1) s += __shfl_xor(s, w, 64);
+    __shared__ T sh[kBlock / 64];
+    if ((threadIdx.x & 63) == 0) sh[threadIdx.x >> 6] = s;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < kBlock / 64; w++) s += sh[w];
+        y[(int64_t)m * sym] = s;
+    }
+}
+
+// Returns false when neither vector kernel fits the strides (the tile kernel then handles the call).
+template <class T>
+bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t stream, int32_t* status) {
+    if (g.N != 1 || g.nbatch != 0 || g.M > (int64_t)kMaxItems) return false;
+    *status = DNH_OK;
+    if (g.K == 0) return false;
+    const uint32_t M = (uint32_t)g.M;
+    const int cus = device_cus();
+    constexpr int V = 16 / (int)sizeof(T);
+    T* partial = nullptr;
+    if (g.sak == 1 || g.M == 1) {
+        const bool vec = g.sak == 1 && g.sbk == 1 && (g.sam % V) == 0 && aligned_to(a, 16) && aligned_to(x, 16);
+        const int v = vec ? V : 1;
+        const int tpr = g.K >= (int64_t)256 * v * 2 ? 256 : (g.K >= (int64_t)64 * v ? 64 : 16);
+        const int64_t row_blocks = (M + kBlock / tpr - 1) / (kBlock / tpr);
+        uint32_t splits = 1;
+        int64_t chunk = g.K;
+        if (tpr == 256 && row_blocks < (int64_t)cus * 4) {
+            const int64_t min_chunk = (int64_t)256 * v * 8;
+            int64_t sp = ((int64_t)cus * 8 + row_blocks - 1) / row_blocks;
+            const int64_t maxs = (g.K + min_chunk - 1) / min_chunk;
+            if (sp > maxs) sp = maxs;
+            if (sp > 1) {
+                chunk = (g.K + sp - 1) / sp;
+                chunk = ((chunk + 256 * v - 1) / (256 * v)) * (256 * v);
+                splits = (uint32_t)((g.K + chunk - 1) / chunk);
+            }
+        }
+        if (splits > 1 && (*status = workspace(stream, sizeof(T) * (size_t)M * splits, (void**)&partial)) != DNH_OK) return true;
+        const dim3 grid((unsigned)row_blocks, splits);
+#define DNH_GEMV(VV, TPR) hipLaunchKernelGGL((gemv_rows_kernel<T, VV, TPR>), grid, dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sam, g.sak, g.sbk, g.scm, chunk, splits)
+        if (vec) { if (tpr == 256) DNH_GEMV(V, 256); else if (tpr == 64) DNH_GEMV(V, 64); else DNH_GEMV(V, 16); }
+        else { if (tpr == 256) DNH_GEMV(1, 256); else if (tpr == 64) DNH_GEMV(1, 64); else DNH_GEMV(1, 16); }
+#undef DNH_GEMV
+        if (splits > 1) hipLaunchKernelGGL(gemv_finish_kernel<T>, dim3(M), dim3(kBlock), 0, stream, y, (const T*)partial, M, splits, g.scm);
+    } else if (g.sam == 1) {
+        const bool vec = (M % V) == 0 && (g.sak % V) == 0 && aligned_to(a, 16);
+        const int v = vec ? V : 1;
+        const int64_t mblocks = (M / v + kBlock - 1) / kBlock;
+        uint32_t splits = 1;
+        int64_t chunk = g.K;
+        if (mblocks < (int64_t)cus * 4) {
+            int64_t sp = ((int64_t)cus * 4 + mblocks - 1) / mblocks;
+            const int64_t maxs = (g.K + 63) / 64;
+            if (sp > maxs) sp = maxs;
+            if (sp > 1) {
+                chunk = (g.K + sp - 1) / sp;
+                splits = (uint32_t)((g.K + chunk - 1) / chunk);
+            }
+        }
+        if (splits > 65535) return false;
+        if (splits > 1 && (*status = workspace(stream, sizeof(T) * (size_t)M * splits, (void**)&partial)) != DNH_OK) return true;
+        if (vec) hipLaunchKernelGGL((gemv_cols_kernel<T, V>), dim3((unsigned)mblocks, splits), dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sak, g.sbk, g.scm, chunk, splits);
+        else hipLaunchKernelGGL((gemv_cols_kernel<T, 1>), dim3((unsigned)mblocks, splits), dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sak, g.sbk, g.scm, chunk, splits);
+        if (splits > 1) hipLaunchKernelGGL(gemv_finish_kernel<T>, dim3(M), dim3(kBlock), 0, stream, y, (const T*)partial, M, splits, g.scm);
+    } else {
+        return false;
+    }
+    if (hipGetLastError() != hipSuccess) *status = fail(DNH_ERR_HIP, "gemv launch failed");
+    return true;
+}
+
 }  // namespace
 
 extern "C" int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream) {
@@ -294,6 +459,9 @@ extern "C" int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTens
     g.tiles_m = cdiv(g.M, BM);
     g.tiles_n = cdiv(g.N, BN);
     hipStream_t s = (hipStream_t)stream;
+    int32_t st = DNH_OK;
+    if (t->dtype == DNH_F32 && try_gemv<float>(g, (float*)elem_ptr(t), (const float*)elem_ptr(a), (const float*)elem_ptr(b), s, &st)) return st;
+    if (t->dtype == DNH_F64 && try_gemv<double>(g, (double*)elem_ptr(t), (const double*)elem_ptr(a), (const double*)elem_ptr(b), s, &st)) return st;
     if (t->dtype == DNH_F32) return launch_gemm<float>(g, (float*)elem_ptr(t), (const float*)elem_ptr(a), (const float*)elem_ptr(b), batch, s);
     return launch_gemm<double>(g, (double*)elem_ptr(t), (const double*)elem_ptr(a), (const double*)elem_ptr(b), batch, s);
 }

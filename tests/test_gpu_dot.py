@@ -103,3 +103,37 @@ def test_non_float_dot_not_supported(G):
     a = G.ofNumpy(np.ones((4, 4), np.int32))
     with pytest.raises(NotImplementedError):
         a @ a
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_vector_forms_layouts_and_sizes(H, G, rng, dt):
+    """MatVecDot / VecVecDot on the dedicated reduction kernels: row-major and transposed matrices, strided and offset vectors,
+    ragged and long K (split over several blocks)."""
+    for m, k in [(1, 1), (3, 5), (257, 1030), (2000, 64), (5, 70001), (4096, 4099)]:
+        a = rng.standard_normal((m, k)).astype(dt)
+        x = rng.standard_normal(k).astype(dt)
+        ref, got = both(H, G, lambda a, x: a @ x, a, x)
+        check_dot(ref, got, a, x)
+        # transposed view of a k-by-m matrix (m has stride 1)
+        at = np.ascontiguousarray(a.T)
+        ref, got = both(H, G, lambda at, x: at.T @ x, at, x)
+        check_dot(ref, got, a, x)
+    a = rng.standard_normal((300, 200)).astype(dt)
+    x2 = rng.standard_normal((200, 3)).astype(dt)
+    ref, got = both(H, G, lambda a, x: a[10:290, 5:195] @ x[5:195, 1], a, x2)        # offsets and a strided vector
+    check_dot(ref, got, a[10:290, 5:195], x2[5:195, 1])
+    u = rng.standard_normal(1_000_003).astype(dt)
+    v = rng.standard_normal(1_000_003).astype(dt)
+    ref, got = both(H, G, lambda u, v: u @ v, u, v)
+    check_dot(ref.reshape(1), got.reshape(1), u[None, :], v)
+    ref, got = both(H, G, lambda u, v: u[::1][3:100000] @ v.reverseAxis(0)[3:100000], u, v)
+    check_dot(ref.reshape(1), got.reshape(1), u[None, 3:100000], v[::-1][3:100000])
+    # a target with a stride (a column of a matrix)
+    def f(a, x):
+        t = type(a).new([300, 4], a.Dev, a.DataType)
+        t.FillConst(0)
+        t[:, 2].FillDot(a, x)
+        return t
+    ref, got = both(H, G, f, a, x2[:, 0].copy())
+    check_dot(ref[:, 2], got[:, 2], a, x2[:, 0])
+    assert (got[:, [0, 1, 3]] == 0).all()
