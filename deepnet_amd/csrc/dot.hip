@@ -4,15 +4,15 @@
 // One strided-batched GEMM kernel, C[b] = A[b] * B[b] (alpha 1, beta 0), written for gfx950:
 //   - 128x128 block tile, K step 16, 256 threads = 4 wavefronts in a 2x2 arrangement, each owning a 64x64 sub-tile;
 //   - fp32: four 32x32 accumulators per wavefront on v_mfma_f32_32x32x2_f32 (A and B operands one dword per lane);
-//     fp64: an 8x8 register micro-tile per thread on vector FMA;
+//     fp64: sixteen 16x16 accumulators per wavefront on v_mfma_f64_16x16x4_f64;
 //   - A is staged k-major ([k][m]) and B as [k][n] in LDS, double buffered, so every MFMA operand fetch is a
 //     conflict-free 4-byte LDS read of consecutive addresses; the next K step's global loads are issued before the
 //     MFMAs of the current one; workgroup ids are remapped so that each XCD (own L2) gets a contiguous range of tiles;
 //   - operands are addressed straight from the descriptors (any strides, broadcast batch dimensions, row-major
 //     target written directly): no pointer arrays, no column-major temporary and transposing copy-back as on the
 //     reference's BLAS paths (Tensor/Tensor/BlasSupport.fs:173-190, Cuda/CudaBLAS.fs:28-38).
-// The "fast" instantiation requires row-major, 16-byte aligned A and B and full tiles and uses 16-byte global loads;
-// every other case runs the same kernel with guarded scalar loads.
+// The "fast" instantiation (row-major, 16-byte aligned A and B) uses 16-byte global loads on interior tiles and guarded
+// scalar loads on edge tiles; every other layout runs the same kernel with guarded scalar loads throughout.
 #include "map_kernels.h"
 
 using namespace dnh;
@@ -23,6 +23,7 @@ constexpr int BM = 128, BN = 128, PAD = 4;
 template <class T> constexpr int kBK = sizeof(T) == 8 ? 8 : 16;  // K step: keeps the double-buffered tiles within 64 KB of LDS
 
 typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef double f64x4 __attribute__((ext_vector_type(4)));
 
 struct GemmArgs {
     int64_t M, N, K;
@@ -68,8 +69,11 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
     constexpr int SPT = BM * BK / kBlock;  // elements of each tile per thread
     T ra[SPT], rb[SPT];
 
-    auto load_tiles = [&](int64_t k0) {
-        if constexpr (FAST) {
+    // FAST = row-major, 16-byte aligned operands: interior tiles (decided per block and per K step) use 16-byte loads, edge
+    // tiles and every tile of other layouts use guarded scalar loads into the same LDS layout.
+    const bool full_mn = m0 + BM <= g.M && n0 + BN <= g.N;
+    auto load_tiles = [&](int64_t k0) -> bool {
+        if (FAST && full_mn && k0 + BK <= g.K) {
             constexpr int V = 16 / (int)sizeof(T);           // elements per 16-byte load
             constexpr int APT = (BM * BK) / (kBlock * V);     // loads per thread for A (fp32: 2, fp64: 4)
             constexpr int KV = BK / V;                        // vectors per A row
@@ -90,6 +94,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
 #pragma unroll
                 for (int e = 0; e < V; e++) rb[i * V + e] = v.v[e];
             }
+            return true;
         } else {
 #pragma unroll
             for (int i = 0; i < SPT; i++) {
@@ -105,10 +110,11 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
                     rb[i] = (k < g.K && n < g.N) ? b[k * g.sbk + n * g.sbn] : T(0);
                 }
             }
+            return false;
         }
     };
-    auto store_tiles = [&](int buf) {
-        if constexpr (FAST) {
+    auto store_tiles = [&](int buf, bool vec_layout) {
+        if (vec_layout) {
             constexpr int V = 16 / (int)sizeof(T);
             constexpr int APT = (BM * BK) / (kBlock * V);
             constexpr int KV = BK / V;
@@ -149,14 +155,14 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-        load_tiles(0);
-        store_tiles(0);
+        bool vl = load_tiles(0);
+        store_tiles(0, vl);
         __syncthreads();
         int cur = 0;
         const int lk = lane >> 5, lm = lane & 31;
         for (int64_t k0 = 0; k0 < g.K; k0 += BK) {
             const bool more = k0 + BK < g.K;
-            if (more) load_tiles(k0 + BK);
+            if (more) vl = load_tiles(k0 + BK);
             // Operand reads stay interleaved with the MFMAs (four per pair of LDS reads): hoisting all 32 reads of a K step
             // ahead of the MFMA chain costs 27 more registers, drops occupancy from 4 to 3 wavefronts per SIMD and measured
             // 6 % slower; with 4 wavefronts per SIMD the other wavefronts' MFMAs cover each LDS round trip.
@@ -172,7 +178,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
                 acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
             }
             if (more) {
-                store_tiles(cur ^ 1);
+                store_tiles(cur ^ 1, vl);
                 __syncthreads();
                 cur ^= 1;
             }
@@ -186,48 +192,53 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
                 for (int r = 0; r < 16; r++) {
                     const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
                     const int64_t n = n0 + wn + j * 32 + lm;
-                    if (FAST || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
+                    if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
                 }
     } else {
-        // fp64: each thread owns an 8x8 micro-tile (rows ty*8.., columns tx*8..)
-        const int ty = tid / 16, tx = tid % 16;
-        T acc[8][8];
+        // fp64: sixteen 16x16 accumulators per wavefront on v_mfma_f64_16x16x4_f64.  Operand lane l supplies A[l%16][l/16] and
+        // B[l/16][l%16]; accumulator register r of lane l holds row 4*r + l/16, column l%16 of its 16x16 tile.
+        f64x4 acc[4][4];
 #pragma unroll
-        for (int i = 0; i < 8; i++)
+        for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int j = 0; j < 8; j++) acc[i][j] = T(0);
-        load_tiles(0);
-        store_tiles(0);
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc[i][j][r] = 0.0;
+        bool vl = load_tiles(0);
+        store_tiles(0, vl);
         __syncthreads();
         int cur = 0;
+        const int lk = lane >> 4, lm = lane & 15;
         for (int64_t k0 = 0; k0 < g.K; k0 += BK) {
             const bool more = k0 + BK < g.K;
-            if (more) load_tiles(k0 + BK);
-#pragma unroll 4
-            for (int kk = 0; kk < BK; kk++) {
-                T av[8], bv[8];
+            if (more) vl = load_tiles(k0 + BK);
 #pragma unroll
-                for (int i = 0; i < 8; i++) av[i] = As[cur][kk][ty * 8 + i];
+            for (int kk = 0; kk < BK; kk += 4) {
+                double av[4], bv[4];
 #pragma unroll
-                for (int j = 0; j < 8; j++) bv[j] = Bs[cur][kk][tx * 8 + j];
+                for (int i = 0; i < 4; i++) av[i] = As[cur][kk + lk][wm + i * 16 + lm];
 #pragma unroll
-                for (int i = 0; i < 8; i++)
+                for (int j = 0; j < 4; j++) bv[j] = Bs[cur][kk + lk][wn + j * 16 + lm];
 #pragma unroll
-                    for (int j = 0; j < 8; j++) acc[i][j] = fma(av[i], bv[j], acc[i][j]);
+                for (int i = 0; i < 4; i++)
+#pragma unroll
+                    for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i], bv[j], acc[i][j], 0, 0, 0);
             }
             if (more) {
-                store_tiles(cur ^ 1);
+                store_tiles(cur ^ 1, vl);
                 __syncthreads();
                 cur ^= 1;
             }
         }
 #pragma unroll
-        for (int i = 0; i < 8; i++)
+        for (int i = 0; i < 4; i++)
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-                const int64_t m = m0 + ty * 8 + i, n = n0 + tx * 8 + j;
-                if (FAST || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j];
-            }
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    const int64_t m = m0 + wm + i * 16 + 4 * r + lk, n = n0 + wn + j * 16 + lm;
+                    if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
+                }
     }
 }
 
@@ -238,7 +249,7 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
     if (blocks > 0x7FFFFFFF) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: too many output tiles");
     g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
     constexpr int V = 16 / (int)sizeof(T);
-    bool fast = g.sak == 1 && g.sbn == 1 && (g.M % BM) == 0 && (g.N % BN) == 0 && (g.K % kBK<T>) == 0 && g.K > 0 &&
+    bool fast = g.sak == 1 && g.sbn == 1 && g.K > 0 &&
                 (g.sam % V) == 0 && (g.sbk % V) == 0 && aligned_to(a, 16) && aligned_to(b, 16);
     for (int d = 0; d < g.nbatch && fast; d++) fast = (g.bsa[d] % V) == 0 && (g.bsb[d] % V) == 0;
     if (fast) hipLaunchKernelGGL((gemm_kernel<T, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
