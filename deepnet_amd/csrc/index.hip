@@ -297,13 +297,27 @@ __device__ __forceinline__ uint64_t block_exclusive_scan64(uint64_t c, uint64_t*
     return base + inc - c;
 }
 
+// Counts the selected elements of each block's region (kFastJ * 256 * VEC consecutive mask bytes).  Counting is order-free,
+// so the region is read with 16-byte loads regardless of how the move pass assigns elements to threads.
 template <int VEC>
 __global__ __launch_bounds__(kBlock) void compact_count_fast_kernel(const uint8_t* mask, uint32_t nvec, uint32_t* counts) {
+    constexpr uint32_t REGION = kFastJ * kBlock * VEC;                 // mask bytes per block
+    const uint64_t n = (uint64_t)nvec * VEC;
+    const uint64_t r0 = (uint64_t)blockIdx.x * REGION;
+    const uint64_t r1 = r0 + REGION < n ? r0 + REGION : n;
     uint32_t c = 0;
+    for (uint64_t i = r0 + (uint64_t)threadIdx.x * 16; i < r1; i += (uint64_t)kBlock * 16) {
+        if (i + 16 <= r1) {
+            const Pack<uint32_t, 4> v = load_pack<uint32_t, 4>((const uint32_t*)(mask + i));
 #pragma unroll
-    for (int j = 0; j < kFastJ; j++) {
-        const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
-        if (v < nvec) c += __popc(mask_flags<VEC>(mask + (size_t)v * VEC));
+            for (int w = 0; w < 4; w++) {
+                // bytes are 0/1 booleans in the common case, but any nonzero byte counts as true
+                const uint32_t x = v.v[w];
+                c += ((x & 0xFFu) != 0) + ((x & 0xFF00u) != 0) + ((x & 0xFF0000u) != 0) + ((x & 0xFF000000u) != 0);
+            }
+        } else {
+            for (uint64_t j = i; j < r1; j++) c += mask[j] != 0;
+        }
     }
     uint32_t total;
     block_exclusive_scan(c, &total);
@@ -394,7 +408,7 @@ bool try_compaction_fast(const MaskArgs& m, void* full, void* out, const Lay& ol
     if (olay.nd != 1 || olay.stride[0] != 1) return false;
     if (n > (int64_t)kMaxItems || n == 0 || nout == 0) return false;
     const int vec = 16 / esize;
-    if ((n % vec) != 0 || !aligned_to(full, 16) || !aligned_to(m.mask[0], vec)) return false;
+    if ((n % vec) != 0 || !aligned_to(full, 16) || !aligned_to(m.mask[0], 16)) return false;
     switch (esize) {
         case 1: *status = run_compaction_fast<uint8_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
         case 4: *status = run_compaction_fast<uint32_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
