@@ -88,6 +88,11 @@ class DnhDeviceInfo(C.Structure):
     ]
 
 
+class DnhPoolStats(C.Structure):
+    _fields_ = [("live_bytes", C.c_int64), ("cached_bytes", C.c_int64), ("limit_bytes", C.c_int64),
+                ("hits", C.c_int64), ("misses", C.c_int64)]
+
+
 def make_descriptor(base: int, dtype, shape, stride, offset: int) -> DnhTensor:
     """Builds a descriptor from a storage pointer and a TensorLayout triple (elements, not bytes)."""
     nd = len(shape)
@@ -132,7 +137,8 @@ OP_SIGNATURES = {
 # every symbol include/tensor_hip.h declares
 EXPORTED_SYMBOLS = [
     "dnh_init", "dnh_device_info", "dnh_last_error", "dnh_async_error",
-    "dnh_alloc", "dnh_free", "dnh_host_alloc", "dnh_host_free", "dnh_memset",
+    "dnh_alloc", "dnh_free", "dnh_alloc_async", "dnh_free_async", "dnh_pool_trim", "dnh_pool_set_limit", "dnh_pool_stats",
+    "dnh_host_alloc", "dnh_host_free", "dnh_memset",
     "dnh_memcpy_h2d", "dnh_memcpy_d2h", "dnh_memcpy_d2d",
     "dnh_stream_create", "dnh_stream_destroy", "dnh_stream_sync", "dnh_device_sync",
     "dnh_event_create", "dnh_event_destroy", "dnh_event_record", "dnh_event_sync", "dnh_event_elapsed_ms",

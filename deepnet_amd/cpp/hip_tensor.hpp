@@ -178,19 +178,31 @@ struct Cfg {
     static bool& Stacktrace() { thread_local bool v = true; return v; }
 };
 
-// Device memory owned by one tensor storage (Cuda/CudaBackend.fs:54-93).
+// Device memory owned by one tensor storage (Cuda/CudaBackend.fs:54-93).  The block comes from the library's stream-ordered
+// cache under the stream current at creation; while every use is issued on that stream it is released without waiting for
+// the device, otherwise with the synchronising dnh_free.
 template <class T>
 class TensorHipStorage {
   public:
-    explicit TensorHipStorage(int64_t nElems) : nElems_(nElems) { check(dnh_alloc((size_t)(nElems > 0 ? nElems : 1) * sizeof(T), &ptr_)); }
-    ~TensorHipStorage() { if (ptr_) dnh_free(ptr_); }
+    explicit TensorHipStorage(int64_t nElems) : nElems_(nElems), stream_(Cfg::Stream()) {
+        check(dnh_alloc_async((size_t)(nElems > 0 ? nElems : 1) * sizeof(T), stream_, &ptr_));
+    }
+    ~TensorHipStorage() {
+        if (!ptr_) return;
+        if (singleStream_) dnh_free_async(ptr_, stream_); else dnh_free(ptr_);
+    }
     TensorHipStorage(const TensorHipStorage&) = delete;
     TensorHipStorage& operator=(const TensorHipStorage&) = delete;
-    void* Ptr() const { return ptr_; }
+    void* Ptr() const {
+        if (Cfg::Stream() != stream_) singleStream_ = false;
+        return ptr_;
+    }
     int64_t NElems() const { return nElems_; }
   private:
     void* ptr_ = nullptr;
     int64_t nElems_;
+    void* stream_;
+    mutable bool singleStream_ = true;
 };
 
 struct TensorHipDevice {                                      // Cuda/CudaBackend.fs:497-507

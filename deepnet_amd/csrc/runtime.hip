@@ -5,6 +5,7 @@
 
 #include <map>
 #include <mutex>
+#include <unordered_map>
 
 namespace dnh {
 
@@ -20,6 +21,36 @@ struct Workspace {
     size_t bytes = 0;
 };
 std::map<hipStream_t, Workspace> g_ws;
+
+// Stream-ordered block cache behind dnh_alloc_async / dnh_free_async.  A block released on stream S goes to S's free
+// list and may be handed out again only to an allocation on S: work already queued on S that still touches the block
+// runs before anything the new owner queues on S, so no wait is needed.  hipMalloc / hipFree (which synchronise the
+// device) are left for cache misses, trimming and out-of-memory retries.
+struct Pool {
+    std::mutex mu;
+    std::map<hipStream_t, std::multimap<size_t, void*>> free_blocks;
+    std::unordered_map<void*, size_t> live;  // blocks handed out and not yet released -> rounded size
+    size_t cached_bytes = 0, live_bytes = 0, limit_bytes = 0;  // limit 0 = keep everything until trimmed
+    uint64_t hits = 0, misses = 0;
+};
+Pool g_pool;
+
+size_t pool_round(size_t bytes) {
+    if (bytes == 0) bytes = 1;
+    const size_t g = bytes < ((size_t)1 << 20) ? 512 : ((size_t)2 << 20);
+    return (bytes + g - 1) / g * g;
+}
+
+// caller holds g_pool.mu
+int32_t pool_trim_locked() {
+    if (g_pool.cached_bytes == 0) return DNH_OK;
+    DNH_HIP(hipDeviceSynchronize());
+    for (auto& per_stream : g_pool.free_blocks)
+        for (auto& blk : per_stream.second) (void)hipFree(blk.second);
+    g_pool.free_blocks.clear();
+    g_pool.cached_bytes = 0;
+    return DNH_OK;
+}
 }  // namespace
 
 std::string& last_error() {
@@ -150,7 +181,99 @@ int32_t dnh_alloc(size_t bytes, void** out) {
 int32_t dnh_free(void* ptr) {
     if (!ptr) return DNH_OK;
     DNH_TRY(ensure_init());
+    {
+        std::lock_guard<std::mutex> lock(g_pool.mu);
+        auto it = g_pool.live.find(ptr);
+        if (it != g_pool.live.end()) {
+            g_pool.live_bytes -= it->second;
+            g_pool.live.erase(it);
+        }
+    }
     DNH_HIP(hipFree(ptr));  // hipFree waits for outstanding work that may still use the buffer
+    return DNH_OK;
+}
+
+int32_t dnh_alloc_async(size_t bytes, void* stream, void** out) {
+    if (!out) return fail(DNH_ERR_INVALID_ARG, "dnh_alloc_async: null argument");
+    DNH_TRY(ensure_init());
+    *out = nullptr;
+    const size_t want = pool_round(bytes);
+    std::lock_guard<std::mutex> lock(g_pool.mu);
+    auto fs = g_pool.free_blocks.find((hipStream_t)stream);
+    if (fs != g_pool.free_blocks.end()) {
+        auto it = fs->second.lower_bound(want);
+        if (it != fs->second.end() && it->first <= want + want / 4) {  // bounded waste: at most 25 % over the request
+            *out = it->second;
+            g_pool.live[*out] = it->first;
+            g_pool.live_bytes += it->first;
+            g_pool.cached_bytes -= it->first;
+            fs->second.erase(it);
+            g_pool.hits++;
+            return DNH_OK;
+        }
+    }
+    g_pool.misses++;
+    hipError_t e = hipMalloc(out, want);
+    if (e == hipErrorOutOfMemory) {
+        // the reference collects garbage and retries (Cuda/CudaUtils.fs:183-194); here the cache is what can be given back
+        (void)hipGetLastError();
+        DNH_TRY(pool_trim_locked());
+        e = hipMalloc(out, want);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *out = nullptr;
+        if (e == hipErrorOutOfMemory)
+            return fail(DNH_ERR_OUT_OF_MEMORY, "device memory allocation of %zu MB failed", want >> 20);
+        return fail(DNH_ERR_HIP, "hipMalloc(%zu): %s", want, hipGetErrorString(e));
+    }
+    g_pool.live[*out] = want;
+    g_pool.live_bytes += want;
+    return DNH_OK;
+}
+
+int32_t dnh_free_async(void* ptr, void* stream) {
+    if (!ptr) return DNH_OK;
+    DNH_TRY(ensure_init());
+    size_t bytes = 0;
+    {
+        std::lock_guard<std::mutex> lock(g_pool.mu);
+        auto it = g_pool.live.find(ptr);
+        if (it != g_pool.live.end()) {
+            bytes = it->second;
+            g_pool.live.erase(it);
+            g_pool.live_bytes -= bytes;
+            if (g_pool.limit_bytes == 0 || g_pool.cached_bytes + bytes <= g_pool.limit_bytes) {
+                g_pool.free_blocks[(hipStream_t)stream].emplace(bytes, ptr);
+                g_pool.cached_bytes += bytes;
+                return DNH_OK;
+            }
+        }
+    }
+    DNH_HIP(hipFree(ptr));  // not from the cache, or the cache is full
+    return DNH_OK;
+}
+
+int32_t dnh_pool_trim(void) {
+    DNH_TRY(ensure_init());
+    std::lock_guard<std::mutex> lock(g_pool.mu);
+    return pool_trim_locked();
+}
+
+int32_t dnh_pool_set_limit(size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_pool.mu);
+    g_pool.limit_bytes = bytes;
+    return DNH_OK;
+}
+
+int32_t dnh_pool_stats(DnhPoolStats* stats) {
+    if (!stats) return fail(DNH_ERR_INVALID_ARG, "dnh_pool_stats: null argument");
+    std::lock_guard<std::mutex> lock(g_pool.mu);
+    stats->live_bytes = (int64_t)g_pool.live_bytes;
+    stats->cached_bytes = (int64_t)g_pool.cached_bytes;
+    stats->limit_bytes = (int64_t)g_pool.limit_bytes;
+    stats->hits = (int64_t)g_pool.hits;
+    stats->misses = (int64_t)g_pool.misses;
     return DNH_OK;
 }
 
@@ -207,6 +330,17 @@ int32_t dnh_stream_destroy(void* stream) {
     if (!stream) return DNH_OK;
     DNH_HIP(hipStreamSynchronize((hipStream_t)stream));
     drop_workspace((hipStream_t)stream);
+    {
+        // everything queued on the stream has finished, so its cached blocks are free for any stream; keep them under
+        // the default stream, whose later work is ordered after this point on the host
+        std::lock_guard<std::mutex> lock(g_pool.mu);
+        auto it = g_pool.free_blocks.find((hipStream_t)stream);
+        if (it != g_pool.free_blocks.end()) {
+            auto& dflt = g_pool.free_blocks[(hipStream_t) nullptr];
+            for (auto& blk : it->second) dflt.emplace(blk.first, blk.second);
+            g_pool.free_blocks.erase((hipStream_t)stream);
+        }
+    }
     DNH_HIP(hipStreamDestroy((hipStream_t)stream));
     return DNH_OK;
 }

@@ -42,14 +42,23 @@ module internal Desc =
         d
 
 /// Device memory owned by one tensor storage (CudaBackend.fs:54-93).
+/// The block comes from the library's stream-ordered cache under the stream current at creation.  While every use was
+/// issued on that stream the finalizer hands it back without waiting for the device (the finalizer runs after the last
+/// operation on the storage was queued, whichever thread it runs on); otherwise it uses the synchronising free.
 type TensorHipStorage<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> ValueType> (nElems: int64) =
     let bytes = unativeint (max nElems 1L) * unativeint sizeof<'T>
+    let stream = Cfg.Stream
+    let mutable singleStream = true
     let mutable ptr = IntPtr.Zero
-    do Native.check (Native.dnh_alloc (bytes, &ptr))
+    do Native.check (Native.dnh_alloc_async (bytes, stream, &ptr))
 
-    member this.Ptr = ptr
+    member this.Ptr =
+        if Cfg.Stream <> stream then singleStream <- false
+        ptr
     member this.NElems = nElems
-    override this.Finalize () = if ptr <> IntPtr.Zero then Native.dnh_free ptr |> ignore
+    override this.Finalize () =
+        if ptr <> IntPtr.Zero then
+            (if singleStream then Native.dnh_free_async (ptr, stream) else Native.dnh_free ptr) |> ignore
 
     interface ITensorStorage<'T> with
         member this.Backend layout = TensorHipBackend<'T> (layout, this) :> ITensorBackend<_>

@@ -43,6 +43,9 @@ module internal Native =
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_async_error (nativeint stream, int& code)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_alloc (unativeint bytes, nativeint& ptr)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_free (nativeint ptr)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_alloc_async (unativeint bytes, nativeint stream, nativeint& ptr)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_free_async (nativeint ptr, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_pool_trim ()
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_memcpy_h2d (nativeint dst, nativeint src, unativeint bytes, nativeint stream, int sync)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_memcpy_d2h (nativeint dst, nativeint src, unativeint bytes, nativeint stream, int sync)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_stream_sync (nativeint stream)

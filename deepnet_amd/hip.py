@@ -34,18 +34,27 @@ Cfg = _Cfg()
 
 
 class TensorHipStorage(ITensorStorage):
-    """Owns one device allocation (CudaBackend.fs:54-93).  Freed when collected."""
+    """Owns one device allocation (CudaBackend.fs:54-93).  Released when collected.
+
+    The block comes from the library's stream-ordered cache, tagged with the stream that is current at creation.  While
+    every operation on the storage is issued on that stream, release hands the block back to the cache without waiting
+    for the device; once its pointer has been taken under another stream it is released with the synchronising free."""
 
     def __init__(self, nElems: int, dtype, dev: "TensorHipDevice"):
         self.Dev = dev
         self.DataType = np.dtype(dtype)
         self.NElems = int(nElems)
         self._lib = native.load()
+        self._stream = Cfg.Stream
+        self._single_stream = True
         ptr = C.c_void_p()
-        native.check(self._lib.dnh_alloc(max(self.NElems, 1) * self.DataType.itemsize, C.byref(ptr)))
+        native.check(self._lib.dnh_alloc_async(max(self.NElems, 1) * self.DataType.itemsize, self._stream, C.byref(ptr)))
         self._ptr = ptr.value
 
     def Pointer(self) -> int:
+        # every operation fetches the pointer when it is issued, under the stream it is issued on
+        if Cfg.Stream != self._stream:
+            self._single_stream = False
         return self._ptr
 
     @property
@@ -58,7 +67,10 @@ class TensorHipStorage(ITensorStorage):
     def __del__(self):
         try:
             if getattr(self, "_ptr", None):
-                self._lib.dnh_free(self._ptr)
+                if self._single_stream:
+                    self._lib.dnh_free_async(self._ptr, self._stream)
+                else:
+                    self._lib.dnh_free(self._ptr)
                 self._ptr = None
         except Exception:
             pass

@@ -34,6 +34,11 @@ def load() -> C.CDLL:
         "dnh_async_error": [vp, C.POINTER(i32)],
         "dnh_alloc": [sz, C.POINTER(vp)],
         "dnh_free": [vp],
+        "dnh_alloc_async": [sz, vp, C.POINTER(vp)],
+        "dnh_free_async": [vp, vp],
+        "dnh_pool_trim": [],
+        "dnh_pool_set_limit": [sz],
+        "dnh_pool_stats": [C.POINTER(abi.DnhPoolStats)],
         "dnh_host_alloc": [sz, C.POINTER(vp)],
         "dnh_host_free": [vp],
         "dnh_memset": [vp, i32, sz, vp],

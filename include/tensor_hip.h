@@ -81,6 +81,15 @@ typedef struct DnhDeviceInfo {
     char    arch[64];
 } DnhDeviceInfo;
 
+/* State of the block cache behind dnh_alloc_async / dnh_free_async. */
+typedef struct DnhPoolStats {
+    int64_t live_bytes;    /* handed out and not yet released                      */
+    int64_t cached_bytes;  /* released and kept for reuse                          */
+    int64_t limit_bytes;   /* cap on cached_bytes, 0 = none                        */
+    int64_t hits;          /* allocations served from the cache                    */
+    int64_t misses;        /* allocations that went to the driver                  */
+} DnhPoolStats;
+
 /* Unary element ops: ITensorBackend UnaryPlus..Truncate (TensorBackend.fs:74-94), Negate (:113);
  * scalar semantics Host/ScalarOps.fs:381-493, ScalarPrimitives.fs:54-150, Sgn.fs:11-15.
  * Round is ties-to-even (F# `round`), unlike the reference CUDA kernel (Cuda/Kernels/Elemwise.cuh:128). */
@@ -135,6 +144,18 @@ int32_t dnh_async_error(void* stream, int32_t* code);
  * ------------------------------------------------------------------------------------------------- */
 int32_t dnh_alloc(size_t bytes, void** out);          /* at least one byte is allocated (CudaBackend.fs:56-58) */
 int32_t dnh_free(void* ptr);                          /* waits for in-flight work; callable from any thread    */
+/* Stream-ordered storage for tensors created inside a chain of operations (every Tensor op allocates its result,
+ * Tensor.fs:317-325, and the reference pays a driver allocation plus GC pressure handling for each one,
+ * Cuda/CudaUtils.fs:179-210).  A block released with dnh_free_async(ptr, stream) is handed out again only to
+ * dnh_alloc_async calls that name the same stream, so neither call waits for the device.  `stream` must be the one
+ * stream all work on the block was queued on; a block used from several streams is released with dnh_free.
+ * When the driver is out of memory the cache is emptied and the allocation retried once (the reference's GC retry).
+ * dnh_free accepts blocks from either allocator. */
+int32_t dnh_alloc_async(size_t bytes, void* stream, void** out);
+int32_t dnh_free_async(void* ptr, void* stream);
+int32_t dnh_pool_trim(void);                          /* waits for the device, returns every cached block to the driver */
+int32_t dnh_pool_set_limit(size_t bytes);             /* cap on cached bytes; 0 (default) = no cap                      */
+int32_t dnh_pool_stats(DnhPoolStats* stats);
 int32_t dnh_host_alloc(size_t bytes, void** out);     /* pinned host memory for transfers                      */
 int32_t dnh_host_free(void* ptr);
 int32_t dnh_memset(void* dst, int32_t byte_value, size_t bytes, void* stream);
