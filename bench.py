@@ -28,8 +28,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, vendor figure
 FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by the plain-copy calibration
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): 2.0 * 262162.9 KiB + 262145.4 KiB for Add.
-TRAFFIC_BYTES = {"Add": int((2.0 * 262162.9 + 262145.4) * 1024)}
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): 2.0 * 262151.3 KiB + 262144.9 KiB for Add.
+TRAFFIC_BYTES = {"Add": int((2.0 * 262151.3 + 262144.9) * 1024)}
 
 
 def log(*a):
@@ -243,7 +243,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "fp32 8192x8192 (64Mi elems): Add, Tanh, Sum/Max/ArgMax along last axis and along first axis, full Sum; "
                                "inputs resident in HBM, targets preallocated, seed 123",
-                   "bytes_per_step": total_bytes, "device": info.name.decode()},
+                   "bytes_per_step": total_bytes, "device": info.name.decode() or info.arch.decode()},
         "roofline": roofline, "cpu_baseline": cpu, "per_kernel": per_kernel,
     }))
 

@@ -153,6 +153,37 @@ class Tensor:
         t.Backend.FillIncrementing(np.dtype(dtype).type(0), np.dtype(dtype).type(1), t)
         return t
 
+    @staticmethod
+    def arange(start, incr, stop, dev, dtype) -> "Tensor":
+        """Tensor.fs:3853-3861: max 0 ((stop - start) / incr) elements, the division done in the element type."""
+        dt = np.dtype(dtype)
+        if dt.kind == "f":
+            n = int(dt.type(dt.type(stop) - dt.type(start)) / dt.type(incr))
+        else:
+            q = abs(int(stop) - int(start)) // abs(int(incr))             # integer division truncates toward zero
+            n = q if (int(stop) - int(start)) * int(incr) >= 0 else -q
+        t = Tensor.new([max(0, n)], dev, dtype)
+        t.Backend.FillIncrementing(dt.type(start), dt.type(incr), t)
+        return t
+
+    @staticmethod
+    def linspace(start, stop, nElems, dev, dtype) -> "Tensor":
+        """Tensor.fs:3879-3886."""
+        if nElems < 2:
+            raise ValueError("linspace requires at least two elements.")
+        dt = np.dtype(dtype)
+        incr = dt.type(dt.type(stop) - dt.type(start)) / dt.type(nElems - 1)
+        t = Tensor.new([nElems], dev, dtype)
+        t.Backend.FillIncrementing(dt.type(start), dt.type(incr), t)
+        return t
+
+    @staticmethod
+    def identity(size, dev, dtype) -> "Tensor":
+        """Tensor.fs:3813-3817: zeros, then ones on the diagonal view."""
+        x = Tensor.zeros([size, size], dev, dtype)
+        x.diagAxis(0, 1).FillConst(np.dtype(dtype).type(1))
+        return x
+
     def FillConst(self, value):
         self.Backend.FillConst(value, self)
 

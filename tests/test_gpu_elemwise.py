@@ -215,6 +215,25 @@ def test_fill_and_counting(H, G):
     assert got.shape == (3, 0, 4)
 
 
+def test_arange_linspace_identity(H, G):
+    """Tensor.fs:3813-3886.  arange 1 1 10 has nine elements (BaseTests.fs:55); arange 1 2 10 has four (RatTests.fs:127)."""
+    for dt in NUM:
+        for args in ((1, 1, 10), (1, 2, 10), (0, 3, 100), (5, 1, 5)):
+            ref, got = both(H, G, lambda x: type(x).arange(*args, x.Dev, x.DataType), np.zeros(1, dt))
+            assert_exact(ref, got)
+            assert_exact(np.arange(args[0], args[0] + len(got) * args[1], args[1]).astype(dt), got)
+            assert len(got) == max(0, (args[2] - args[0]) // args[1])
+        ref, got = both(H, G, lambda x: type(x).identity(37, x.Dev, x.DataType), np.zeros(1, dt))
+        assert_exact(ref, got)
+        assert_exact(np.eye(37, dtype=dt), got)
+    for dt in (np.float32, np.float64):
+        ref, got = both(H, G, lambda x: type(x).linspace(0, 5, 11, x.Dev, x.DataType), np.zeros(1, dt))
+        assert_exact(ref, got)
+        np.testing.assert_allclose(got, np.linspace(0, 5, 11), rtol=1e-6)
+    with pytest.raises(ValueError):
+        G.Dev and type(G.zeros([1], np.float32)).linspace(0, 1, 1, G.Dev, np.float32)
+
+
 def test_empty_and_scalar(H, G):
     ref, got = both(H, G, lambda a, b: a + b, np.zeros((0, 5), np.float32), np.zeros((0, 5), np.float32))
     assert got.shape == (0, 5)
