@@ -146,7 +146,7 @@ def main():
                         G.synchronize()
                         ts.append((time.perf_counter() - t0) * 1e3)
                     out.write(f"{m},{shape_s},{tname},Hip,{np.mean(ts):.4f},{np.std(ts):.4f}\n")
-                except (NotImplementedError, ValueError, TypeError, AttributeError) as e:
+                except (NotImplementedError, ValueError, TypeError, ArithmeticError):
                     out.write(f"{m},{shape_s},{tname},Hip,NA,NA\n")
                     G.synchronize()
                 out.flush()

@@ -18,6 +18,7 @@ DNH_ERR_OUT_OF_MEMORY = 3
 DNH_ERR_HIP = 4
 DNH_ERR_INDEX_OUT_OF_RANGE = 5
 DNH_ERR_NOT_INITIALIZED = 6
+DNH_ERR_SINGULAR_MATRIX = 7
 
 # DnhDType
 DNH_BOOL, DNH_U8, DNH_I8, DNH_I32, DNH_U32, DNH_I64, DNH_U64, DNH_F32, DNH_F64 = range(9)
@@ -132,6 +133,7 @@ OP_SIGNATURES = {
     "masked_set": [_T, _TT, C.c_int32, _T],
     "true_indices": [_T, _T],
     "dot": [_T, _T, _T],
+    "batched_invert": [_T, _T],
 }
 
 # every symbol include/tensor_hip.h declares

@@ -16,6 +16,10 @@ from . import abi
 from .layout import TensorLayout
 
 
+class SingularMatrixException(ArithmeticError):
+    """Raised when a matrix that is not invertible is inverted (Tensor/Tensor/Tensor.fs:2831-2834)."""
+
+
 class ITensorDevice:
     """TensorBackend.fs:22-30.  Devices compare by Id (BaseTensorDevice, TensorBackend.fs:149-180)."""
     Id: str = "?"
@@ -208,12 +212,12 @@ class CAbiTensorBackend:
     def MatMatDot(self, trgt, src1, src2): self._dot(trgt, src1, src2)
     def BatchedMatMatDot(self, trgt, src1, src2): self._dot(trgt, src1, src2)
 
-    # not on the accelerated path (the reference's CUDA backend also leaves SVD/eigen unsupported, CudaBackend.fs:486-492)
+    # the reference's CUDA backend also leaves SVD/eigen unsupported (CudaBackend.fs:486-492)
     def BatchedSVD(self, trgtS, trgtUV, src1):
         raise NotImplementedError("BatchedSVD is not supported by this backend")
 
     def BatchedInvert(self, trgt, src1):
-        raise NotImplementedError("BatchedInvert is not supported by this backend")
+        self._call("batched_invert", C.byref(self._desc(trgt)), C.byref(self._desc(src1)))
 
     def SymmetricEigenDecomposition(self, part, trgtEigVals, trgtEigVecs, src):
         raise NotImplementedError("SymmetricEigenDecomposition is not supported by this backend")

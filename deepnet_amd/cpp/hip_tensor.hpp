@@ -7,7 +7,8 @@
 //   Tensor<T> ............................. the prepare-target / broadcast-sources / one-backend-call frontend of
 //                                            Tensor/Tensor/Tensor.fs (helpers :4520-4597)
 // .NET exceptions map to: InvalidOperation/Argument -> std::invalid_argument, NotSupported -> NotSupportedException,
-// IndexOutOfRange -> std::out_of_range, OutOfMemory -> std::bad_alloc, other HIP failures -> HipException.
+// IndexOutOfRange -> std::out_of_range, OutOfMemory -> std::bad_alloc, SingularMatrixException under its own name,
+// other HIP failures -> HipException.
 // No arithmetic on tensor data happens here; every operation is one call into libtensor_hip.so.
 #pragma once
 
@@ -29,6 +30,7 @@ using Shape = std::vector<int64_t>;
 
 struct NotSupportedException : std::runtime_error { using std::runtime_error::runtime_error; };
 struct HipException : std::runtime_error { using std::runtime_error::runtime_error; };
+struct SingularMatrixException : std::runtime_error { using std::runtime_error::runtime_error; };   // Tensor.fs:2831-2834
 
 constexpr int64_t NotFound = DNH_NOT_FOUND;                         // SpecialIdx.NotFound, TensorRng.fs:24
 constexpr int64_t Remainder = (-9223372036854775807LL - 1LL) + 3;   // SpecialIdx.Remainder, TensorRng.fs:21
@@ -167,6 +169,7 @@ inline void check(int32_t status) {
         case DNH_ERR_NOT_SUPPORTED: throw NotSupportedException(buf);
         case DNH_ERR_OUT_OF_MEMORY: throw std::bad_alloc();
         case DNH_ERR_INDEX_OUT_OF_RANGE: throw std::out_of_range(buf);
+        case DNH_ERR_SINGULAR_MATRIX: throw SingularMatrixException(buf);
         default: throw HipException(buf);
     }
 }
@@ -324,7 +327,7 @@ struct TensorHipBackend {
     static void MatVecDot(const Tensor<T>& t, const Tensor<T>& a, const Tensor<T>& b) { dot(t, a, b); }
     static void MatMatDot(const Tensor<T>& t, const Tensor<T>& a, const Tensor<T>& b) { dot(t, a, b); }
     static void BatchedMatMatDot(const Tensor<T>& t, const Tensor<T>& a, const Tensor<T>& b) { dot(t, a, b); }
-    static void BatchedInvert(const Tensor<T>&, const Tensor<T>&) { throw NotSupportedException("BatchedInvert is not supported by the HIP backend"); }
+    static void BatchedInvert(const Tensor<T>& trgt, const Tensor<T>& src) { auto t = desc(trgt); auto s = desc(src); check(dnh_batched_invert(&t, &s, Cfg::Stream())); }
 };
 
 // ---- Tensor<'T> frontend (Tensor.fs), the part that drives the backend path -----------------------------------------------------------
@@ -506,6 +509,13 @@ class Tensor {
         Tensor<bool> fm = mask.flatten();
         Backend::MaskedSet(Relayout(*view), {&fm}, value.broadcastTo(Shape{mask.countTrue()}));
     }
+
+    // (batched) matrix inverse (Tensor.fs:2807-2839)
+    void FillInvert(const Tensor& a) const {
+        if (a.NDims() < 2) throw std::invalid_argument("Need at least a matrix to invert.");
+        Backend::BatchedInvert(*this, a.broadcastTo(Shape_()));
+    }
+    static Tensor invert(const Tensor& a) { Tensor t(a.Shape_()); t.FillInvert(a); return t; }
 
     // dot, dispatched by rank as Tensor.(.*) / FillDot (Tensor.fs:2714-2797)
     Tensor dot(const Tensor& b) const {

@@ -33,6 +33,7 @@ struct GemmArgs {
     int64_t bsa[DNH_MAX_DIMS], bsb[DNH_MAX_DIMS], bsc[DNH_MAX_DIMS];
     uint32_t tiles_m, tiles_n;
     uint32_t xcd_chunk;                           // total tiles / 8 when divisible, else 0 (identity order)
+    uint32_t accumulate;                          // 1: c += a.b (used by the blocked matrix inversion), 0: c = a.b
 };
 
 template <class T, bool FAST>
@@ -192,7 +193,10 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
                 for (int r = 0; r < 16; r++) {
                     const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
                     const int64_t n = n0 + wn + j * 32 + lm;
-                    if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
+                    if (full_mn || (m < g.M && n < g.N)) {
+                        T* dst = c + m * g.scm + n * g.scn;
+                        *dst = g.accumulate ? *dst + acc[i][j][r] : acc[i][j][r];
+                    }
                 }
     } else {
         // fp64: sixteen 16x16 accumulators per wavefront on v_mfma_f64_16x16x4_f64.  Operand lane l supplies A[l%16][l/16] and
@@ -237,7 +241,10 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
 #pragma unroll
                 for (int r = 0; r < 4; r++) {
                     const int64_t m = m0 + wm + i * 16 + 4 * r + lk, n = n0 + wn + j * 16 + lm;
-                    if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
+                    if (full_mn || (m < g.M && n < g.N)) {
+                        T* dst = c + m * g.scm + n * g.scn;
+                        *dst = g.accumulate ? *dst + acc[i][j][r] : acc[i][j][r];
+                    }
                 }
     }
 }
@@ -424,6 +431,30 @@ bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t strea
 }
 
 }  // namespace
+
+namespace dnh {
+// c[b] (M x N, row stride ldc) += a[b] (M x K, row stride lda) . b[b] (K x N, row stride ldb) for b < batch; all row-major.
+int32_t gemm_accumulate(int32_t dtype, void* c, const void* a, const void* b, int64_t M, int64_t N, int64_t K, int64_t lda,
+                        int64_t ldb, int64_t ldc, int64_t batch, int64_t bsa, int64_t bsb, int64_t bsc, hipStream_t stream) {
+    if (M == 0 || N == 0 || K == 0 || batch == 0) return DNH_OK;
+    if (batch > 0xFFFFFFFFLL) return fail(DNH_ERR_NOT_SUPPORTED, "gemm_accumulate: batch too large");
+    GemmArgs g;
+    memset(&g, 0, sizeof(g));
+    g.M = M; g.N = N; g.K = K;
+    g.sam = lda; g.sak = 1; g.sbk = ldb; g.sbn = 1; g.scm = ldc; g.scn = 1;
+    g.accumulate = 1;
+    if (batch > 1) {
+        g.nbatch = 1;
+        g.bshape[0] = (uint32_t)batch;
+        g.bsa[0] = bsa; g.bsb[0] = bsb; g.bsc[0] = bsc;
+    }
+    g.tiles_m = cdiv(M, BM);
+    g.tiles_n = cdiv(N, BN);
+    if (dtype == DNH_F32) return launch_gemm<float>(g, (float*)c, (const float*)a, (const float*)b, batch, stream);
+    if (dtype == DNH_F64) return launch_gemm<double>(g, (double*)c, (const double*)a, (const double*)b, batch, stream);
+    return fail(DNH_ERR_NOT_SUPPORTED, "gemm_accumulate: only single and double");
+}
+}  // namespace dnh
 
 extern "C" int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream) {
     DNH_TRY(ensure_init());

@@ -1,0 +1,347 @@
+// ITensorBackend.BatchedInvert (Tensor/Tensor/TensorBackend.fs:144; host: LAPACK getrf + getri per matrix,
+// Host/HostBackend.fs:548-576; CUDA: cuBLAS getrfBatched + getriBatched, Cuda/CudaBackend.fs:451-484).
+//
+// Blocked in-place Gauss-Jordan inversion with partial (row) pivoting, all matrices of the batch side by side:
+//   for each block of NB columns
+//     1. panel kernel (one workgroup per matrix): NB Gauss-Jordan steps restricted to the block's columns, over all rows;
+//        the pivot of step k is the entry of largest magnitude in column k among rows >= k (lowest row on ties, as LAPACK's
+//        i?amax); rows are exchanged inside the panel and the exchange recorded.  In-place Gauss-Jordan leaves the column of
+//        the elimination matrix where the eliminated column was, so afterwards the panel holds G = columns of the product of
+//        the NB elimination steps.
+//     2. swap kernel: the recorded row exchanges are applied to the other columns, and the block's rows are copied to T.
+//     3. one GEMM on the matrix cores: W += (G - I_block) . T, i.e. the NB elimination steps applied to every other column.
+//   finally the row exchanges are undone as column exchanges in reverse order (composed into one permutation, one pass).
+// A pivot that is exactly zero marks the matrix singular (LAPACK's info > 0), reported as DNH_ERR_SINGULAR_MATRIX.
+// Floating point only; the work is 2 n^3 flops per matrix, nearly all of it in step 3.
+#include "common.h"
+
+namespace dnh {
+int32_t gemm_accumulate(int32_t dtype, void* c, const void* a, const void* b, int64_t M, int64_t N, int64_t K, int64_t lda,
+                        int64_t ldb, int64_t ldc, int64_t batch, int64_t bsa, int64_t bsb, int64_t bsc, hipStream_t stream);
+}
+
+using namespace dnh;
+
+namespace {
+
+constexpr int NB = 32;             // panel width = K of the update GEMM
+constexpr int kMaxPanelThreads = 1024;
+
+template <class T>
+__device__ inline T abs_of(T x) { return x < T(0) ? -x : x; }
+
+// (value, row) candidates are combined so that the largest magnitude wins and, on equal magnitudes, the lowest row.
+template <class T>
+__device__ inline void block_arg_max(T& best, int& bi, T* red_v, int* red_i) {
+    const int tid = threadIdx.x, nwaves = blockDim.x >> 6;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) {
+        const T ov = __shfl_xor(best, off, 64);
+        const int oi = __shfl_xor(bi, off, 64);
+        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+    if ((tid & 63) == 0) { red_v[tid >> 6] = best; red_i[tid >> 6] = bi; }
+    __syncthreads();
+    best = red_v[0];
+    bi = red_i[0];
+    for (int k = 1; k < nwaves; k++) {
+        const T ov = red_v[k];
+        const int oi = red_i[k];
+        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+    }
+}
+
+// Thread layout of the panel kernel: lane l of a wavefront works on panel column l % 32 of row l / 32 + 2 * (wavefront, pass),
+// so one wavefront instruction touches two whole 32-element row segments (coalesced), and the multiplier of a row — its entry in
+// the pivot column — comes from the lane that holds it by a shuffle.
+template <class T>
+__global__ __launch_bounds__(kMaxPanelThreads) void invert_panel_kernel(T* __restrict__ w, T* __restrict__ gbuf, int32_t* __restrict__ ipiv,
+                                                                        int32_t* singular, int n, int ld, int kb, int wc, int64_t bs_w,
+                                                                        int64_t bs_g) {
+    T* P = w + (int64_t)blockIdx.x * bs_w;
+    T* G = gbuf + (int64_t)blockIdx.x * bs_g;
+    int32_t* piv = ipiv + (int64_t)blockIdx.x * n;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const int jj = tid & 31, rsub = tid >> 5, rpp = nt >> 5, half = tid & 32;
+    const bool in_panel = jj < wc;
+    __shared__ T srow[NB];
+    __shared__ T red_v[2][kMaxPanelThreads / 64];
+    __shared__ int red_i[2][kMaxPanelThreads / 64];
+
+    // pivot candidates of the panel's first column; for the later columns they are collected while the column is updated
+    T best = T(-1);
+    int bi = n;
+    for (int r = kb + tid; r < n; r += nt) {
+        const T v = abs_of(P[(int64_t)r * ld + kb]);
+        if (v > best) { best = v; bi = r; }
+    }
+    for (int j = 0; j < wc; j++) {
+        const int col = kb + j;
+        block_arg_max(best, bi, red_v[j & 1], red_i[j & 1]);   // NaN never wins; lowest row on ties
+        int p = bi;
+        if (!(best > T(0))) {   // zero column (or nothing comparable): singular; carry on so every thread reaches the end
+            p = col;
+            if (tid == 0) *singular = 1;
+        }
+        if (tid == 0) piv[col] = p;
+        if (p != col && tid < wc) {
+            T* x = P + (int64_t)col * ld + kb + tid;
+            T* y = P + (int64_t)p * ld + kb + tid;
+            const T t = *x; *x = *y; *y = t;
+        }
+        __syncthreads();
+        // the pivot row, scaled: the in-place form puts 1/pivot where the pivot was
+        if (tid < wc) {
+            const T pv = P[(int64_t)col * ld + col];
+            const T x = P[(int64_t)col * ld + kb + tid];
+            srow[tid] = (tid == j ? T(1) : x) / pv;
+        }
+        __syncthreads();
+        const T sj = in_panel ? srow[jj] : T(0);
+        best = T(-1);
+        bi = n;
+        constexpr int U = 4;
+        for (int r0 = rsub; r0 < n; r0 += rpp * U) {
+            T v[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int r = r0 + u * rpp;
+                v[u] = (in_panel && r < n) ? P[(int64_t)r * ld + kb + jj] : T(0);
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int r = r0 + u * rpp;
+                const T f = __shfl(v[u], half | j, 64);   // this row's entry in the pivot column
+                if (in_panel && r < n) {
+                    const T nv = (r == col) ? sj : ((jj == j) ? T(0) : v[u]) - f * sj;
+                    P[(int64_t)r * ld + kb + jj] = nv;
+                    if (jj == j + 1 && r > col) {           // next column's pivot candidates, rows in ascending order per thread
+                        const T a = abs_of(nv);
+                        if (a > best) { best = a; bi = r; }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    // G - I_block for the update of the other columns; columns beyond the panel's width are never read (the GEMM's K is wc)
+    if (in_panel)
+        for (int r = rsub; r < n; r += rpp)
+            G[(int64_t)r * NB + jj] = P[(int64_t)r * ld + kb + jj] - ((r == kb + jj) ? T(1) : T(0));
+}
+
+// One thread per column outside the panel: applies the panel's row exchanges in order, then copies the block's rows to T.
+// Panel columns of T are zero so the update leaves the panel as it is.
+template <class T>
+__global__ __launch_bounds__(256) void invert_swap_kernel(T* __restrict__ w, T* __restrict__ tbuf, const int32_t* __restrict__ ipiv, int n,
+                                                          int ld, int kb, int wc, int64_t bs_w, int64_t bs_t) {
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= n) return;
+    T* P = w + (int64_t)blockIdx.y * bs_w;
+    T* Tb = tbuf + (int64_t)blockIdx.y * bs_t;
+    const int32_t* piv = ipiv + (int64_t)blockIdx.y * n;
+    if (c >= kb && c < kb + wc) {
+        for (int j = 0; j < wc; j++) Tb[(int64_t)j * ld + c] = T(0);
+        return;
+    }
+    // the rows that take part: the block's own rows and the rows they were exchanged with.  The exchanges are replayed on
+    // registers, so memory sees one round of loads and one round of stores instead of wc dependent round trips.
+    T own[NB], other[NB];
+    int prow[NB];
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        if (j < wc) {
+            prow[j] = piv[kb + j];
+            own[j] = P[(int64_t)(kb + j) * ld + c];
+            other[j] = P[(int64_t)prow[j] * ld + c];
+        }
+    }
+    // replay: position kb+j <-> position prow[j].  A position outside the block may appear several times in prow, and a
+    // position inside the block may be the partner of an earlier step; track values by position.
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        if (j < wc) {
+            const int p = prow[j];
+            if (p != kb + j) {
+                // current value at position p: inside the block -> own[p-kb]; outside -> the latest copy among other[]
+                if (p < kb + wc) {
+                    const T t = own[j];
+#pragma unroll
+                    for (int q = 0; q < NB; q++)
+                        if (q == p - kb) { own[j] = own[q]; own[q] = t; }
+                } else {
+                    // find the first slot that represents position p (the canonical holder of its current value)
+                    int holder = j;
+#pragma unroll
+                    for (int q = NB - 1; q >= 0; q--)
+                        if (q < j && prow[q] == p) holder = q;
+                    T cur;
+                    cur = other[j];
+#pragma unroll
+                    for (int q = 0; q < NB; q++)
+                        if (q == holder) cur = other[q];
+                    const T t = own[j];
+                    own[j] = cur;
+#pragma unroll
+                    for (int q = 0; q < NB; q++)
+                        if (q == holder) other[q] = t;
+                }
+            }
+        }
+    }
+    // write back: block rows, then every outside position once (from its canonical holder)
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        if (j < wc) {
+            P[(int64_t)(kb + j) * ld + c] = own[j];
+            Tb[(int64_t)j * ld + c] = own[j];
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+        if (j < wc) {
+            const int p = prow[j];
+            if (p >= kb + wc) {
+                bool first = true;
+#pragma unroll
+                for (int q = 0; q < NB; q++)
+                    if (q < j && prow[q] == p) first = false;
+                if (first) P[(int64_t)p * ld + c] = other[j];
+            }
+        }
+    }
+}
+
+// Composes the column permutation that undoes the row exchanges: exchanges are applied to columns in reverse order.
+// perm[j] = the column of the work matrix that becomes column j of the inverse.
+__global__ __launch_bounds__(256) void invert_perm_kernel(int32_t* __restrict__ perm, const int32_t* __restrict__ ipiv, int n, int use_lds) {
+    extern __shared__ int32_t sp[];
+    int32_t* out = perm + (int64_t)blockIdx.x * n;
+    const int32_t* piv = ipiv + (int64_t)blockIdx.x * n;
+    int32_t* cur = use_lds ? sp : out;
+    for (int i = threadIdx.x; i < n; i += 256) cur[i] = i;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = n - 1; k >= 0; k--) {
+            const int p = piv[k];
+            if (p != k) { const int32_t t = cur[k]; cur[k] = cur[p]; cur[p] = t; }
+        }
+    }
+    __syncthreads();
+    if (use_lds)
+        for (int i = threadIdx.x; i < n; i += 256) out[i] = sp[i];
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void invert_unpermute_kernel(T* __restrict__ out, const T* __restrict__ w, const int32_t* __restrict__ perm,
+                                                               int n, int ld, int64_t bs_w) {
+    const int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= n) return;
+    const int i = blockIdx.y;
+    const int64_t b = blockIdx.z;
+    out[(b * n + i) * (int64_t)n + j] = w[b * bs_w + (int64_t)i * ld + perm[b * n + j]];
+}
+
+__global__ void invert_clear_flag_kernel(int32_t* flag) { *flag = 0; }
+
+size_t align_up(size_t x) { return (x + 255) / 256 * 256; }
+
+template <class T>
+int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream) {
+    const int nd = t->ndims;
+    const int64_t n64 = t->shape[nd - 1];
+    int64_t batch = 1;
+    for (int d = 0; d < nd - 2; d++) batch *= t->shape[d];
+    if (n64 == 0 || batch == 0) return DNH_OK;
+    if (n64 > 46340 || batch > 65535) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_batched_invert: matrix size or batch too large");
+    const int n = (int)n64;
+    const int ld = (n + 3) / 4 * 4;  // rows start 16-byte aligned, which the update GEMM's vector loads need
+    const int64_t bs_w = (int64_t)n * ld, bs_g = (int64_t)n * NB, bs_t = (int64_t)NB * ld;
+
+    bool t_is_c = true;
+    {
+        int64_t expect = 1;
+        for (int d = nd - 1; d >= 0; d--) {
+            if (t->shape[d] > 1 && t->stride[d] != expect) t_is_c = false;
+            expect *= t->shape[d];
+        }
+    }
+    const size_t sz_w = align_up((size_t)batch * bs_w * sizeof(T)), sz_g = align_up((size_t)batch * bs_g * sizeof(T));
+    const size_t sz_t = align_up((size_t)batch * bs_t * sizeof(T)), sz_i = align_up((size_t)batch * n * sizeof(int32_t));
+    const size_t sz_r = t_is_c ? 0 : align_up((size_t)batch * n * n * sizeof(T));
+    void* block = nullptr;
+    DNH_TRY(dnh_alloc_async(sz_w + sz_g + sz_t + 2 * sz_i + sz_r + 256, stream, &block));
+    char* base = (char*)block;
+    T* W = (T*)base;
+    T* G = (T*)(base + sz_w);
+    T* Tb = (T*)(base + sz_w + sz_g);
+    int32_t* ipiv = (int32_t*)(base + sz_w + sz_g + sz_t);
+    int32_t* perm = (int32_t*)(base + sz_w + sz_g + sz_t + sz_i);
+    T* R = t_is_c ? (T*)elem_ptr(t) : (T*)(base + sz_w + sz_g + sz_t + 2 * sz_i);
+    int32_t* flag = (int32_t*)(base + sz_w + sz_g + sz_t + 2 * sz_i + sz_r);
+
+    int32_t st = DNH_OK;
+    auto body = [&]() -> int32_t {
+        // src (any layout, broadcast batch dimensions included) -> W, rows padded to ld
+        DnhTensor wd = *t;
+        wd.base = W;
+        wd.offset = 0;
+        int64_t acc = 1;
+        for (int d = nd - 1; d >= 0; d--) {
+            if (d == nd - 1) { wd.stride[d] = 1; acc = ld; }
+            else { wd.stride[d] = acc; acc *= t->shape[d]; }
+        }
+        DNH_TRY(dnh_copy(&wd, src, stream));
+        hipLaunchKernelGGL(invert_clear_flag_kernel, dim3(1), dim3(1), 0, stream, flag);
+        int threads = (n + 63) / 64 * 64;
+        if (threads > kMaxPanelThreads) threads = kMaxPanelThreads;
+        for (int kb = 0; kb < n; kb += NB) {
+            const int wc = (n - kb < NB) ? n - kb : NB;
+            hipLaunchKernelGGL((invert_panel_kernel<T>), dim3((unsigned)batch), dim3(threads), 0, stream, W, G, ipiv, flag, n, ld, kb, wc,
+                               bs_w, bs_g);
+            if (n > wc) {
+                hipLaunchKernelGGL((invert_swap_kernel<T>), dim3((unsigned)cdiv(n, 256), (unsigned)batch), dim3(256), 0, stream, W, Tb, ipiv, n,
+                                   ld, kb, wc, bs_w, bs_t);
+                DNH_TRY(gemm_accumulate(t->dtype, W, G, Tb, n, n, wc, NB, ld, ld, batch, bs_g, bs_t, bs_w, stream));
+            }
+        }
+        const int use_lds = (size_t)n * sizeof(int32_t) <= 48 * 1024;
+        hipLaunchKernelGGL(invert_perm_kernel, dim3((unsigned)batch), dim3(256), use_lds ? (size_t)n * sizeof(int32_t) : 0, stream, perm, ipiv,
+                           n, use_lds);
+        hipLaunchKernelGGL((invert_unpermute_kernel<T>), dim3((unsigned)cdiv(n, 256), (unsigned)n, (unsigned)batch), dim3(256), 0, stream, R, W,
+                           perm, n, ld, bs_w);
+        DNH_LAUNCH_CHECK();
+        if (!t_is_c) {
+            DnhTensor rd = *t;
+            rd.base = R;
+            rd.offset = 0;
+            int64_t a2 = 1;
+            for (int d = nd - 1; d >= 0; d--) { rd.stride[d] = a2; a2 *= t->shape[d]; }
+            DNH_TRY(dnh_copy(t, &rd, stream));
+        }
+        int32_t host_flag = 0;
+        DNH_HIP(hipMemcpyAsync(&host_flag, flag, sizeof(int32_t), hipMemcpyDeviceToHost, stream));
+        DNH_HIP(hipStreamSynchronize(stream));
+        if (host_flag) return fail(DNH_ERR_SINGULAR_MATRIX, "cannot invert singular matrix");
+        return DNH_OK;
+    };
+    st = body();
+    (void)dnh_free_async(block, stream);
+    return st;
+}
+
+}  // namespace
+
+extern "C" int32_t dnh_batched_invert(const DnhTensor* t, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    DNH_TRY(check_tensor(t, "dnh_batched_invert"));
+    DNH_TRY(check_tensor(src, "dnh_batched_invert"));
+    if (t->dtype != src->dtype) return fail(DNH_ERR_INVALID_ARG, "dnh_batched_invert: dtypes differ");
+    if (!dtype_is_fp(t->dtype))
+        return fail(DNH_ERR_NOT_SUPPORTED, "dnh_batched_invert: this operation is only supported for floating point numbers");
+    if (!same_shape(t, src)) return fail(DNH_ERR_INVALID_ARG, "dnh_batched_invert: source is not broadcast to the target's shape");
+    if (t->ndims < 2) return fail(DNH_ERR_INVALID_ARG, "dnh_batched_invert: need at least a matrix");
+    if (t->shape[t->ndims - 1] != t->shape[t->ndims - 2]) return fail(DNH_ERR_INVALID_ARG, "dnh_batched_invert: matrices are not square");
+    if (t->dtype == DNH_F32) return invert_impl<float>(t, src, (hipStream_t)stream);
+    return invert_impl<double>(t, src, (hipStream_t)stream);
+}

@@ -225,7 +225,9 @@ and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> Valu
         member this.BatchedMatMatDot (t, a, b) = dot t a b
 
         // not on the accelerated path; the CUDA backend leaves SVD and the eigen-decomposition unsupported too (CudaBackend.fs:486-492)
-        member this.BatchedInvert (trgt, src) = raise (NotSupportedException "BatchedInvert is not supported by the HIP backend")
+        member this.BatchedInvert (trgt, src) =
+            let mutable t, s = desc trgt, desc src
+            Native.check (Native.dnh_batched_invert (&t, &s, Cfg.Stream))
         member this.BatchedSVD (trgtS, trgtUV, src) = raise (NotSupportedException "BatchedSVD is not supported by the HIP backend")
         member this.SymmetricEigenDecomposition (part, eigVals, eigVecs, src) =
             raise (NotSupportedException "SymmetricEigenDecomposition is not supported by the HIP backend")

@@ -16,6 +16,7 @@ type internal Status =
     | Hip = 4
     | IndexOutOfRange = 5
     | NotInitialized = 6
+    | SingularMatrix = 7
 
 /// DnhDType — the element types the reference marshals to kernels (Cuda/NativeTensor.fs:22-34).
 type internal DType =
@@ -68,6 +69,7 @@ module internal Native =
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_masked_set (DnhTensor& t, nativeint[] masks, int nMasks, DnhTensor& src, nativeint stream)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_true_indices (DnhTensor& t, DnhTensor& src, nativeint stream)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_dot (DnhTensor& t, DnhTensor& a, DnhTensor& b, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_batched_invert (DnhTensor& t, DnhTensor& src, nativeint stream)
 
     /// Maps a status to the exception type the reference's backends raise for the same condition.
     let check (status: int) =
@@ -80,4 +82,5 @@ module internal Native =
             | Status.NotSupported -> raise (NotSupportedException msg)
             | Status.OutOfMemory -> raise (OutOfMemoryException msg)
             | Status.IndexOutOfRange -> raise (IndexOutOfRangeException msg)
+            | Status.SingularMatrix -> raise (Tensor.SingularMatrixException msg)
             | _ -> failwithf "HIP tensor backend error %d: %s" status msg

@@ -9,6 +9,9 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "libtensor_
 _lib = None
 
 
+from .backend import SingularMatrixException  # noqa: E402
+
+
 class HipError(RuntimeError):
     pass
 
@@ -72,6 +75,7 @@ _EXC = {
     abi.DNH_ERR_HIP: HipError,
     abi.DNH_ERR_INDEX_OUT_OF_RANGE: IndexError,
     abi.DNH_ERR_NOT_INITIALIZED: HipError,
+    abi.DNH_ERR_SINGULAR_MATRIX: SingularMatrixException,
 }
 
 

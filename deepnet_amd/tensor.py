@@ -546,6 +546,20 @@ class Tensor:
         else:
             raise ValueError(f"Cannot compute dot product between tensors of shapes {a.Shape} and {b.Shape} into tensor of shape {self.Shape}.")
 
+    # ---- inversion (Tensor.fs:2799-2839) ----------------------------------------------------------------------------------
+    def FillInvert(self, a: "Tensor"):
+        _same_storage([self, a])
+        if a.NDims < 2:
+            raise ValueError(f"Need at least a matrix to invert but got shape {a.Shape}.")
+        a = a.broadcastTo(self.Shape)
+        self.Backend.BatchedInvert(self, a)
+
+    @staticmethod
+    def invert(a: "Tensor") -> "Tensor":
+        trgt = Tensor.new(a.Shape, a.Dev, a.DataType)
+        trgt.FillInvert(a)
+        return trgt
+
     def __matmul__(self, b: "Tensor") -> "Tensor":
         a = self
         _same_storage([a, b])

@@ -39,7 +39,8 @@ typedef enum DnhStatus {
     DNH_ERR_OUT_OF_MEMORY = 3,    /* -> OutOfCudaMemoryException analogue (CudaUtils.fs:183-210) */
     DNH_ERR_HIP = 4,              /* -> CudaException analogue                                  */
     DNH_ERR_INDEX_OUT_OF_RANGE = 5, /* -> IndexOutOfRangeException (Host/FastAccess.fs:51-61)   */
-    DNH_ERR_NOT_INITIALIZED = 6
+    DNH_ERR_NOT_INITIALIZED = 6,
+    DNH_ERR_SINGULAR_MATRIX = 7   /* -> SingularMatrixException (Tensor.fs:2831-2834)               */
 } DnhStatus;
 
 /* Element types: the set the reference marshals to kernels (Cuda/NativeTensor.fs:22-34). bool is one byte 0/1. */
@@ -231,6 +232,12 @@ int32_t dnh_true_indices(const DnhTensor* t_i64, const DnhTensor* src_bool, void
  * (Tensor.fs:2714-2730): (0,1,1) (1,2,1) (2,2,2) or (n,n,n) with n>2.  fp32 and fp64.
  * ------------------------------------------------------------------------------------------------- */
 int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream);
+
+/* ITensorBackend.BatchedInvert (TensorBackend.fs:144; Host/HostBackend.fs:548-576 LAPACK getrf + getri;
+ * Cuda/CudaBackend.fs:451-484 getrfBatched + getriBatched).  t and src have shape [b_1..b_k; n; n] (src broadcast to
+ * t's shape by the frontend, Tensor.fs:2811-2815), single or double; any strides; t may be src.  Partial pivoting; a pivot
+ * that is exactly zero gives DNH_ERR_SINGULAR_MATRIX (LAPACK info > 0).  Synchronises the stream to read that flag. */
+int32_t dnh_batched_invert(const DnhTensor* t, const DnhTensor* src, void* stream);
 
 #ifdef __cplusplus
 }

@@ -11,6 +11,8 @@
 //   address math and index checks ...... Tensor/Tensor/Host/FastAccess.fs:41-61, 67-123
 //   which ops run single-threaded ...... Tensor/Tensor/Host/VectorOps.fs:254-301 (SIMD list), Host/HostBackend.fs:187-389
 //   dot ................................ Tensor/Tensor/Host/HostBackend.fs:463-546 (BLAS for fp32/fp64, multiply+sum otherwise)
+//   batched inversion .................. Tensor/Tensor/Host/HostBackend.fs:548-576 (LAPACK getrf + getri per matrix),
+//                                        matrix hand-over Tensor/Tensor/BlasSupport.fs:148-190
 //   special values ..................... Tensor/Tensor/TensorRng.fs:24 (NotFound)
 //
 // Pinning (what each function is checked against, see tests/test_oracle_*.py):
@@ -20,8 +22,11 @@
 //   argMax/argMin: np.argmax/argmin (first occurrence) + planted ties + NotFound rows by hand; find: brute force;
 //   gather/scatter/maskedGet/maskedSet/trueIndices: NumPy fancy indexing, np.add.at, boolean masks, np.argwhere + doc vectors;
 //   dot: fp64 matmul as truth within the stated K-term bound, doc vector, structural identities.
+//   batched inversion: the reference's own fixture (Tensor.Test/TestData/MatInv.h5, BaseTests.fs:214-233: inv(Kk).Kk = I to 1e-5),
+//     its doc example and singular-matrix test, closed forms (Hilbert, diagonal, permutation, 2x2) and A.inv(A) = I.
 //   PARITY UNPINNED at bit level (tolerance-level only): fp32 transcendental last bits (FSharp.Core + libm, not in the
-//   reference tree) and the summation order inside MKL sgemm/sdot (binary not in the reference tree).
+//   reference tree); the summation order inside MKL sgemm/sdot and the blocking inside MKL getrf/getri (binary not in the
+//   reference tree: the published unblocked LAPACK algorithms getf2 / trti2 / getri are restated).
 //
 // Build: g++ -O2 -fopenmp -ffp-contract=off (no fast-math) — every + and * rounds separately, as in the reference.
 
@@ -773,6 +778,126 @@ int32_t href_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b) {
     switch (t->dtype) { HREF_NUMERIC_CASES(MDOT) default: return DNH_ERR_NOT_SUPPORTED; }
 #undef MDOT
     return DNH_OK;
+}
+
+}  // extern "C"
+
+namespace {
+// BatchedInvert: HostBackend.fs:548-576.  The reference copies src into trgt, hands each matrix to LAPACKE_?getrf and
+// LAPACKE_?getri in column-major order and raises SingularMatrixException when either reports info > 0.  BLAS.GetMatrix
+// (BlasSupport.fs:148-190, canTranspose=true) passes a row-major matrix as the column-major matrix with the same memory, i.e.
+// LAPACK factors the transpose; a column-major matrix is passed as it is; any other layout goes through a column-major copy.
+// MKL's binary is not in the reference tree, so LAPACK's published unblocked algorithms are restated in T:
+//   getf2: for each column j, the first entry of largest magnitude at or below the diagonal becomes the pivot, rows are
+//          exchanged, the column is scaled by 1/pivot (reciprocal when |pivot| >= sfmin) and the trailing block updated;
+//   getri: inv(U) by trti2 (column by column), then inv(A).L = inv(U) solved from the last column backwards, then the
+//          row exchanges undone as column exchanges in reverse order.
+template <class T>
+int32_t invert_colmajor(T* a, int64_t n, std::vector<int64_t>& ipiv, std::vector<T>& work) {
+    auto A = [&](int64_t i, int64_t j) -> T& { return a[i + j * n]; };
+    const T sfmin = std::numeric_limits<T>::min();
+    int64_t info = 0;
+    for (int64_t j = 0; j < n; j++) {
+        int64_t jp = j;
+        T best = std::fabs(A(j, j));
+        for (int64_t i = j + 1; i < n; i++) {
+            const T v = std::fabs(A(i, j));
+            if (v > best) { best = v; jp = i; }
+        }
+        ipiv[(size_t)j] = jp;
+        if (A(jp, j) != T(0)) {
+            if (jp != j)
+                for (int64_t c = 0; c < n; c++) std::swap(A(j, c), A(jp, c));
+            if (std::fabs(A(j, j)) >= sfmin) {
+                const T r = T(1) / A(j, j);
+                for (int64_t i = j + 1; i < n; i++) A(i, j) = A(i, j) * r;
+            } else {
+                for (int64_t i = j + 1; i < n; i++) A(i, j) = A(i, j) / A(j, j);
+            }
+        } else if (info == 0) {
+            info = j + 1;
+        }
+        for (int64_t c = j + 1; c < n; c++) {
+            const T u = A(j, c);
+            for (int64_t i = j + 1; i < n; i++) A(i, c) = A(i, c) - A(i, j) * u;
+        }
+    }
+    if (info > 0) return DNH_ERR_SINGULAR_MATRIX;
+    // trti2, upper, non-unit
+    for (int64_t j = 0; j < n; j++) {
+        if (A(j, j) == T(0)) return DNH_ERR_SINGULAR_MATRIX;
+        A(j, j) = T(1) / A(j, j);
+        const T ajj = -A(j, j);
+        // x := inv(U)[0:j, 0:j] * x for x = A[0:j, j] (trmv, upper, no transpose, non-unit): columns left to right
+        for (int64_t c = 0; c < j; c++) {
+            const T temp = A(c, j);
+            if (temp != T(0)) {
+                for (int64_t i = 0; i < c; i++) A(i, j) = A(i, j) + temp * A(i, c);
+                A(c, j) = A(c, j) * A(c, c);
+            }
+        }
+        for (int64_t i = 0; i < j; i++) A(i, j) = ajj * A(i, j);
+    }
+    // inv(A) * L = inv(U), last column first
+    for (int64_t j = n - 1; j >= 0; j--) {
+        for (int64_t i = j + 1; i < n; i++) { work[(size_t)i] = A(i, j); A(i, j) = T(0); }
+        for (int64_t c = j + 1; c < n; c++) {
+            const T wv = work[(size_t)c];
+            if (wv != T(0))
+                for (int64_t i = 0; i < n; i++) A(i, j) = A(i, j) - wv * A(i, c);
+        }
+    }
+    for (int64_t j = n - 2; j >= 0; j--) {
+        const int64_t jp = ipiv[(size_t)j];
+        if (jp != j)
+            for (int64_t i = 0; i < n; i++) std::swap(A(i, j), A(i, jp));
+    }
+    return DNH_OK;
+}
+
+template <class T>
+int32_t batched_invert_t(const DnhTensor* t, const DnhTensor* s) {
+    const int nd = t->ndims;
+    const int64_t n = t->shape[nd - 1];
+    int64_t batch = 1;
+    for (int d = 0; d < nd - 2; d++) batch *= t->shape[d];
+    if (batch == 0 || n == 0) return DNH_OK;
+    const int64_t sr = t->stride[nd - 2], sc = t->stride[nd - 1];
+    // row-major (passed transposed) or column-major / copied (passed as it is)
+    const bool as_transpose = (sc == 1 && sr >= std::max<int64_t>(1, n));
+    std::vector<T> a((size_t)(n * n)), work((size_t)n);
+    std::vector<int64_t> ipiv((size_t)n);
+    T* tp = (T*)t->base;
+    const T* sp = (const T*)s->base;
+    for (int64_t b = 0; b < batch; b++) {
+        int64_t to = t->offset, so = s->offset, r = b;
+        for (int d = nd - 3; d >= 0; d--) { const int64_t p = r % t->shape[d]; r /= t->shape[d]; to += p * t->stride[d]; so += p * s->stride[d]; }
+        for (int64_t i = 0; i < n; i++)
+            for (int64_t j = 0; j < n; j++) {
+                const T v = sp[so + i * s->stride[nd - 2] + j * s->stride[nd - 1]];
+                if (as_transpose) a[(size_t)(j + i * n)] = v; else a[(size_t)(i + j * n)] = v;
+            }
+        const int32_t st = invert_colmajor<T>(a.data(), n, ipiv, work);
+        if (st != DNH_OK) return st;
+        for (int64_t i = 0; i < n; i++)
+            for (int64_t j = 0; j < n; j++)
+                tp[to + i * sr + j * sc] = as_transpose ? a[(size_t)(j + i * n)] : a[(size_t)(i + j * n)];
+    }
+    return DNH_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+int32_t href_batched_invert(const DnhTensor* t, const DnhTensor* s) {
+    if (!valid(t) || !valid(s) || t->dtype != s->dtype || t->ndims != s->ndims || t->ndims < 2) return DNH_ERR_INVALID_ARG;
+    for (int d = 0; d < t->ndims; d++)
+        if (t->shape[d] != s->shape[d]) return DNH_ERR_INVALID_ARG;
+    if (t->shape[t->ndims - 1] != t->shape[t->ndims - 2]) return DNH_ERR_INVALID_ARG;
+    if (t->dtype == DNH_F32) return batched_invert_t<float>(t, s);
+    if (t->dtype == DNH_F64) return batched_invert_t<double>(t, s);
+    return DNH_ERR_NOT_SUPPORTED;  // "this operation is only supported for floating point numbers" (HostBackend.fs:549-550)
 }
 
 }  // extern "C"

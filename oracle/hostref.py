@@ -15,7 +15,7 @@ import numpy as np
 
 from deepnet_amd import abi
 from deepnet_amd import layout as L
-from deepnet_amd.backend import CAbiTensorBackend, ITensorDevice, ITensorStorage
+from deepnet_amd.backend import CAbiTensorBackend, ITensorDevice, ITensorStorage, SingularMatrixException
 from deepnet_amd.tensor import Tensor
 
 _DIR = os.path.dirname(os.path.abspath(__file__))
@@ -47,6 +47,7 @@ _EXC = {
     abi.DNH_ERR_INVALID_ARG: ValueError,
     abi.DNH_ERR_NOT_SUPPORTED: NotImplementedError,
     abi.DNH_ERR_INDEX_OUT_OF_RANGE: IndexError,
+    abi.DNH_ERR_SINGULAR_MATRIX: SingularMatrixException,
 }
 
 

@@ -29,6 +29,7 @@ int32_t href_scatter(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_
 int32_t href_masked_get(const DnhTensor* t, const DnhTensor* s, const DnhTensor* const* masks, int32_t n_masks);
 int32_t href_true_indices(const DnhTensor* t, const DnhTensor* s);
 int32_t href_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b);
+int32_t href_batched_invert(const DnhTensor* t, const DnhTensor* s);
 }
 
 namespace tn = Tensor;
@@ -266,6 +267,17 @@ static void doc_examples() {
     expect_throws<std::invalid_argument>("doc.dot.shapeMismatch", [&] { m1.dot(TF::ofHost({1, 2, 3}, {3})); });
     expect_throws<std::invalid_argument>("doc.broadcast.mismatch", [&] { u + TF::ofHost({1, 2}, {2}); });
     expect_throws<tn::NotSupportedException>("doc.int.log.notSupported", [&] { i.un(tn::TensorHipBackend<int32_t>::Log); });
+    // invert example (Tensor.fs:2820-2825) and the singular matrix of BaseTests.fs:204-211
+    {
+        std::string why;
+        auto inv = download(tn::Tensor<double>::invert(tn::Tensor<double>::ofHost({1, 2, 3, 4}, {2, 2})));
+        std::vector<double> want{-2, 1, 1.5, -0.5};
+        bool ok = true;
+        for (int k = 0; k < 4; k++) ok = ok && std::fabs(inv[k] - want[k]) <= 2e-15;
+        report("doc.invert", ok);
+        expect_throws<tn::SingularMatrixException>("doc.invert.singular", [] { tn::Tensor<double>::invert(tn::Tensor<double>::ofHost({1, 0, 0, 1, 2, 0, 1, 0, 0}, {3, 3})); });
+        expect_throws<tn::NotSupportedException>("doc.invert.int", [] { tn::Tensor<int32_t>::invert(tn::Tensor<int32_t>::ofHost({1, 0, 0, 1}, {2, 2})); });
+    }
     // counting / convert / reshape of a transposed view copies
     EXPECT("doc.counting", download(TI::counting(5)) == (std::vector<int64_t>{0, 1, 2, 3, 4}));
     EXPECT("doc.convert", download(TF::ofHost({1.7f, -1.7f, 3.0f}, {3}).convert<int32_t>()) == (std::vector<int32_t>{1, -1, 3}));
@@ -374,6 +386,14 @@ static void oracle_parity() {
             for (size_t k = 0; ok && k < want.size(); k++) if (std::fabs(got[k] - want[k]) > 48 * 2.3e-16 * 48 * 4) { ok = false; why = "at " + std::to_string(k); }
             report("parity.f64.dot.matmat", ok, why);
         }
+    }
+    // batched inverse against the oracle's LU inverse: diagonally dominant matrices (cond < 3), |diff| <= 64 n eps max|inv|
+    {
+        HostT<float> a = randf({4, 70, 70}, -1.f, 1.f);
+        for (int b = 0; b < 4; b++) for (int i = 0; i < 70; i++) (*a.data)[(size_t)(b * 4900 + i * 71)] += 70.f;
+        HostT<float> want({4, 70, 70}); auto dw = want.desc(), da = a.desc();
+        if (href_batched_invert(&dw, &da)) std::abort();
+        check_close("parity.f32.invert.batched", tn::Tensor<float>::invert(a.toDevice()), want, 0, 64 * 70 * 1.2e-7 * 0.02);
     }
     // a second stream through Cfg::Stream
     {
