@@ -100,7 +100,7 @@ __global__ __launch_bounds__(kMaxPanelThreads) void invert_panel_kernel(T* __res
         const T sj = in_panel ? srow[jj] : T(0);
         best = T(-1);
         bi = n;
-        constexpr int U = 4;
+        constexpr int U = 16;   // loads in flight per thread: the update is bound by the latency of its cache round trips
         for (int r0 = rsub; r0 < n; r0 += rpp * U) {
             T v[U];
 #pragma unroll
@@ -130,86 +130,170 @@ __global__ __launch_bounds__(kMaxPanelThreads) void invert_panel_kernel(T* __res
             G[(int64_t)r * NB + jj] = P[(int64_t)r * ld + kb + jj] - ((r == kb + jj) ? T(1) : T(0));
 }
 
-// One thread per column outside the panel: applies the panel's row exchanges in order, then copies the block's rows to T.
-// Panel columns of T are zero so the update leaves the panel as it is.
+// The same Gauss-Jordan steps on a sub-panel of sw <= CW columns held in LDS, so that the dependent chain pivot search ->
+// exchange -> pivot row -> update runs at LDS latency instead of cache round trips.  Element (r, c) of the sub-panel lives at
+// L[r * CW + c] and is owned by thread (r % rows_per_pass) * CW + c: every access of the update is linear in the thread index,
+// the CW lanes of a row sit in one wavefront, and the row's multiplier (its entry in the pivot column) is read by all of them
+// before the owner of that column overwrites it — same wavefront, program order — so the update needs no second buffer.
+// gsub receives the sub-panel minus the identity (n x sw, row stride gld) for the update of the other columns.
+template <class T, int CW>
+__global__ __launch_bounds__(kMaxPanelThreads) void invert_subpanel_lds_kernel(T* __restrict__ w, T* __restrict__ gsub, int32_t* __restrict__ ipiv,
+                                                                               int32_t* singular, int n, int ld, int cs, int sw, int gld,
+                                                                               int64_t bs_w, int64_t bs_gs) {
+    extern __shared__ __align__(16) unsigned char lds_raw[];
+    T* P = w + (int64_t)blockIdx.x * bs_w;
+    T* Gs = gsub + (int64_t)blockIdx.x * bs_gs;
+    int32_t* piv = ipiv + (int64_t)blockIdx.x * n;
+    const int tid = threadIdx.x, nt = blockDim.x;
+    const int c = tid % CW, rsub = tid / CW, rpp = nt / CW;
+    const bool in_panel = c < sw;
+    T* L = (T*)lds_raw;
+    __shared__ T red_v[2][kMaxPanelThreads / 64];
+    __shared__ int red_i[2][kMaxPanelThreads / 64];
+    __shared__ int piv_s[NB];   // pivots go to memory once, at the end: a barrier waits for the stores issued before it
+    {
+        // sixteen loads in flight per thread: a single workgroup fetches the whole sub-panel, so the fetch is latency-bound
+        constexpr int UL = 16;
+        for (int r0 = rsub; r0 < n; r0 += UL * rpp) {
+            T v[UL];
+#pragma unroll
+            for (int u = 0; u < UL; u++) {
+                const int r = r0 + u * rpp;
+                v[u] = (in_panel && r < n) ? P[(int64_t)r * ld + cs + c] : T(0);
+            }
+#pragma unroll
+            for (int u = 0; u < UL; u++) {
+                const int r = r0 + u * rpp;
+                if (r < n) L[r * CW + c] = v[u];
+            }
+        }
+    }
+    __syncthreads();
+    T best = T(-1);
+    int bi = n;
+    for (int r = cs + tid; r < n; r += nt) {
+        const T v = abs_of(L[r * CW]);
+        if (v > best) { best = v; bi = r; }
+    }
+    for (int j = 0; j < sw; j++) {
+        const int col = cs + j;
+        block_arg_max(best, bi, red_v[j & 1], red_i[j & 1]);
+        int p = bi;
+        if (!(best > T(0))) {
+            p = col;
+            if (tid == 0) *singular = 1;
+        }
+        if (tid == 0) piv_s[j] = p;
+        if (p != col && tid < CW) {
+            const T t = L[col * CW + tid];
+            L[col * CW + tid] = L[p * CW + tid];
+            L[p * CW + tid] = t;
+        }
+        __syncthreads();
+        const T sj = (c == j ? T(1) : L[col * CW + c]) / L[col * CW + j];   // my column's entry of the scaled pivot row
+        __syncthreads();                                                    // everyone has read the pivot row before it changes
+        best = T(-1);
+        bi = n;
+        const bool is_pivot_col = c == j, is_next_col = c == j + 1;
+        // four rows per round: all reads of a round are issued before its writes (the rows of a round are distinct, and the
+        // lanes of a row read its multiplier before the owner of the pivot column overwrites it)
+        constexpr int U = 4;
+        for (int r0 = rsub; r0 < n; r0 += U * rpp) {
+            T v[U], f[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int r = r0 + u * rpp;
+                if (r < n) { v[u] = L[r * CW + c]; f[u] = L[r * CW + j]; }
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int r = r0 + u * rpp;
+                if (r < n) {
+                    const T nv = (r == col) ? sj : (is_pivot_col ? T(0) : v[u]) - f[u] * sj;
+                    L[r * CW + c] = nv;
+                    if (is_next_col && r > col) {   // the next column's pivot candidates, rows ascending per thread
+                        const T a = abs_of(nv);
+                        if (a > best) { best = a; bi = r; }
+                    }
+                }
+            }
+        }
+        __syncthreads();
+    }
+    if (tid < sw) piv[cs + tid] = piv_s[tid];
+    if (in_panel)
+        for (int r = rsub; r < n; r += rpp) {
+            const T v = L[r * CW + c];
+            P[(int64_t)r * ld + cs + c] = v;
+            Gs[(int64_t)r * gld + c] = v - ((r == cs + c) ? T(1) : T(0));
+        }
+}
+
+// G - I_block of a panel that was processed in sub-panels.
 template <class T>
-__global__ __launch_bounds__(256) void invert_swap_kernel(T* __restrict__ w, T* __restrict__ tbuf, const int32_t* __restrict__ ipiv, int n,
-                                                          int ld, int kb, int wc, int64_t bs_w, int64_t bs_t) {
-    const int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= n) return;
+__global__ __launch_bounds__(256) void invert_extract_g_kernel(const T* __restrict__ w, T* __restrict__ gbuf, int n, int ld, int kb, int wc,
+                                                               int64_t bs_w, int64_t bs_g) {
+    const int idx = blockIdx.x * 256 + threadIdx.x;
+    if (idx >= n * wc) return;
+    const int r = idx / wc, c = idx - r * wc;
+    gbuf[(int64_t)blockIdx.y * bs_g + (int64_t)r * NB + c] = w[(int64_t)blockIdx.y * bs_w + (int64_t)r * ld + kb + c] - ((r == kb + c) ? T(1) : T(0));
+}
+
+// One thread per column in [c_begin, c_end) outside the block's own columns [kb, kb + wc): applies the block's row exchanges in
+// order, then copies the block's rows to T.  The block's own columns of T are zero so the update leaves them as they are.
+// The exchanges are first replayed on row numbers (thread 0, at most 2 * NB rows take part: the block's rows and their
+// partners), which gives for every affected row the row its final content comes from; the columns then see one round of
+// independent loads and one round of stores instead of wc dependent round trips.
+constexpr int kSwapThreads = 64;
+template <class T>
+__global__ __launch_bounds__(kSwapThreads) void invert_swap_kernel(T* __restrict__ w, T* __restrict__ tbuf, const int32_t* __restrict__ ipiv,
+                                                                   int n, int ld, int kb, int wc, int c_begin, int c_end, int64_t bs_w,
+                                                                   int64_t bs_t) {
+    __shared__ int pos[2 * NB];   // affected row positions: the block's rows first, then partners outside the block
+    __shared__ int src[2 * NB];   // the row whose content ends up at pos[i]
+    __shared__ int pv[NB];
+    __shared__ int cnt;
+    const int32_t* piv = ipiv + (int64_t)blockIdx.y * n;
+    if (threadIdx.x < wc) pv[threadIdx.x] = piv[kb + threadIdx.x];
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int m = wc;
+        for (int j = 0; j < wc; j++) { pos[j] = kb + j; src[j] = kb + j; }
+        for (int j = 0; j < wc; j++) {
+            const int p = pv[j];
+            if (p == kb + j) continue;
+            int ip = -1;
+            if (p < kb + wc) {
+                ip = p - kb;
+            } else {
+                for (int q = wc; q < m; q++)
+                    if (pos[q] == p) { ip = q; break; }
+                if (ip < 0) { ip = m; pos[m] = p; src[m] = p; m++; }
+            }
+            const int t = src[j]; src[j] = src[ip]; src[ip] = t;
+        }
+        cnt = m;
+    }
+    __syncthreads();
+    const int c = c_begin + blockIdx.x * kSwapThreads + threadIdx.x;
+    if (c >= c_end) return;
     T* P = w + (int64_t)blockIdx.y * bs_w;
     T* Tb = tbuf + (int64_t)blockIdx.y * bs_t;
-    const int32_t* piv = ipiv + (int64_t)blockIdx.y * n;
     if (c >= kb && c < kb + wc) {
         for (int j = 0; j < wc; j++) Tb[(int64_t)j * ld + c] = T(0);
         return;
     }
-    // the rows that take part: the block's own rows and the rows they were exchanged with.  The exchanges are replayed on
-    // registers, so memory sees one round of loads and one round of stores instead of wc dependent round trips.
-    T own[NB], other[NB];
-    int prow[NB];
+    const int m = cnt;
+    T val[2 * NB];
 #pragma unroll
-    for (int j = 0; j < NB; j++) {
-        if (j < wc) {
-            prow[j] = piv[kb + j];
-            own[j] = P[(int64_t)(kb + j) * ld + c];
-            other[j] = P[(int64_t)prow[j] * ld + c];
+    for (int i = 0; i < 2 * NB; i++)
+        if (i < m) val[i] = P[(int64_t)src[i] * ld + c];
+#pragma unroll
+    for (int i = 0; i < 2 * NB; i++)
+        if (i < m) {
+            if (src[i] != pos[i]) P[(int64_t)pos[i] * ld + c] = val[i];
+            if (i < wc) Tb[(int64_t)i * ld + c] = val[i];
         }
-    }
-    // replay: position kb+j <-> position prow[j].  A position outside the block may appear several times in prow, and a
-    // position inside the block may be the partner of an earlier step; track values by position.
-#pragma unroll
-    for (int j = 0; j < NB; j++) {
-        if (j < wc) {
-            const int p = prow[j];
-            if (p != kb + j) {
-                // current value at position p: inside the block -> own[p-kb]; outside -> the latest copy among other[]
-                if (p < kb + wc) {
-                    const T t = own[j];
-#pragma unroll
-                    for (int q = 0; q < NB; q++)
-                        if (q == p - kb) { own[j] = own[q]; own[q] = t; }
-                } else {
-                    // find the first slot that represents position p (the canonical holder of its current value)
-                    int holder = j;
-#pragma unroll
-                    for (int q = NB - 1; q >= 0; q--)
-                        if (q < j && prow[q] == p) holder = q;
-                    T cur;
-                    cur = other[j];
-#pragma unroll
-                    for (int q = 0; q < NB; q++)
-                        if (q == holder) cur = other[q];
-                    const T t = own[j];
-                    own[j] = cur;
-#pragma unroll
-                    for (int q = 0; q < NB; q++)
-                        if (q == holder) other[q] = t;
-                }
-            }
-        }
-    }
-    // write back: block rows, then every outside position once (from its canonical holder)
-#pragma unroll
-    for (int j = 0; j < NB; j++) {
-        if (j < wc) {
-            P[(int64_t)(kb + j) * ld + c] = own[j];
-            Tb[(int64_t)j * ld + c] = own[j];
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < NB; j++) {
-        if (j < wc) {
-            const int p = prow[j];
-            if (p >= kb + wc) {
-                bool first = true;
-#pragma unroll
-                for (int q = 0; q < NB; q++)
-                    if (q < j && prow[q] == p) first = false;
-                if (first) P[(int64_t)p * ld + c] = other[j];
-            }
-        }
-    }
 }
 
 // Composes the column permutation that undoes the row exchanges: exchanges are applied to columns in reverse order.
@@ -270,7 +354,7 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
     const size_t sz_t = align_up((size_t)batch * bs_t * sizeof(T)), sz_i = align_up((size_t)batch * n * sizeof(int32_t));
     const size_t sz_r = t_is_c ? 0 : align_up((size_t)batch * n * n * sizeof(T));
     void* block = nullptr;
-    DNH_TRY(dnh_alloc_async(sz_w + sz_g + sz_t + 2 * sz_i + sz_r + 256, stream, &block));
+    DNH_TRY(dnh_alloc_async(sz_w + 2 * sz_g + sz_t + 2 * sz_i + sz_r + 256, stream, &block));
     char* base = (char*)block;
     T* W = (T*)base;
     T* G = (T*)(base + sz_w);
@@ -279,6 +363,7 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
     int32_t* perm = (int32_t*)(base + sz_w + sz_g + sz_t + sz_i);
     T* R = t_is_c ? (T*)elem_ptr(t) : (T*)(base + sz_w + sz_g + sz_t + 2 * sz_i);
     int32_t* flag = (int32_t*)(base + sz_w + sz_g + sz_t + 2 * sz_i + sz_r);
+    T* Gs = (T*)(base + sz_w + sz_g + sz_t + 2 * sz_i + sz_r + 256);   // sub-panel multipliers (n x sb per matrix, sb <= NB)
 
     int32_t st = DNH_OK;
     auto body = [&]() -> int32_t {
@@ -295,13 +380,54 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
         hipLaunchKernelGGL(invert_clear_flag_kernel, dim3(1), dim3(1), 0, stream, flag);
         int threads = (n + 63) / 64 * 64;
         if (threads > kMaxPanelThreads) threads = kMaxPanelThreads;
+        // widest sub-panel (a power of two <= NB) whose rows fit in the LDS a workgroup may use; 0 = none fits
+        int lds_limit = 0, dev = 0;
+        DNH_HIP(hipGetDevice(&dev));
+        DNH_HIP(hipDeviceGetAttribute(&lds_limit, hipDeviceAttributeMaxSharedMemoryPerBlock, dev));
+        auto lds_need = [&](int cw) { return (size_t)n * cw * sizeof(T); };
+        int sb = 0;
+        for (int cand = NB; cand >= 1; cand >>= 1)
+            if (lds_need(cand) + 1024 <= (size_t)lds_limit) { sb = cand; break; }
+        auto launch_subpanel = [&](int cw, T* g, int cs, int sw, int gld) -> int32_t {
+            const size_t lds = lds_need(cw);
+#define DNH_SUBPANEL(CWV)                                                                                                              \
+    case CWV:                                                                                                                          \
+        if (lds > 32 * 1024)                                                                                                           \
+            DNH_HIP(hipFuncSetAttribute((const void*)invert_subpanel_lds_kernel<T, CWV>, hipFuncAttributeMaxDynamicSharedMemorySize,  \
+                                        (int)lds));                                                                                    \
+        hipLaunchKernelGGL((invert_subpanel_lds_kernel<T, CWV>), dim3((unsigned)batch), dim3(threads), lds, stream, W, g, ipiv, flag, n, ld, \
+                           cs, sw, gld, bs_w, bs_g);                                                                                   \
+        break;
+            switch (cw) {
+                DNH_SUBPANEL(32) DNH_SUBPANEL(16) DNH_SUBPANEL(8) DNH_SUBPANEL(4) DNH_SUBPANEL(2) DNH_SUBPANEL(1)
+            }
+#undef DNH_SUBPANEL
+            return DNH_OK;
+        };
         for (int kb = 0; kb < n; kb += NB) {
             const int wc = (n - kb < NB) ? n - kb : NB;
-            hipLaunchKernelGGL((invert_panel_kernel<T>), dim3((unsigned)batch), dim3(threads), 0, stream, W, G, ipiv, flag, n, ld, kb, wc,
-                               bs_w, bs_g);
+            if (sb == NB) {
+                DNH_TRY(launch_subpanel(NB, G, kb, wc, NB));
+            } else if (sb > 0) {
+                for (int cs = kb; cs < kb + wc; cs += sb) {
+                    const int sw = (kb + wc - cs < sb) ? kb + wc - cs : sb;
+                    DNH_TRY(launch_subpanel(sb, Gs, cs, sw, sb));
+                    if (wc > sw) {
+                        // the sub-panel's steps applied to the panel's other columns
+                        hipLaunchKernelGGL((invert_swap_kernel<T>), dim3(1, (unsigned)batch), dim3(kSwapThreads), 0, stream, W, Tb, ipiv, n, ld,
+                                           cs, sw, kb, kb + wc, bs_w, bs_t);
+                        DNH_TRY(gemm_accumulate(t->dtype, W + kb, Gs, Tb + kb, n, wc, sw, sb, ld, ld, batch, bs_g, bs_t, bs_w, stream));
+                    }
+                }
+                hipLaunchKernelGGL((invert_extract_g_kernel<T>), dim3((unsigned)cdiv((int64_t)n * wc, 256), (unsigned)batch), dim3(256), 0, stream,
+                                   W, G, n, ld, kb, wc, bs_w, bs_g);
+            } else {
+                hipLaunchKernelGGL((invert_panel_kernel<T>), dim3((unsigned)batch), dim3(threads), 0, stream, W, G, ipiv, flag, n, ld, kb, wc,
+                                   bs_w, bs_g);
+            }
             if (n > wc) {
-                hipLaunchKernelGGL((invert_swap_kernel<T>), dim3((unsigned)cdiv(n, 256), (unsigned)batch), dim3(256), 0, stream, W, Tb, ipiv, n,
-                                   ld, kb, wc, bs_w, bs_t);
+                hipLaunchKernelGGL((invert_swap_kernel<T>), dim3((unsigned)cdiv(n, kSwapThreads), (unsigned)batch), dim3(kSwapThreads), 0, stream,
+                                   W, Tb, ipiv, n, ld, kb, wc, 0, n, bs_w, bs_t);
                 DNH_TRY(gemm_accumulate(t->dtype, W, G, Tb, n, n, wc, NB, ld, ld, batch, bs_g, bs_t, bs_w, stream));
             }
         }
