@@ -36,7 +36,7 @@ struct GemmArgs {
     uint32_t accumulate;                          // 1: c += a.b (used by the blocked matrix inversion), 0: c = a.b
 };
 
-template <class T, bool FAST>
+template <class T, bool FAST, bool ACC>
 __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, const T* __restrict__ a, const T* __restrict__ b, GemmArgs g) {
     constexpr int BK = kBK<T>;
     __shared__ T As[2][BK][BM + PAD];
@@ -195,7 +195,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
                     const int64_t n = n0 + wn + j * 32 + lm;
                     if (full_mn || (m < g.M && n < g.N)) {
                         T* dst = c + m * g.scm + n * g.scn;
-                        *dst = g.accumulate ? *dst + acc[i][j][r] : acc[i][j][r];
+                        *dst = ACC ? *dst + acc[i][j][r] : acc[i][j][r];
                     }
                 }
     } else {
@@ -243,7 +243,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_kernel(T* __restrict__ c, cons
                     const int64_t m = m0 + wm + i * 16 + 4 * r + lk, n = n0 + wn + j * 16 + lm;
                     if (full_mn || (m < g.M && n < g.N)) {
                         T* dst = c + m * g.scm + n * g.scn;
-                        *dst = g.accumulate ? *dst + acc[i][j][r] : acc[i][j][r];
+                        *dst = ACC ? *dst + acc[i][j][r] : acc[i][j][r];
                     }
                 }
     }
@@ -259,8 +259,13 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
     bool fast = g.sak == 1 && g.sbn == 1 && g.K > 0 &&
                 (g.sam % V) == 0 && (g.sbk % V) == 0 && aligned_to(a, 16) && aligned_to(b, 16);
     for (int d = 0; d < g.nbatch && fast; d++) fast = (g.bsa[d] % V) == 0 && (g.bsb[d] % V) == 0;
-    if (fast) hipLaunchKernelGGL((gemm_kernel<T, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
-    else hipLaunchKernelGGL((gemm_kernel<T, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+    if (g.accumulate) {
+        if (fast) hipLaunchKernelGGL((gemm_kernel<T, true, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+        else hipLaunchKernelGGL((gemm_kernel<T, false, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+    } else {
+        if (fast) hipLaunchKernelGGL((gemm_kernel<T, true, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+        else hipLaunchKernelGGL((gemm_kernel<T, false, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+    }
     DNH_LAUNCH_CHECK();
     return DNH_OK;
 }
