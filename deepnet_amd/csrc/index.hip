@@ -361,19 +361,37 @@ __global__ __launch_bounds__(kBlock) void compact_move_fast_kernel(const uint8_t
     uint64_t total;
     const uint64_t pre = block_exclusive_scan64(packed, &total);
     uint32_t seg_base = PREFIXED ? block_base[blockIdx.x] : block_sum_before(block_base, blockIdx.x);
+    if constexpr (!SET && sizeof(W) >= 4) {
+        // masked get: the block's selected elements are gathered in LDS at their rank inside the block and leave as one
+        // contiguous run, so every store instruction of a wavefront writes 64 consecutive elements
+        __shared__ W stage[kFastJ * kBlock * VEC];
+        uint32_t lbase = 0;
 #pragma unroll
-    for (int j = 0; j < kFastJ; j++) {
-        uint32_t k = seg_base + (uint32_t)((pre >> (16 * j)) & 0xFFFF);
-        seg_base += (uint32_t)((total >> (16 * j)) & 0xFFFF);
-        const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+        for (int j = 0; j < kFastJ; j++) {
+            uint32_t k = lbase + (uint32_t)((pre >> (16 * j)) & 0xFFFF);
+            lbase += (uint32_t)((total >> (16 * j)) & 0xFFFF);
 #pragma unroll
-        for (int e = 0; e < VEC; e++) {
-            if (flags[j] & (1u << e)) {
-                if (k < nout) {
-                    if constexpr (SET) full[(size_t)v * VEC + e] = out[k];
-                    else out[k] = data[j].v[e];
+            for (int e = 0; e < VEC; e++)
+                if (flags[j] & (1u << e)) stage[k++] = data[j].v[e];
+        }
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < lbase; i += kBlock)
+            if (seg_base + i < nout) out[seg_base + i] = stage[i];
+    } else {
+#pragma unroll
+        for (int j = 0; j < kFastJ; j++) {
+            uint32_t k = seg_base + (uint32_t)((pre >> (16 * j)) & 0xFFFF);
+            seg_base += (uint32_t)((total >> (16 * j)) & 0xFFFF);
+            const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                if (flags[j] & (1u << e)) {
+                    if (k < nout) {
+                        if constexpr (SET) full[(size_t)v * VEC + e] = out[k];
+                        else out[k] = data[j].v[e];
+                    }
+                    k++;
                 }
-                k++;
             }
         }
     }

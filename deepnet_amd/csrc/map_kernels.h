@@ -30,21 +30,40 @@ struct Pack {
     T v[N];
 };
 
+// packs wider than 16 bytes move as consecutive 16-byte words
 template <class T, int N>
 __device__ __forceinline__ Pack<T, N> load_pack(const T* p) {
-    using W = typename RawWord<sizeof(T) * N>::type;
-    W w = __builtin_nontemporal_load((const W*)p);
     Pack<T, N> r;
-    __builtin_memcpy(&r, &w, sizeof(w));
+    if constexpr (sizeof(T) * N <= 16) {
+        using W = typename RawWord<sizeof(T) * N>::type;
+        W w = __builtin_nontemporal_load((const W*)p);
+        __builtin_memcpy(&r, &w, sizeof(w));
+    } else {
+        using W = typename RawWord<16>::type;
+        constexpr int NW = (int)(sizeof(T) * N / 16);
+        W w[NW];
+#pragma unroll
+        for (int i = 0; i < NW; i++) w[i] = __builtin_nontemporal_load((const W*)p + i);
+        __builtin_memcpy(&r, w, sizeof(w));
+    }
     return r;
 }
 
 template <class T, int N>
 __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& r) {
-    using W = typename RawWord<sizeof(T) * N>::type;
-    W w;
-    __builtin_memcpy(&w, &r, sizeof(w));
-    __builtin_nontemporal_store(w, (W*)p);
+    if constexpr (sizeof(T) * N <= 16) {
+        using W = typename RawWord<sizeof(T) * N>::type;
+        W w;
+        __builtin_memcpy(&w, &r, sizeof(w));
+        __builtin_nontemporal_store(w, (W*)p);
+    } else {
+        using W = typename RawWord<16>::type;
+        constexpr int NW = (int)(sizeof(T) * N / 16);
+        W w[NW];
+        __builtin_memcpy(w, &r, sizeof(w));
+#pragma unroll
+        for (int i = 0; i < NW; i++) __builtin_nontemporal_store(w[i], (W*)p + i);
+    }
 }
 
 template <class T, int N>
@@ -354,7 +373,9 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
         for (int k = 1; k < NOPS; k++)
             if (p.stride[k][0] == 1) al = al && aligned_to(p.ptr[k], VEC * es[k]);
         if (al) {
-            // one 16-byte vector per thread: measured fastest on MI355X (more per-thread unrolling lowers achieved bandwidth)
+            // one 16-byte vector per thread: measured fastest on MI355X (more per-thread unrolling lowers achieved bandwidth; for
+            // narrowing ops such as int32 -> bool compares, four consecutive loads per thread to reach a 16-byte store measured
+            // 25 % slower: each load instruction then uses only 32 bytes of every 128-byte line it touches)
             constexpr int UNROLL = 1;
             const int64_t nvec = p.total / VEC;
             const unsigned blocks = nvec ? cdiv(nvec, (int64_t)kBlock * UNROLL) : 1;
