@@ -39,8 +39,8 @@ struct GemmArgs {
 template <class T, bool FAST, bool ACC>
 __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void gemm_kernel(T* __restrict__ c, const T* __restrict__ a, const T* __restrict__ b, GemmArgs g) {
     constexpr int BK = kBK<T>;
-    __shared__ T As[2][BK][BM + PAD];
-    __shared__ T Bs[2][BK][BN + PAD];
+    __shared__ __align__(16) T As[2][BK][BM + PAD];
+    __shared__ __align__(16) T Bs[2][BK][BN + PAD];
 
     // XCD-aware tile order: consecutive workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Remapping
     // id -> (id % 8) * (total / 8) + id / 8 hands every XCD one contiguous range of tiles, so the tiles of one matrix pair
@@ -163,8 +163,13 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
             for (int i = 0; i < APT; i++) {
                 const int idx = tid + i * kBlock;
                 const int kk = idx / NV, nv = (idx % NV) * V;
+                // one 16-byte LDS store (element stores of this pattern collide four ways on the banks)
+                Pack<T, V> v;
 #pragma unroll
-                for (int e = 0; e < V; e++) Bs[buf][kk][nv + e] = rb[i * V + e];
+                for (int e = 0; e < V; e++) v.v[e] = rb[i * V + e];
+                typename RawWord<16>::type w;
+                __builtin_memcpy(&w, &v, 16);
+                *reinterpret_cast<typename RawWord<16>::type*>(&Bs[buf][kk][nv]) = w;
             }
         } else if (!LEAN && where == kScalar) {
 #pragma unroll
