@@ -94,12 +94,14 @@ Dev = TensorHostRefDevice()
 
 def ofNumpy(arr: np.ndarray) -> Tensor:
     """Row-major host tensor holding a copy of `arr`."""
+    arr = np.asarray(arr)
+    shape = arr.shape                       # np.ascontiguousarray turns a 0-d array into shape (1,)
     arr = np.ascontiguousarray(arr)
     flat = arr.reshape(-1).copy()
     if flat.size == 0:
         flat = np.zeros(1, dtype=arr.dtype)
     st = TensorHostRefStorage(arr.size, arr.dtype, Dev, flat)
-    return Tensor(L.newC(arr.shape), st)
+    return Tensor(L.newC(shape), st)
 
 
 def toNumpy(t: Tensor) -> np.ndarray:

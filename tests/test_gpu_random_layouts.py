@@ -1,0 +1,126 @@
+"""Differential test over seeded random shapes and views: the same frontend call sequence on the oracle device and on the GPU,
+integer element types so every comparison is bit-exact.  Views are built from permutations, slices, reversed axes, inserted and
+broadcast axes; extents include 1 and ragged sizes around the vector widths and tile edges of the kernels."""
+import numpy as np
+import pytest
+
+from deepnet_amd.tensor import Tensor
+from util import assert_exact
+
+pytestmark = pytest.mark.gpu
+
+EXTENTS = [1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 31, 33, 63, 64, 65, 127, 130, 257]
+
+
+def random_view(rng, t):
+    """A random view of tensor t (same on both devices because only layout operations are applied)."""
+    nd = t.NDims
+    if nd >= 2 and rng.random() < 0.6:
+        perm = list(rng.permutation(nd))
+        t = t.permuteAxes([int(p) for p in perm])
+    for ax in range(t.NDims):
+        r = rng.random()
+        n = t.Shape[ax]
+        if r < 0.25 and n > 2:
+            lo = int(rng.integers(0, n // 2))
+            hi = int(rng.integers(lo + 1, n + 1))
+            key = [slice(None)] * t.NDims
+            key[ax] = slice(lo, hi)
+            t = t[tuple(key)]
+        elif r < 0.4 and n > 1:
+            t = t.reverseAxis(ax)
+    return t
+
+
+def make_operands(rng, H, G, dtype, max_elems=200_000):
+    nd = int(rng.integers(0, 5))
+    shape = []
+    total = 1
+    for _ in range(nd):
+        e = int(rng.choice(EXTENTS))
+        if total * e > max_elems:
+            e = 1
+        shape.append(e)
+        total *= e
+    info = np.iinfo(dtype) if np.dtype(dtype).kind in "iu" else None
+    lo, hi = (max(info.min, -1000), min(info.max, 1000)) if info else (0, 1)
+    a = rng.integers(lo, hi + 1, size=shape).astype(dtype) if info else (rng.random(shape) < 0.5)
+    return a
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_views_elementwise_and_folds(H, G, seed):
+    rng = np.random.default_rng(1000 + seed)
+    for case in range(25):
+        dtype = [np.int32, np.int64, np.uint8, np.int8][int(rng.integers(0, 4))]
+        a_np = make_operands(rng, H, G, dtype)
+        b_np = rng.integers(-50, 50, size=a_np.shape).astype(dtype) if dtype != np.uint8 else rng.integers(0, 100, size=a_np.shape).astype(dtype)
+        state = rng.bit_generator.state
+        outs = []
+        for M in (H, G):
+            rng.bit_generator.state = state                      # identical random choices on both devices
+            a = random_view(rng, M.ofNumpy(a_np))
+            # b: same shape as the view of a, possibly with broadcast axes
+            b_full = M.ofNumpy(b_np)
+            b = b_full
+            # bring b to a's view shape by replaying a compatible construction: copy a's view of b_np's layout
+            b = b.Relayout(type(a.Layout)(a.Layout.Shape, a.Layout.Offset, a.Layout.Stride)) if b_np.shape == a_np.shape else b
+            r = []
+            r.append(M.toNumpy(a + b))
+            r.append(M.toNumpy(a * b - a))
+            r.append(M.toNumpy(a > b))
+            r.append(M.toNumpy(Tensor.ifThenElse(a > b, a, b)))
+            r.append(M.toNumpy(a.Copy()))
+            r.append(M.toNumpy(Tensor.maxElemwise(a, b)))
+            if a.NDims >= 1:
+                ax = int(rng.integers(0, a.NDims))
+                r.append(M.toNumpy(a.sumAxis(ax)))
+                r.append(M.toNumpy(a.maxAxis(ax)))
+                r.append(M.toNumpy(a.argMaxAxis(ax)))
+                r.append(M.toNumpy(a.argMinAxis(ax)))
+                r.append(M.toNumpy((a > b).countTrueAxis(ax)))
+                r.append(M.toNumpy(a.findAxis(dtype(3), ax)))
+                if a.Shape[ax] > 1 and rng.random() < 0.5:         # broadcast operand along one axis
+                    col = a.sumAxis(ax).insertAxis(ax)
+                    r.append(M.toNumpy(a - col))
+            if a.NElems > 0:
+                r.append(M.toNumpy(a.convert(np.int64)))
+                m = a > b
+                r.append(M.toNumpy(a.flatten().M(m.flatten())))
+                r.append(M.toNumpy(m.trueIdx()))
+            outs.append(r)
+        assert len(outs[0]) == len(outs[1])
+        for k, (ref, got) in enumerate(zip(*outs)):
+            try:
+                assert_exact(ref, got)
+            except AssertionError as e:
+                raise AssertionError(f"seed {seed} case {case} result {k} dtype {np.dtype(dtype)} shape {a_np.shape}: {e}") from None
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_gather_scatter(H, G, seed):
+    rng = np.random.default_rng(2000 + seed)
+    for case in range(15):
+        nd = int(rng.integers(1, 4))
+        shape = [int(rng.choice([1, 3, 8, 17, 64, 100])) for _ in range(nd)]
+        src_np = rng.integers(-1000, 1000, size=shape).astype(np.int32)
+        ishape = [int(rng.choice([1, 5, 33, 200])) for _ in range(int(rng.integers(1, 3)))]
+        use = [bool(rng.random() < 0.7) for _ in range(nd)]
+        if not any(use):
+            use[0] = True
+        # unspecified dimensions take the target position, so the index shape must cover them: pad the index shape to rank nd
+        full_ishape = ([1] * (nd - len(ishape)) + ishape)[-nd:] if len(ishape) <= nd else ishape[-nd:]
+        for d in range(nd):
+            if not use[d]:
+                full_ishape[d] = min(full_ishape[d], shape[d]) if full_ishape[d] > shape[d] else full_ishape[d]
+                full_ishape[d] = shape[d] if full_ishape[d] > shape[d] else full_ishape[d]
+        idx_np = [rng.integers(0, shape[d], size=full_ishape).astype(np.int64) if use[d] else None for d in range(nd)]
+        outs = []
+        for M in (H, G):
+            src = M.ofNumpy(src_np)
+            idx = [M.ofNumpy(i) if i is not None else None for i in idx_np]
+            g = Tensor.gather(idx, src)
+            s = Tensor.scatter(idx, shape, g)
+            outs.append([M.toNumpy(g), M.toNumpy(s)])
+        for ref, got in zip(*outs):
+            assert_exact(ref, got)
