@@ -124,3 +124,42 @@ def test_random_gather_scatter(H, G, seed):
             outs.append([M.toNumpy(g), M.toNumpy(s)])
         for ref, got in zip(*outs):
             assert_exact(ref, got)
+
+
+@pytest.mark.parametrize("seed", range(16))
+def test_random_views_float(H, G, seed):
+    """fp32 / fp64: exactly rounded operations, comparisons, max/min and arg folds are bit-exact; sums within (n + 64) u S."""
+    rng = np.random.default_rng(3000 + seed)
+    for case in range(20):
+        dtype = [np.float32, np.float64][int(rng.integers(0, 2))]
+        shape = list(make_operands(rng, H, G, np.int32).shape)
+        a_np = rng.standard_normal(shape).astype(dtype)
+        b_np = (rng.standard_normal(shape) + 3.0).astype(dtype)
+        if rng.random() < 0.3 and a_np.size:                       # planted ties and infinities
+            a_np.flat[rng.integers(0, a_np.size, size=max(1, a_np.size // 7))] = dtype(1.5)
+            a_np.flat[rng.integers(0, a_np.size)] = -np.inf
+        state = rng.bit_generator.state
+        outs, sums = [], []
+        for M in (H, G):
+            rng.bit_generator.state = state
+            a = random_view(rng, M.ofNumpy(a_np))
+            b = M.ofNumpy(b_np).Relayout(type(a.Layout)(a.Layout.Shape, a.Layout.Offset, a.Layout.Stride))
+            r = [M.toNumpy(a + b), M.toNumpy(a * b), M.toNumpy(a / b), M.toNumpy(a - b), M.toNumpy(a > b), M.toNumpy(a.abs().sqrt()),
+                 M.toNumpy(Tensor.minElemwise(a, b)), M.toNumpy(Tensor.ifThenElse(a < b, a, b)), M.toNumpy(-a), M.toNumpy(a.floor()),
+                 M.toNumpy(a.round()), M.toNumpy(a.sgn()), M.toNumpy(a.isFinite())]
+            s = []
+            if a.NDims >= 1:
+                ax = int(rng.integers(0, a.NDims))
+                r += [M.toNumpy(a.maxAxis(ax)), M.toNumpy(a.minAxis(ax)), M.toNumpy(a.argMaxAxis(ax)), M.toNumpy(a.argMinAxis(ax))]
+                s = [M.toNumpy(b.sumAxis(ax)), M.toNumpy(b.abs().sumAxis(ax)), b.Shape[ax]]      # b holds no infinities
+            outs.append(r)
+            sums.append(s)
+        for k, (ref, got) in enumerate(zip(*outs)):
+            try:
+                assert_exact(ref, got)
+            except AssertionError as e:
+                raise AssertionError(f"seed {seed} case {case} result {k} dtype {np.dtype(dtype)} shape {a_np.shape}: {e}") from None
+        if sums[0]:
+            ref, got, S, n = sums[0][0], sums[1][0], sums[0][1], sums[0][2]
+            u = 2.0 ** -24 if dtype == np.float32 else 2.0 ** -53
+            assert np.all(np.abs(ref.astype(np.float64) - got.astype(np.float64)) <= (n + 64) * u * S.astype(np.float64))
