@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """bench.py — headline benchmark of the HIP tensor backend on one MI355X.
 
-Metric (BASELINE.json): achieved HBM GB/s (% of peak) for fp32 element-wise + axis-reduce at 64 Mi elements.
+Metric: achieved HBM GB/s (% of peak) for fp32 element-wise + axis-reduce at 64 Mi elements.
 
 A "step" is one pass of the hot path over one batch of synthetic fp32 tensors of 8192 x 8192 = 67 108 864 elements
 already resident in HBM: Add and Tanh (element-wise) and Sum / Max / ArgMax along the last axis and along the first
