@@ -84,6 +84,8 @@ __device__ __forceinline__ typename Op::T apply_op(const Op& op, typename Op::A 
 
 // ---- flat ---------------------------------------------------------------------------------------------------------------
 
+constexpr uint32_t kXcdRun = 64;
+
 template <class Op, int VEC, int UNROLL>
 __global__ __launch_bounds__(kBlock) void map_flat_kernel(Op op, typename Op::T* __restrict__ t, const typename Op::A* a,
                                                           const typename Op::B* b, const typename Op::C* c, int sa, int sb, int sc,
@@ -93,7 +95,18 @@ __global__ __launch_bounds__(kBlock) void map_flat_kernel(Op op, typename Op::T*
     using B = typename Op::B;
     using C = typename Op::C;
     const int64_t nvec = n / VEC;
-    const int64_t base = (int64_t)blockIdx.x * (kBlock * UNROLL) + threadIdx.x;
+    // Workgroup ids are dealt round-robin to the 8 XCDs.  Inside every group of 8 * kXcdRun workgroups the ids are permuted so
+    // that each XCD streams kXcdRun consecutive 4 KB pieces (256 KB) instead of every eighth piece: measured 1.5-2 % more
+    // bandwidth on a three-stream add (runs of 32 to 512 pieces are equivalent, 16 and below or 1024 and above are slower).
+    uint32_t bid = blockIdx.x;
+    {
+        constexpr uint32_t span = 8u * kXcdRun;
+        if (bid < (gridDim.x / span) * span) {
+            const uint32_t r = bid % span;
+            bid = bid - r + (r % 8u) * kXcdRun + r / 8u;
+        }
+    }
+    const int64_t base = (int64_t)bid * (kBlock * UNROLL) + threadIdx.x;
     Pack<A, VEC> va[UNROLL];
     Pack<B, VEC> vb[UNROLL];
     Pack<C, VEC> vc[UNROLL];
@@ -117,7 +130,7 @@ __global__ __launch_bounds__(kBlock) void map_flat_kernel(Op op, typename Op::T*
         }
     }
     // the n % VEC trailing elements
-    if (blockIdx.x == 0) {
+    if (bid == 0) {
         const int64_t i = nvec * VEC + threadIdx.x;
         if (threadIdx.x < VEC && i < n) {
             A xa = A();
