@@ -126,20 +126,29 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(R r, const void* sr
     }
 }
 
+// Grid: one workgroup per (row chunk, other, column tile), linearised with the column tile fastest.  Workgroup ids are dealt
+// round-robin to the 8 XCDs; `xcd_chunk` (total / 8 when divisible, else 0) re-numbers them so that every XCD takes one contiguous
+// range of that order (with 8 column tiles the plain order would pin each XCD to one 4 KB-wide column strip).
+// Partials of a split axis are stored [other][split][column]: the VEC states of a thread are contiguous (one vector store).
 template <class R, int VEC, int WX>
 __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(R r, const typename R::In* src, typename R::Out* out,
-                                                             typename R::State* partial, OuterArgs o, uint32_t col_tiles, uint32_t nc,
-                                                             int64_t tc_stride, int64_t n, int64_t sr, int64_t chunk, uint32_t splits) {
+                                                             typename R::State* partial, OuterArgs o, uint32_t col_tiles, uint32_t base_blocks,
+                                                             uint32_t xcd_chunk, uint32_t nc, int64_t tc_stride, int64_t n, int64_t sr,
+                                                             int64_t chunk, uint32_t splits) {
     using State = typename R::State;
     using In = typename R::In;
     constexpr int NY = kBlock / WX;
     constexpr int U = 2;
     const uint32_t x = threadIdx.x % WX, y = threadIdx.x / WX;
-    const uint32_t tile = blockIdx.x % col_tiles, other = blockIdx.x / col_tiles;
+    uint32_t bid = blockIdx.x;
+    if (xcd_chunk) bid = (bid % 8u) * xcd_chunk + bid / 8u;
+    const uint32_t split = bid / base_blocks;
+    bid -= split * base_blocks;
+    const uint32_t tile = bid % col_tiles, other = bid / col_tiles;
     const uint32_t col0 = (tile * WX + x) * VEC;
     int64_t toff, soff;
     outer_offsets(o, other, toff, soff);
-    const int64_t r0 = (int64_t)blockIdx.y * chunk;
+    const int64_t r0 = (int64_t)split * chunk;
     const int64_t r1 = (r0 + chunk < n) ? r0 + chunk : n;
     State st[VEC];
 #pragma unroll
@@ -178,13 +187,47 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(R r, const typename
         }
     }
     if (y == 0 && active) {
+        if (splits == 1) {
 #pragma unroll
-        for (int e = 0; e < VEC; e++) {
-            State s = st[e];
-            const uint32_t col = col0 + e;
-            if (splits == 1) out[toff + (int64_t)col * tc_stride] = r.extract(s);
-            else partial[((int64_t)other * nc + col) * splits + blockIdx.y] = s;
+            for (int e = 0; e < VEC; e++) out[toff + (int64_t)(col0 + e) * tc_stride] = r.extract(st[e]);
+        } else {
+            State* q = partial + ((int64_t)other * splits + split) * nc + col0;
+            if constexpr (VEC > 1 && sizeof(State) * VEC == 16) {
+                // VEC > 1 implies nc % VEC == 0, so q is 16-byte aligned like the workspace
+                typename RawWord<16>::type w;
+                __builtin_memcpy(&w, st, 16);
+                *reinterpret_cast<typename RawWord<16>::type*>(q) = w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC; e++) q[e] = st[e];
+            }
         }
+    }
+}
+
+// Finishing pass of a split column reduction: partials [other][split][column] -> out.  WX lanes along the columns (coalesced reads
+// of State), kBlock / WX groups share the splits and are combined through LDS in a fixed order.
+template <class R, int WX>
+__global__ __launch_bounds__(kBlock) void reduce_cols_finish_kernel(R r, const typename R::State* partial, typename R::Out* out, OuterArgs o,
+                                                                    uint32_t col_tiles, uint32_t nc, int64_t tc_stride, uint32_t splits) {
+    using State = typename R::State;
+    constexpr int NY = kBlock / WX;
+    const uint32_t x = threadIdx.x % WX, y = threadIdx.x / WX;
+    const uint32_t tile = blockIdx.x % col_tiles, other = blockIdx.x / col_tiles;
+    const uint32_t col = tile * WX + x;
+    State st = r.init();
+    if (col < nc) {
+        const State* p = partial + (int64_t)other * splits * nc + col;
+        for (uint32_t s = y; s < splits; s += NY) st = r.combine(st, p[(int64_t)s * nc]);
+    }
+    __shared__ State sh[NY][WX];
+    sh[y][x] = st;
+    __syncthreads();
+    if (y == 0 && col < nc) {
+        for (int w = 1; w < NY; w++) st = r.combine(st, sh[w][x]);
+        int64_t toff, soff;
+        outer_offsets(o, other, toff, soff);
+        out[toff + (int64_t)col * tc_stride] = r.extract(st);
     }
 }
 
@@ -350,23 +393,23 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
             }
             wx = 64;
         }
-        if (base_blocks <= 0x7FFFFFFF && splits <= 65535) {
+        const int64_t total_blocks = base_blocks * splits;
+        if (total_blocks <= 0x7FFFFFFF) {
             State* partial = nullptr;
             if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial));
-            const dim3 grid((unsigned)base_blocks, splits);
-#define DNH_COLS(V, W) hipLaunchKernelGGL((reduce_cols_kernel<R, V, W>), grid, dim3(kBlock), 0, stream, r, src, out, partial, oo, col_tiles, nc, tc_stride, n, sr, chunk, splits)
+            const dim3 grid((unsigned)total_blocks);
+            const uint32_t xcd_chunk = (total_blocks % 8 == 0 && total_blocks >= 64) ? (uint32_t)(total_blocks / 8) : 0u;
+#define DNH_COLS(V, W) hipLaunchKernelGGL((reduce_cols_kernel<R, V, W>), grid, dim3(kBlock), 0, stream, r, src, out, partial, oo, col_tiles, (uint32_t)base_blocks, xcd_chunk, nc, tc_stride, n, sr, chunk, splits)
             if (vec) { if (wx == 256) DNH_COLS(VEC, 256); else DNH_COLS(VEC, 64); }
             else { if (wx == 256) DNH_COLS(1, 256); else DNH_COLS(1, 64); }
 #undef DNH_COLS
             DNH_LAUNCH_CHECK();
             if (splits > 1) {
-                // partials are laid out [others][nc][splits]; enumerate outputs in that order for the finishing pass
-                OuterArgs fo = oo;
-                fo.shape[fo.nd] = nc;
-                fo.tstride[fo.nd] = tc_stride;
-                fo.sstride[fo.nd] = 0;
-                fo.nd++;
-                DNH_TRY(launch_finish(r, partial, out, fo, nout, splits, stream));
+                constexpr int FW = 32;
+                const uint32_t ftiles = cdiv(nc, FW);
+                hipLaunchKernelGGL((reduce_cols_finish_kernel<R, FW>), dim3(ftiles * others), dim3(kBlock), 0, stream, r, (const State*)partial, out,
+                                   oo, ftiles, nc, tc_stride, splits);
+                DNH_LAUNCH_CHECK();
             }
             return DNH_OK;
         }
