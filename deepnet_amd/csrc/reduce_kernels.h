@@ -405,7 +405,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
 #undef DNH_COLS
             DNH_LAUNCH_CHECK();
             if (splits > 1) {
-                constexpr int FW = 32;
+                constexpr int FW = 16;
                 const uint32_t ftiles = cdiv(nc, FW);
                 hipLaunchKernelGGL((reduce_cols_finish_kernel<R, FW>), dim3(ftiles * others), dim3(kBlock), 0, stream, r, (const State*)partial, out,
                                    oo, ftiles, nc, tc_stride, splits);
