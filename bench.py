@@ -28,8 +28,8 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, vendor figure
 FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by the plain-copy calibration
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): 2.0 * 262151.3 KiB + 262144.9 KiB for Add.
-TRAFFIC_BYTES = {"Add": int((2.0 * 262151.3 + 262144.9) * 1024)}
+# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): 2.0 * 262157.8 KiB + 262144.1 KiB for Add.
+TRAFFIC_BYTES = {"Add": int((2.0 * 262157.8 + 262144.1) * 1024)}
 
 
 def log(*a):
