@@ -214,9 +214,14 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
                 acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
                 acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
                 acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+                // FAST kernel: the next step's tiles go to the other LDS buffer inside the MFMA chain (their loads were issued a
+                // thousand cycles earlier), so only the barrier is left at the end of the step: +2-7 % (the four wavefronts of
+                // a SIMD run in phase, so whatever follows the last MFMA of a step leaves the matrix pipe idle).  The general
+                // kernel, whose element loads take longer to arrive, measured 5 % slower that way and stores at the end.
+                if (FAST && kk == 4 && more) store_tiles(cur ^ 1, vl);
             }
             if (more) {
-                store_tiles(cur ^ 1, vl);
+                if (!FAST) store_tiles(cur ^ 1, vl);
                 __syncthreads();
                 cur ^= 1;
             }
@@ -266,7 +271,7 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
                     for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[i], bv[j], acc[i][j], 0, 0, 0);
             }
             if (more) {
-                store_tiles(cur ^ 1, vl);
+                store_tiles(cur ^ 1, vl);   // storing inside the MFMA chain (as the fp32 path does) measured no gain for fp64
                 __syncthreads();
                 cur ^= 1;
             }
