@@ -3,6 +3,7 @@
 // :206-270 transfers, Cuda/CudaRegMem.fs pinned memory, Cuda/CudaCfg.fs:16-27 stream).
 #include "common.h"
 
+#include <atomic>
 #include <map>
 #include <mutex>
 #include <unordered_map>
@@ -11,6 +12,7 @@ namespace dnh {
 
 namespace {
 std::mutex g_mu;
+std::atomic<uint64_t> g_epoch{1};   // bumped whenever the active device changes
 bool g_init = false;
 int g_device = 0;
 int g_cus = 256;
@@ -74,17 +76,22 @@ static int32_t init_locked(int device) {
     }
     g_device = device;
     g_init = true;
+    g_epoch.fetch_add(1, std::memory_order_release);
     return DNH_OK;
 }
 
 int32_t ensure_init() {
+    // HIP's current device is per host thread: the first call of a thread (and the first after dnh_init selected another
+    // device) binds the thread to our device; later calls cost one thread-local compare.
+    thread_local int t_bound_device = -1;
+    thread_local uint64_t t_bound_epoch = 0;
+    if (t_bound_device >= 0 && t_bound_epoch == g_epoch.load(std::memory_order_acquire)) return DNH_OK;
     std::lock_guard<std::mutex> lock(g_mu);
-    if (g_init) {
-        // HIP's current device is per host thread; make the calling thread use ours.
-        DNH_HIP(hipSetDevice(g_device));
-        return DNH_OK;
-    }
-    return init_locked(0);
+    if (!g_init) DNH_TRY(init_locked(0));
+    DNH_HIP(hipSetDevice(g_device));
+    t_bound_device = g_device;
+    t_bound_epoch = g_epoch.load(std::memory_order_acquire);
+    return DNH_OK;
 }
 
 int device_cus() { return g_cus; }
