@@ -1,0 +1,61 @@
+"""Thread safety of the C ABI: several host threads, each on its own stream (Cfg.Stream is thread-local, as in the reference's
+Cuda/CudaCfg.fs:16), run chains that allocate from the block cache and use the per-stream workspace (split reductions,
+compaction) at the same time.  ctypes releases the GIL during every call, so the calls really overlap."""
+import ctypes as C
+import threading
+
+import numpy as np
+import pytest
+
+from deepnet_amd import native
+
+pytestmark = pytest.mark.gpu
+
+
+def test_concurrent_threads_on_their_own_streams(G, H):
+    lib = native.load()
+    nthreads, rounds = 4, 6
+    rng = np.random.default_rng(7)
+    inputs = [(rng.integers(-1000, 1000, (600, 700)).astype(np.int32), rng.integers(-1000, 1000, (600, 700)).astype(np.int32))
+              for _ in range(nthreads)]
+
+    def chain(M, a, b):
+        x, y = M.ofNumpy(a), M.ofNumpy(b)
+        out = []
+        for _ in range(rounds):
+            x = (x * y + x) - y                       # temporaries from the block cache
+            out.append(M.toNumpy(x.sumAxis(0)))       # column fold with a finishing pass (per-stream workspace)
+            out.append(M.toNumpy(x.flatten().sumAxis(0)))
+            m = x > y
+            out.append(M.toNumpy(x.flatten().M(m.flatten())))     # compaction: counts in the workspace
+            out.append(M.toNumpy(x.argMaxAxis(1)))
+        return out
+
+    want = [chain(H, a, b) for a, b in inputs]
+    got = [None] * nthreads
+    errors = []
+
+    def worker(i):
+        try:
+            s = C.c_void_p()
+            native.check(lib.dnh_stream_create(C.byref(s)))
+            G.Cfg.Stream = s.value
+            try:
+                got[i] = chain(G, *inputs[i])
+            finally:
+                G.synchronize()
+                G.Cfg.Stream = 0
+                native.check(lib.dnh_stream_destroy(s))
+        except Exception as e:  # noqa: BLE001
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(nthreads)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    for i in range(nthreads):
+        assert got[i] is not None
+        for ref, g in zip(want[i], got[i]):
+            np.testing.assert_array_equal(ref, g)
