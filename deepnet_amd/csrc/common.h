@@ -47,7 +47,7 @@ inline int32_t fail(int32_t code, const char* fmt, ...) {
 
 int32_t ensure_init();                       // DNH_ERR_NOT_INITIALIZED-free lazy init on the current device
 int device_cus();                            // compute units of the active device
-int32_t* error_flag_ptr();                   // device int32 set by gather/scatter kernels on a bad index
+int32_t error_flag_ptr(hipStream_t stream, int32_t** out);   // the stream's device int32 set by gather/scatter kernels on a bad index
 // Per-stream scratch buffer owned by the library (partials of two-pass reductions, block counts of compactions).
 // Kernels on one stream are ordered, so one buffer per stream is race-free; it grows on demand.
 int32_t workspace(hipStream_t stream, size_t bytes, void** out);

@@ -484,11 +484,13 @@ extern "C" int32_t dnh_gather(const DnhTensor* t, const DnhTensor* const* idx, i
     if (n == 0) return DNH_OK;
     if (n > (int64_t)kMaxItems) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_gather: more than 2^32 elements");
     hipStream_t s = (hipStream_t)stream;
+    int32_t* eflag = nullptr;
+    DNH_TRY(error_flag_ptr(s, &eflag));
     const dim3 grid(cdiv(n, kBlock));
     switch (dtype_size(t->dtype)) {
-        case 1: hipLaunchKernelGGL(gather_kernel<uint8_t>, grid, dim3(kBlock), 0, s, (uint8_t*)elem_ptr(t), (const uint8_t*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
-        case 4: hipLaunchKernelGGL(gather_kernel<uint32_t>, grid, dim3(kBlock), 0, s, (uint32_t*)elem_ptr(t), (const uint32_t*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
-        case 8: hipLaunchKernelGGL(gather_kernel<uint64_t>, grid, dim3(kBlock), 0, s, (uint64_t*)elem_ptr(t), (const uint64_t*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
+        case 1: hipLaunchKernelGGL(gather_kernel<uint8_t>, grid, dim3(kBlock), 0, s, (uint8_t*)elem_ptr(t), (const uint8_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
+        case 4: hipLaunchKernelGGL(gather_kernel<uint32_t>, grid, dim3(kBlock), 0, s, (uint32_t*)elem_ptr(t), (const uint32_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
+        case 8: hipLaunchKernelGGL(gather_kernel<uint64_t>, grid, dim3(kBlock), 0, s, (uint64_t*)elem_ptr(t), (const uint64_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
         default: return fail(DNH_ERR_NOT_SUPPORTED, "dnh_gather: unsupported element width");
     }
     DNH_LAUNCH_CHECK();
@@ -503,11 +505,13 @@ extern "C" int32_t dnh_scatter(const DnhTensor* t, const DnhTensor* const* idx, 
     if (n == 0) return DNH_OK;
     if (n > (int64_t)kMaxItems) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_scatter: more than 2^32 elements");
     hipStream_t s = (hipStream_t)stream;
+    int32_t* eflag = nullptr;
+    DNH_TRY(error_flag_ptr(s, &eflag));
     const dim3 grid(cdiv(n, kBlock));
-#define CASE(DT, X) case DT: hipLaunchKernelGGL(scatter_kernel<X>, grid, dim3(kBlock), 0, s, (X*)elem_ptr(t), (const X*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
+#define CASE(DT, X) case DT: hipLaunchKernelGGL(scatter_kernel<X>, grid, dim3(kBlock), 0, s, (X*)elem_ptr(t), (const X*)elem_ptr(src), a, (uint32_t)n, eflag); break;
     switch (t->dtype) {
         CASE(DNH_U8, uint8_t)
-        case DNH_I8: hipLaunchKernelGGL(scatter_kernel<uint8_t>, grid, dim3(kBlock), 0, s, (uint8_t*)elem_ptr(t), (const uint8_t*)elem_ptr(src), a, (uint32_t)n, error_flag_ptr()); break;
+        case DNH_I8: hipLaunchKernelGGL(scatter_kernel<uint8_t>, grid, dim3(kBlock), 0, s, (uint8_t*)elem_ptr(t), (const uint8_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
         CASE(DNH_I32, int32_t) CASE(DNH_U32, uint32_t) CASE(DNH_I64, int64_t) CASE(DNH_U64, uint64_t) CASE(DNH_F32, float) CASE(DNH_F64, double)
         default: return fail(DNH_ERR_NOT_SUPPORTED, "dnh_scatter on %s", dtype_name(t->dtype));
     }

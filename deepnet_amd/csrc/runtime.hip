@@ -16,7 +16,7 @@ std::atomic<uint64_t> g_epoch{1};   // bumped whenever the active device changes
 bool g_init = false;
 int g_device = 0;
 int g_cus = 256;
-int32_t* g_error_flag = nullptr;
+std::map<hipStream_t, int32_t*> g_error_flags;   // one index-error word per stream, so concurrent streams do not see each other's errors
 
 struct Workspace {
     void* ptr = nullptr;
@@ -70,10 +70,6 @@ static int32_t init_locked(int device) {
     hipDeviceProp_t prop;
     DNH_HIP(hipGetDeviceProperties(&prop, device));
     g_cus = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
-    if (!g_error_flag) {
-        DNH_HIP(hipMalloc((void**)&g_error_flag, sizeof(int32_t)));
-        DNH_HIP(hipMemset(g_error_flag, 0, sizeof(int32_t)));
-    }
     g_device = device;
     g_init = true;
     g_epoch.fetch_add(1, std::memory_order_release);
@@ -95,7 +91,16 @@ int32_t ensure_init() {
 }
 
 int device_cus() { return g_cus; }
-int32_t* error_flag_ptr() { return g_error_flag; }
+int32_t error_flag_ptr(hipStream_t stream, int32_t** out) {
+    std::lock_guard<std::mutex> lock(g_mu);
+    int32_t*& p = g_error_flags[stream];
+    if (!p) {
+        DNH_HIP(hipMalloc((void**)&p, sizeof(int32_t)));
+        DNH_HIP(hipMemset(p, 0, sizeof(int32_t)));   // synchronous: done before any kernel that may set it is queued
+    }
+    *out = p;
+    return DNH_OK;
+}
 
 int32_t workspace(hipStream_t stream, size_t bytes, void** out) {
     std::lock_guard<std::mutex> lock(g_mu);
@@ -118,6 +123,11 @@ int32_t workspace(hipStream_t stream, size_t bytes, void** out) {
 
 static void drop_workspace(hipStream_t stream) {
     std::lock_guard<std::mutex> lock(g_mu);
+    auto ef = g_error_flags.find(stream);
+    if (ef != g_error_flags.end()) {
+        if (ef->second) (void)hipFree(ef->second);
+        g_error_flags.erase(ef);
+    }
     auto it = g_ws.find(stream);
     if (it != g_ws.end()) {
         if (it->second.ptr) (void)hipFree(it->second.ptr);
@@ -170,8 +180,10 @@ int32_t dnh_async_error(void* stream, int32_t* code) {
     DNH_TRY(ensure_init());
     int32_t flag = 0;
     DNH_HIP(hipStreamSynchronize((hipStream_t)stream));
-    DNH_HIP(hipMemcpy(&flag, g_error_flag, sizeof(flag), hipMemcpyDeviceToHost));
-    if (flag) DNH_HIP(hipMemset(g_error_flag, 0, sizeof(flag)));
+    int32_t* dev_flag = nullptr;
+    DNH_TRY(error_flag_ptr((hipStream_t)stream, &dev_flag));
+    DNH_HIP(hipMemcpy(&flag, dev_flag, sizeof(flag), hipMemcpyDeviceToHost));
+    if (flag) DNH_HIP(hipMemset(dev_flag, 0, sizeof(flag)));
     *code = flag ? DNH_ERR_INDEX_OUT_OF_RANGE : DNH_OK;
     if (flag) last_error() = "an index tensor held a position outside the indexed tensor's shape";
     return DNH_OK;

@@ -135,7 +135,7 @@ int32_t dnh_device_info(DnhDeviceInfo* info);
 /* Copies the calling thread's last error message (NUL terminated, truncated to n). */
 int32_t dnh_last_error(char* buf, size_t n);
 /* Reads and clears the device-side index error flag set by gather/scatter kernels on `stream`
- * (synchronises the stream).  *code = DNH_OK or DNH_ERR_INDEX_OUT_OF_RANGE.
+ * (synchronises the stream; every stream has its own flag, so concurrent streams do not see each other's errors).  *code = DNH_OK or DNH_ERR_INDEX_OUT_OF_RANGE.
  * Replaces the error word + `Cfg.Stacktrace` read-back of Cuda/CudaKernels.fs:323-342, 385-398. */
 int32_t dnh_async_error(void* stream, int32_t* code);
 

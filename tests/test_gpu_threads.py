@@ -59,3 +59,34 @@ def test_concurrent_threads_on_their_own_streams(G, H):
         assert got[i] is not None
         for ref, g in zip(want[i], got[i]):
             np.testing.assert_array_equal(ref, g)
+
+
+def test_index_error_flag_is_per_stream(G):
+    """An out-of-range gather index on one stream is reported on that stream only."""
+    lib = native.load()
+    s = C.c_void_p()
+    native.check(lib.dnh_stream_create(C.byref(s)))
+    try:
+        src = G.ofNumpy(np.arange(10, dtype=np.int32))
+        bad = G.ofNumpy(np.array([1, 99, 3], dtype=np.int64))
+        good = G.ofNumpy(np.array([1, 2, 3], dtype=np.int64))
+        G.synchronize()
+        stack = G.Cfg.Stacktrace
+        G.Cfg.Stacktrace = False                      # do not read the flag back after each call
+        try:
+            G.Cfg.Stream = s.value
+            type(src).gather([bad], src)              # sets the flag of stream s
+            G.Cfg.Stream = 0
+            type(src).gather([good], src)
+            code = C.c_int32(-1)
+            native.check(lib.dnh_async_error(0, C.byref(code)))
+            assert code.value == 0                    # the default stream saw no error
+            native.check(lib.dnh_async_error(s.value, C.byref(code)))
+            assert code.value == 5                    # DNH_ERR_INDEX_OUT_OF_RANGE, and the read cleared it
+            native.check(lib.dnh_async_error(s.value, C.byref(code)))
+            assert code.value == 0
+        finally:
+            G.Cfg.Stream = 0
+            G.Cfg.Stacktrace = stack
+    finally:
+        native.check(lib.dnh_stream_destroy(s))
