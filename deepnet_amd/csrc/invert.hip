@@ -192,33 +192,38 @@ __global__ __launch_bounds__(kMaxPanelThreads) void invert_subpanel_lds_kernel(T
         __syncthreads();
         const T sj = (c == j ? T(1) : L[col * CW + c]) / L[col * CW + j];   // my column's entry of the scaled pivot row
         __syncthreads();                                                    // everyone has read the pivot row before it changes
-        best = T(-1);
-        bi = n;
-        const bool is_pivot_col = c == j, is_next_col = c == j + 1;
-        // four rows per round: all reads of a round are issued before its writes (the rows of a round are distinct, and the
-        // lanes of a row read its multiplier before the owner of the pivot column overwrites it)
+        const bool is_pivot_col = c == j;
+        // The update is bound by the instruction issue rate of the one CU that runs it, so the loop body is kept minimal: every
+        // row is treated alike (the pivot row is rewritten by its owners afterwards, the next column's pivot search is a separate
+        // short walk instead of a compare in every lane).  Four rows per round: all reads of a round are issued before its writes
+        // (the rows of a round are distinct, and the lanes of a row read its multiplier before the owner of the pivot column
+        // overwrites it).
         constexpr int U = 4;
-        for (int r0 = rsub; r0 < n; r0 += U * rpp) {
+        int r0 = rsub;
+        for (; r0 + (U - 1) * rpp < n; r0 += U * rpp) {
             T v[U], f[U];
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const int r = r0 + u * rpp;
-                if (r < n) { v[u] = L[r * CW + c]; f[u] = L[r * CW + j]; }
+                v[u] = L[(r0 + u * rpp) * CW + c];
+                f[u] = L[(r0 + u * rpp) * CW + j];
             }
 #pragma unroll
-            for (int u = 0; u < U; u++) {
-                const int r = r0 + u * rpp;
-                if (r < n) {
-                    const T nv = (r == col) ? sj : (is_pivot_col ? T(0) : v[u]) - f[u] * sj;
-                    L[r * CW + c] = nv;
-                    if (is_next_col && r > col) {   // the next column's pivot candidates, rows ascending per thread
-                        const T a = abs_of(nv);
-                        if (a > best) { best = a; bi = r; }
-                    }
-                }
-            }
+            for (int u = 0; u < U; u++) L[(r0 + u * rpp) * CW + c] = (is_pivot_col ? T(0) : v[u]) - f[u] * sj;
         }
+        for (; r0 < n; r0 += rpp) {
+            const T v = L[r0 * CW + c], f = L[r0 * CW + j];
+            L[r0 * CW + c] = (is_pivot_col ? T(0) : v) - f * sj;
+        }
+        if (rsub == col % rpp) L[col * CW + c] = sj;   // the owners of the pivot row (they wrote it last, in the loop above)
         __syncthreads();
+        // pivot candidates of the next column
+        best = T(-1);
+        bi = n;
+        if (j + 1 < sw)
+            for (int r = col + 1 + tid; r < n; r += nt) {
+                const T a = abs_of(L[r * CW + j + 1]);
+                if (a > best) { best = a; bi = r; }
+            }
     }
     if (tid < sw) piv[cs + tid] = piv_s[tid];
     if (in_panel)
