@@ -114,6 +114,11 @@ def toNumpy(t: Tensor) -> np.ndarray:
     return out
 
 
+def transfer(t: Tensor) -> Tensor:
+    """HostTensor.transfer: brings a tensor of any device to this host device (Tensor.fs:696-711)."""
+    return t.Transfer(Dev)
+
+
 def set_threads(n: int):
     load().href_set_threads(int(n))
 
