@@ -251,6 +251,71 @@ class Tensor:
             rngs.append(Rng.AllFill)
         return self.Relayout(L.view(rngs, self._layout))
 
+    def __setitem__(self, key, value):
+        """a.[rng] <- value (Tensor.fs:3232-3245): the value is broadcast to the view and copied into it."""
+        view = self[key]
+        if not isinstance(value, Tensor):
+            value = self.scalarLike(value)
+        view.CopyFrom(value)
+
+    # ---- diagonals, trace, concatenation (Tensor.fs:4100-4215, 4401-4436) -------------------------------------------------------
+    def diag(self) -> "Tensor":
+        if self.NDims < 2:
+            raise ValueError(f"Need at least a two dimensional array for diagonal but got shape {self.Shape}.")
+        return self.diagAxis(self.NDims - 2, self.NDims - 1)
+
+    def diagMatAxis(self, ax1, ax2) -> "Tensor":
+        if ax1 == ax2:
+            raise ValueError("axes to use for diagonal must be different")
+        ax1, ax2 = (ax1, ax2) if ax1 < ax2 else (ax2, ax1)
+        if not 0 <= ax1 < self.NDims:
+            raise ValueError(f"Axis {ax1} out of range for tensor of shape {self.Shape}.")
+        if not 0 <= ax2 <= self.NDims:
+            raise ValueError(f"Cannot insert axis at position {ax2} into array of shape {self.Shape}.")
+        dShp = list(self.Shape)
+        dShp.insert(ax2, self.Shape[ax1])
+        d = Tensor.zeros(dShp, self.Dev, self.DataType)
+        d.diagAxis(ax1, ax2).CopyFrom(self)
+        return d
+
+    def diagMat(self) -> "Tensor":
+        if self.NDims < 1:
+            raise ValueError("need at leat a one-dimensional array to create a diagonal matrix")
+        return self.diagMatAxis(self.NDims - 1, self.NDims)
+
+    def traceAxis(self, ax1, ax2) -> "Tensor":
+        tax = ax1 if ax1 < ax2 else ax1 - 1
+        return self.diagAxis(ax1, ax2).sumAxis(tax)
+
+    def trace(self) -> "Tensor":
+        if self.NDims < 2:
+            raise ValueError(f"Need at least a two dimensional array for trace but got shape {self.Shape}.")
+        return self.traceAxis(self.NDims - 2, self.NDims - 1)
+
+    @staticmethod
+    def concat(ax: int, ts) -> "Tensor":
+        ts = list(ts)
+        if not ts:
+            raise ValueError("Cannot concatenate empty sequence of tensors.")
+        shp = ts[0].Shape
+        if not 0 <= ax < len(shp):
+            raise ValueError(f"Concatenation axis {ax} is out of range for shape {shp}.")
+        for i, t in enumerate(ts):
+            if t.Shape[:ax] + t.Shape[ax + 1:] != shp[:ax] + shp[ax + 1:]:
+                raise ValueError(f"Concatentation element with index {i} with shape {t.Shape} must be equal to shape {shp} "
+                                 f"of the first element, except in the concatenation axis {ax}")
+        total = sum(t.Shape[ax] for t in ts)
+        cc = Tensor.new(shp[:ax] + [total] + shp[ax + 1:], ts[0].Dev, ts[0].DataType)
+        pos = 0
+        for t in ts:
+            n = t.Shape[ax]
+            if n > 0:
+                key = [slice(None)] * len(shp)
+                key[ax] = slice(pos, pos + n)
+                cc[tuple(key)] = t
+                pos += n
+        return cc
+
     # ---- element-wise: prepare helpers (Tensor.fs:4520-4597) -------------------------------------------------------------------------
     def _prep1(self, dtype=None) -> "Tensor":
         return Tensor.new(self.Shape, self.Dev, dtype or self.DataType)
