@@ -117,3 +117,48 @@ def test_invert_twice_gives_the_matrix_back(H, G, rng):
         assert almost_equal(G.toNumpy(Tensor.invert(Tensor.invert(t))), x, abs_tol=1e-8, rel_tol=1e-5)
     with pytest.raises(SingularMatrixException):             # BaseTests.fs:204-211
         Tensor.invert(G.ofNumpy(np.array([[1.0, 0.0, 0.0], [1.0, 2.0, 0.0], [1.0, 0.0, 0.0]])))
+
+
+def _brute_gather(a, idxs, tshape):
+    out = np.empty(tshape, a.dtype)
+    for pos in np.ndindex(*tshape):
+        src = tuple(int(np.broadcast_to(i, tshape)[pos]) if i is not None else pos[d] for d, i in enumerate(idxs))
+        out[pos] = a[src]
+    return out
+
+
+def _brute_scatter(a, idxs, tshape):
+    out = np.zeros(tshape, a.dtype)
+    for pos in np.ndindex(*a.shape):
+        trg = tuple(int(np.broadcast_to(i, a.shape)[pos]) if i is not None else pos[d] for d, i in enumerate(idxs))
+        out[trg] += a[pos]
+    return out
+
+
+def test_select_and_disperse(H, G):
+    """BaseTests.fs:261-348 (the reference only prints these; here the results are checked against the definition)."""
+    a = np.arange(12, dtype=np.float64).reshape(4, 3)
+    i0a = np.broadcast_to(np.array([1, 2, 0, 3], dtype=np.int64)[:, None], (4, 2))       # padRight |> broadcastDim 1 2
+    i0b = np.array([[1, 2, 2]], dtype=np.int64)                                           # padLeft
+    i1b = np.array([[0, 0, 1]], dtype=np.int64)
+    gather_cases = [([i0a, None], (4, 2)), ([i0b, None], (1, 3)), ([i0b, i1b], (1, 3))]
+    for idxs, tshape in gather_cases:
+        want = _brute_gather(a, idxs, tshape)
+        for M in (H, G):
+            src = M.ofNumpy(a)
+            ts = []
+            for i in idxs:
+                if i is None:
+                    ts.append(None)
+                elif i is i0a:
+                    ts.append(M.ofNumpy(np.array([1, 2, 0, 3], dtype=np.int64)).padRight().broadcastTo([4, 2]))   # a stride-0 index view
+                else:
+                    ts.append(M.ofNumpy(np.ascontiguousarray(i)))
+            np.testing.assert_array_equal(M.toNumpy(Tensor.gather(ts, src)), want)
+    scatter_cases = [([i0b, i1b], (3, 3)), ([i0b, None], (3, 3)), ([None, None], (5, 3))]
+    for idxs, tshape in scatter_cases:
+        want = _brute_scatter(a, idxs, tshape)
+        for M in (H, G):
+            src = M.ofNumpy(a)
+            ts = [M.ofNumpy(np.ascontiguousarray(i)) if i is not None else None for i in idxs]
+            np.testing.assert_array_equal(M.toNumpy(Tensor.scatter(ts, list(tshape), src)), want)
