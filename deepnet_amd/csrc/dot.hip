@@ -392,10 +392,33 @@ __global__ __launch_bounds__(kBlock) void gemv_cols_kernel(T* y, T* partial, con
 #pragma unroll
         for (int e = 0; e < VEC; e++) acc[e] += v0.v[e] * x0;
     }
+    if (splits == 1) {
 #pragma unroll
-    for (int e = 0; e < VEC; e++) {
-        if (splits == 1) y[(int64_t)(m + e) * sym] = acc[e];
-        else partial[(int64_t)(m + e) * splits + blockIdx.y] = acc[e];
+        for (int e = 0; e < VEC; e++) y[(int64_t)(m + e) * sym] = acc[e];
+    } else {
+        // partials [split][m]: the VEC sums of a thread leave as one vector store (VEC > 1 implies M % VEC == 0)
+        Pack<T, VEC> v;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) v.v[e] = acc[e];
+        store_pack<T, VEC>(partial + (int64_t)blockIdx.y * M + m, v);
+    }
+}
+
+// Sums the [split][m] partials of gemv_cols in split order inside each of the 16 groups, then the groups in order (deterministic).
+template <class T>
+__global__ __launch_bounds__(kBlock) void gemv_cols_finish_kernel(T* y, const T* partial, uint32_t M, uint32_t splits, int64_t sym) {
+    constexpr int WX = 16, NY = kBlock / WX;
+    const uint32_t x = threadIdx.x % WX, g = threadIdx.x / WX;
+    const uint32_t m = blockIdx.x * WX + x;
+    T s = T(0);
+    if (m < M)
+        for (uint32_t i = g; i < splits; i += NY) s += partial[(int64_t)i * M + m];
+    __shared__ T sh[NY][WX];
+    sh[g][x] = s;
+    __syncthreads();
+    if (g == 0 && m < M) {
+        for (int w = 1; w < NY; w++) s += sh[w][x];
+        y[(int64_t)m * sym] = s;
     }
 }
 
@@ -469,7 +492,7 @@ bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t strea
         if (splits > 1 && (*status = workspace(stream, sizeof(T) * (size_t)M * splits, (void**)&partial)) != DNH_OK) return true;
         if (vec) hipLaunchKernelGGL((gemv_cols_kernel<T, V>), dim3((unsigned)mblocks, splits), dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sak, g.sbk, g.scm, chunk, splits);
         else hipLaunchKernelGGL((gemv_cols_kernel<T, 1>), dim3((unsigned)mblocks, splits), dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sak, g.sbk, g.scm, chunk, splits);
-        if (splits > 1) hipLaunchKernelGGL(gemv_finish_kernel<T>, dim3(M), dim3(kBlock), 0, stream, y, (const T*)partial, M, splits, g.scm);
+        if (splits > 1) hipLaunchKernelGGL(gemv_cols_finish_kernel<T>, dim3((M + 15) / 16), dim3(kBlock), 0, stream, y, (const T*)partial, M, splits, g.scm);
     } else {
         return false;
     }
