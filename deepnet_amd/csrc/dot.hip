@@ -367,10 +367,16 @@ __global__ __launch_bounds__(kBlock) void gemv_rows_kernel(T* y, T* partial, con
 
 template <class T, int VEC>
 __global__ __launch_bounds__(kBlock) void gemv_cols_kernel(T* y, T* partial, const T* a, const T* x, uint32_t M, int64_t K, int64_t sak,
-                                                           int64_t sxk, int64_t sym, int64_t chunk, uint32_t splits) {
-    const uint32_t m = (blockIdx.x * kBlock + threadIdx.x) * VEC;
+                                                           int64_t sxk, int64_t sym, int64_t chunk, uint32_t splits, uint32_t mblocks,
+                                                           uint32_t xcd_chunk) {
+    // one workgroup per (split, block of m), the m block fastest; xcd_chunk re-numbers the workgroups so that every XCD takes one
+    // contiguous range of that order (with 8 m blocks the plain order would pin each XCD to one 4 KB-wide strip of the matrix)
+    uint32_t bid = blockIdx.x;
+    if (xcd_chunk) bid = (bid % 8u) * xcd_chunk + bid / 8u;
+    const uint32_t split = bid / mblocks, mb = bid - split * mblocks;
+    const uint32_t m = (mb * kBlock + threadIdx.x) * VEC;
     if (m >= M) return;
-    const int64_t k0 = (int64_t)blockIdx.y * chunk;
+    const int64_t k0 = (int64_t)split * chunk;
     const int64_t k1 = (k0 + chunk < K) ? k0 + chunk : K;
     T acc[VEC];
 #pragma unroll
@@ -400,7 +406,7 @@ __global__ __launch_bounds__(kBlock) void gemv_cols_kernel(T* y, T* partial, con
         Pack<T, VEC> v;
 #pragma unroll
         for (int e = 0; e < VEC; e++) v.v[e] = acc[e];
-        store_pack<T, VEC>(partial + (int64_t)blockIdx.y * M + m, v);
+        store_pack<T, VEC>(partial + (int64_t)split * M + m, v);
     }
 }
 
@@ -490,8 +496,12 @@ bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t strea
         }
         if (splits > 65535) return false;
         if (splits > 1 && (*status = workspace(stream, sizeof(T) * (size_t)M * splits, (void**)&partial)) != DNH_OK) return true;
-        if (vec) hipLaunchKernelGGL((gemv_cols_kernel<T, V>), dim3((unsigned)mblocks, splits), dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sak, g.sbk, g.scm, chunk, splits);
-        else hipLaunchKernelGGL((gemv_cols_kernel<T, 1>), dim3((unsigned)mblocks, splits), dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sak, g.sbk, g.scm, chunk, splits);
+        const int64_t total = mblocks * splits;
+        if (total > 0x7FFFFFFF) return false;
+        // measured: +4 % when the m blocks map one-to-one onto the XCDs (8 blocks), -2 % with 16 blocks, so only the former is re-numbered
+        const uint32_t xcd_chunk = (mblocks <= 8 && total % 8 == 0 && total >= 64) ? (uint32_t)(total / 8) : 0u;
+        if (vec) hipLaunchKernelGGL((gemv_cols_kernel<T, V>), dim3((unsigned)total), dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sak, g.sbk, g.scm, chunk, splits, (uint32_t)mblocks, xcd_chunk);
+        else hipLaunchKernelGGL((gemv_cols_kernel<T, 1>), dim3((unsigned)total), dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sak, g.sbk, g.scm, chunk, splits, (uint32_t)mblocks, xcd_chunk);
         if (splits > 1) hipLaunchKernelGGL(gemv_cols_finish_kernel<T>, dim3((M + 15) / 16), dim3(kBlock), 0, stream, y, (const T*)partial, M, splits, g.scm);
     } else {
         return false;
