@@ -11,15 +11,20 @@ open Tensor.Utils
 open Tensor.Backend
 
 /// Thread-local options (mirror of Tensor.Cuda.Cfg, Cuda/CudaCfg.fs:14-60).
-module Cfg =
-    [<ThreadStatic; DefaultValue>]
-    val mutable private stream: nativeint
-    [<ThreadStatic; DefaultValue>]
-    val mutable private noIndexCheck: bool
+type Cfg private () =
+    static let stream = new System.Threading.ThreadLocal<nativeint> (fun () -> IntPtr.Zero)
+    static let stacktrace = new System.Threading.ThreadLocal<bool> (fun () -> true)
+
     /// hipStream_t all operations of this thread are issued on (IntPtr.Zero = default stream)
-    let Stream with get () = stream and set v = stream <- v
-    /// read the device index-error flag after every Gather/Scatter so a bad index raises at the faulting call (default true)
-    let Stacktrace with get () = not noIndexCheck and set v = noIndexCheck <- not v
+    static member Stream
+        with get () = stream.Value
+        and set v = stream.Value <- v
+
+    /// Read the device index-error flag after every Gather/Scatter so that a bad index raises at the faulting call, as on
+    /// the host backend.  Defaults to true (a device never traps on a bad index, so this is the only way the error surfaces).
+    static member Stacktrace
+        with get () = stacktrace.Value
+        and set v = stacktrace.Value <- v
 
 module internal Desc =
     let dtypeOf (t: Type) =
