@@ -34,6 +34,7 @@ struct GemmArgs {
     uint32_t tiles_m, tiles_n;
     uint32_t xcd_chunk;                           // total tiles / 8 when divisible, else 0 (identity order)
     uint32_t accumulate;                          // 1: c += a.b (used by the blocked matrix inversion), 0: c = a.b
+    int64_t kchunk;                               // > 0: the innermost batch dimension walks K in chunks of this many (split K)
 };
 
 template <class T, bool FAST, bool ACC>
@@ -52,6 +53,7 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
     const uint32_t tm = bid % g.tiles_m;
     bid /= g.tiles_m;
     int64_t oa = 0, ob = 0, oc = 0;
+    int64_t K = g.K;  // this block's extent along k: a chunk of it when K is split
     for (int d = g.nbatch - 1; d >= 0; d--) {
         const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
         const uint32_t i = bid - q * g.bshape[d];
@@ -59,6 +61,7 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
         oa += (int64_t)i * g.bsa[d];
         ob += (int64_t)i * g.bsb[d];
         oc += (int64_t)i * g.bsc[d];
+        if (d == g.nbatch - 1 && g.kchunk > 0) K = min(g.kchunk, g.K - (int64_t)i * g.kchunk);
     }
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     a += oa;
@@ -86,7 +89,7 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
     constexpr bool LEAN = FAST && sizeof(T) == 4;
     const bool n_vec_ok = (g.N % (16 / (int)sizeof(T))) == 0;
     auto load_tiles = [&](int64_t k0, int buf) -> int {
-        if (FAST && (LEAN ? n_vec_ok : full_mn) && k0 + BK <= g.K) {
+        if (FAST && (LEAN ? n_vec_ok : full_mn) && k0 + BK <= K) {
             constexpr int V = 16 / (int)sizeof(T);           // elements per 16-byte load
             constexpr int APT = (BM * BK) / (kBlock * V);     // loads per thread for A (fp32: 2, fp64: 4)
             constexpr int KV = BK / V;                        // vectors per A row
@@ -119,12 +122,12 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
                 {
                     const int row = idx / BK, kk = idx % BK;
                     const int64_t m = m0 + row, k = k0 + kk;
-                    As[buf][kk][row] = (m < g.M && k < g.K) ? a[m * g.sam + k * g.sak] : T(0);
+                    As[buf][kk][row] = (m < g.M && k < K) ? a[m * g.sam + k * g.sak] : T(0);
                 }
                 {
                     const int kk = idx / BN, col = idx % BN;
                     const int64_t k = k0 + kk, n = n0 + col;
-                    Bs[buf][kk][col] = (k < g.K && n < g.N) ? b[k * g.sbk + n * g.sbn] : T(0);
+                    Bs[buf][kk][col] = (k < K && n < g.N) ? b[k * g.sbk + n * g.sbn] : T(0);
                 }
             }
             return kDirect;
@@ -135,12 +138,12 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
                 {
                     const int row = idx / BK, kk = idx % BK;
                     const int64_t m = m0 + row, k = k0 + kk;
-                    ra[i] = (m < g.M && k < g.K) ? a[m * g.sam + k * g.sak] : T(0);
+                    ra[i] = (m < g.M && k < K) ? a[m * g.sam + k * g.sak] : T(0);
                 }
                 {
                     const int kk = idx / BN, col = idx % BN;
                     const int64_t k = k0 + kk, n = n0 + col;
-                    rb[i] = (k < g.K && n < g.N) ? b[k * g.sbk + n * g.sbn] : T(0);
+                    rb[i] = (k < K && n < g.N) ? b[k * g.sbk + n * g.sbn] : T(0);
                 }
             }
             return kScalar;
@@ -198,8 +201,8 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
         __syncthreads();
         int cur = 0;
         const int lk = lane >> 5, lm = lane & 31;
-        for (int64_t k0 = 0; k0 < g.K; k0 += BK) {
-            const bool more = k0 + BK < g.K;
+        for (int64_t k0 = 0; k0 < K; k0 += BK) {
+            const bool more = k0 + BK < K;
             if (more) vl = load_tiles(k0 + BK, cur ^ 1);
             // Operand reads stay interleaved with the MFMAs (four per pair of LDS reads): hoisting all 32 reads of a K step
             // ahead of the MFMA chain costs 27 more registers, drops occupancy from 4 to 3 wavefronts per SIMD and measured
@@ -255,8 +258,8 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
         __syncthreads();
         int cur = 0;
         const int lk = lane >> 4, lm = lane & 15;
-        for (int64_t k0 = 0; k0 < g.K; k0 += BK) {
-            const bool more = k0 + BK < g.K;
+        for (int64_t k0 = 0; k0 < K; k0 += BK) {
+            const bool more = k0 + BK < K;
             if (more) vl = load_tiles(k0 + BK, cur ^ 1);
 #pragma unroll
             for (int kk = 0; kk < BK; kk += 4) {
@@ -291,16 +294,118 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
     }
 }
 
+// Split K.  A product with few output tiles leaves most of the 256 CUs idle (1000 x 1000 x 1000 has 64 tiles), and the one block a
+// CU does get runs a long K loop with nothing to overlap its loads; a tile count just above a multiple of what the chip holds
+// (3000^3: 576 tiles on 1024 block slots) wastes most of its last round.  Such a product is cut along K into `splits` chunks
+// that run as one more (innermost) batch dimension, each writing an M x N partial to the stream's workspace;
+// gemm_split_finish_kernel adds the partials in chunk order (deterministic, no float atomics) and stores, or accumulates into,
+// the target through its strides.
+//
+// The number of chunks minimises a cost model fitted to measurements on MI355X.  A CU that holds r blocks at once takes
+// t(r) = t0 + t1 * r microseconds per K step (fp32, K step 16: 1.9 us for one block, 5.2 us for four; fp64, K step 8: 2.0 us and
+// 2.5 us for two), a block costs about 2.7 K steps of prologue and epilogue, and the partials cost one launch plus their bytes
+// written and read back at about 5 TB/s.  The model reproduces 1000^3, 2000^3 and 3000^3 at 1 to 16 chunks within 6 %.
+template <class T>
+int64_t choose_k_splits(int64_t blocks, int64_t steps, int64_t out_elems) {
+    constexpr int R = sizeof(T) == 4 ? 4 : 2;                      // blocks a CU holds (registers and LDS)
+    constexpr double t0 = sizeof(T) == 4 ? 0.8 : 1.44, t1 = sizeof(T) == 4 ? 1.1 : 0.53;
+    constexpr int64_t kMinSteps = 4;
+    const int64_t cus = device_cus();
+    const int64_t max_splits = steps / kMinSteps;
+    auto cost = [&](int64_t sp) {
+        const int64_t chunk = (steps + sp - 1) / sp;
+        const int64_t real = (steps + chunk - 1) / chunk;          // chunks that are not empty
+        const int64_t per_cu = (blocks * real + cus - 1) / cus;
+        const int64_t rest = per_cu % R;
+        const double step_us = (double)(per_cu / R) * (t0 + t1 * R) + (rest ? t0 + t1 * (double)rest : 0.0);
+        double us = step_us * ((double)chunk + 2.7);
+        if (real > 1) us += 3.0 + (double)real * (double)out_elems * sizeof(T) * 2.0 / 5.0e6;
+        return us;
+    };
+    int64_t best = 1;
+    double best_us = cost(1);
+    for (int64_t k = 1; k <= 16; k++) {                            // the largest chunk count that keeps k blocks per CU
+        const int64_t sp = std::min(max_splits, cus * k / blocks);
+        if (sp < 2) continue;
+        const double us = cost(sp);
+        if (us < best_us * 0.97) {                                 // a split must pay for itself
+            best_us = us;
+            best = sp;
+        }
+    }
+    return best;
+}
+
+// One wavefront covers 64 consecutive output elements (coalesced along n); the SG wavefronts of a block take the chunks
+// s = w, w + SG, ... of those elements, and wavefront 0 adds the SG sums in index order: the result depends on (splits, SG) only.
+template <class T, bool ACC, int SG>
+__global__ __launch_bounds__(64 * SG) void gemm_split_finish_kernel(T* __restrict__ c, const T* __restrict__ ws, GemmArgs g, uint32_t splits, uint32_t total) {
+    __shared__ T red[SG][64];
+    const uint32_t lane = threadIdx.x % 64u, w = threadIdx.x / 64u;
+    const uint32_t e = blockIdx.x * 64u + lane;
+    const uint32_t N = (uint32_t)g.N, M = (uint32_t)g.M;
+    const uint32_t n = e % N, r = e / N, m = r % M;
+    uint32_t bl = r / M;
+    T sum = T(0);
+    if (e < total) {
+        const size_t mn = (size_t)M * N;
+        const T* p = ws + ((size_t)bl * splits * M + m) * N + n;
+        for (uint32_t s = w; s < splits; s += SG) sum += p[s * mn];
+    }
+    red[w][lane] = sum;
+    __syncthreads();
+    if (w != 0 || e >= total) return;
+#pragma unroll
+    for (int i = 1; i < SG; i++) sum += red[i][lane];
+    int64_t oc = (int64_t)m * g.scm + (int64_t)n * g.scn;
+    for (int d = g.nbatch - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bl / g.bshape[d];
+        oc += (int64_t)(bl - q * g.bshape[d]) * g.bsc[d];
+        bl = q;
+    }
+    c[oc] = ACC ? c[oc] + sum : sum;
+}
+
 template <class T>
 int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hipStream_t stream) {
-    const int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
+    int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
     if (blocks == 0) return DNH_OK;
     if (blocks > 0x7FFFFFFF) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: too many output tiles");
-    g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
     constexpr int V = 16 / (int)sizeof(T);
     bool fast = g.sak == 1 && g.sbn == 1 && g.K > 0 &&
                 (g.sam % V) == 0 && (g.sbk % V) == 0 && aligned_to(a, 16) && aligned_to(b, 16);
     for (int d = 0; d < g.nbatch && fast; d++) fast = (g.bsa[d] % V) == 0 && (g.bsb[d] % V) == 0;
+
+    const GemmArgs orig = g;
+    T* target = c;
+    int64_t splits = 1;
+    if (g.nbatch < DNH_MAX_DIMS && blocks <= 4 * (int64_t)device_cus()) {
+        const int64_t steps = (g.K + kBK<T> - 1) / kBK<T>;
+        const int64_t want = choose_k_splits<T>(blocks, steps, batch * g.M * g.N);
+        const int64_t kchunk = ((steps + want - 1) / want) * kBK<T>;
+        splits = (g.K + kchunk - 1) / kchunk;
+        if (splits > 1) {
+            T* ws = nullptr;
+            DNH_TRY(workspace(stream, sizeof(T) * (size_t)batch * splits * g.M * g.N, (void**)&ws));
+            int64_t inner = splits * g.M * g.N;       // workspace layout [batch...][split][M][N]
+            for (int d = g.nbatch - 1; d >= 0; d--) {
+                g.bsc[d] = inner;
+                inner *= g.bshape[d];
+            }
+            g.bshape[g.nbatch] = (uint32_t)splits;
+            g.bsa[g.nbatch] = kchunk * g.sak;
+            g.bsb[g.nbatch] = kchunk * g.sbk;
+            g.bsc[g.nbatch] = g.M * g.N;
+            g.nbatch++;
+            g.kchunk = kchunk;
+            g.scm = g.N;
+            g.scn = 1;
+            g.accumulate = 0;
+            c = ws;
+            blocks *= splits;
+        }
+    }
+    g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
     if (g.accumulate) {
         if (fast) hipLaunchKernelGGL((gemm_kernel<T, true, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
         else hipLaunchKernelGGL((gemm_kernel<T, false, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
@@ -309,6 +414,18 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         else hipLaunchKernelGGL((gemm_kernel<T, false, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
     }
     DNH_LAUNCH_CHECK();
+    if (splits > 1) {
+        const uint32_t total = (uint32_t)(batch * orig.M * orig.N);   // at most 4 tiles per CU: fits 32 bits
+        const unsigned fb = (unsigned)cdiv((int64_t)total, 64);
+#define DNH_FINISH(ACCF, SGV) hipLaunchKernelGGL((gemm_split_finish_kernel<T, ACCF, SGV>), dim3(fb), dim3(64 * SGV), 0, stream, target, (const T*)c, orig, (uint32_t)splits, total)
+        if (splits >= 32) {
+            if (orig.accumulate) DNH_FINISH(true, 16); else DNH_FINISH(false, 16);
+        } else {
+            if (orig.accumulate) DNH_FINISH(true, 4); else DNH_FINISH(false, 4);
+        }
+#undef DNH_FINISH
+        DNH_LAUNCH_CHECK();
+    }
     return DNH_OK;
 }
 

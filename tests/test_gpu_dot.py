@@ -56,6 +56,37 @@ def test_vecvec_matvec(H, G, rng, dt):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("shape_a,shape_b", [
+    ((700, 900), (900, 650)),          # few tiles, long K: K is cut into chunks, the last one ragged
+    ((128, 20000), (20000, 128)),      # one tile, many chunks (the wide finish)
+    ((130, 4099), (4099, 70)),         # edge tiles in m and n, K not a multiple of the K step
+    ((3, 2, 100, 1500), (3, 2, 1500, 60)),   # batch dimensions in front of the chunk dimension
+])
+def test_split_k(H, G, rng, dt, shape_a, shape_b):
+    """Products with few output tiles are cut along K and their partials added in chunk order: same bound as the uncut product,
+    for contiguous operands, for transposed views (the strided kernel) and for a strided target."""
+    a = rng.standard_normal(shape_a).astype(dt)
+    b = rng.standard_normal(shape_b).astype(dt)
+    ref, got = both(H, G, lambda a, b: a @ b, a, b)
+    check_dot(ref, got, a, b)
+    at = np.ascontiguousarray(np.swapaxes(a, -1, -2))
+    bt = np.ascontiguousarray(np.swapaxes(b, -1, -2))
+    ref, got = both(H, G, lambda a, b: a.T @ b.T, at, bt)
+    check_dot(ref, got, a, b)
+
+    def into_transposed_target(a, b):
+        shp = list(a.Shape[:-2]) + [b.Shape[-1], a.Shape[-2]]
+        t = type(a).new(shp, a.Dev, a.DataType)
+        t.T.FillDot(a, b)
+        return t
+    ref, got = both(H, G, into_transposed_target, a, b)
+    check_dot(np.swapaxes(ref, -1, -2), np.swapaxes(got, -1, -2), a, b)
+    # the same call twice gives the same bits (fixed chunk order, no atomics)
+    ta, tb = G.ofNumpy(a), G.ofNumpy(b)
+    assert np.array_equal(G.toNumpy(ta @ tb), G.toNumpy(ta @ tb))
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_batched_equals_loop_and_broadcast(H, G, rng, dt):
     # Tensor.Test/BaseTests.fs:84-96: a batched product equals the loop of 2-d products
     a = rng.standard_normal((3, 4, 128, 48)).astype(dt)
