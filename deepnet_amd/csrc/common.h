@@ -8,6 +8,7 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <string>
 
 #include "../../include/tensor_hip.h"
@@ -48,9 +49,26 @@ inline int32_t fail(int32_t code, const char* fmt, ...) {
 int32_t ensure_init();                       // DNH_ERR_NOT_INITIALIZED-free lazy init on the current device
 int device_cus();                            // compute units of the active device
 int32_t error_flag_ptr(hipStream_t stream, int32_t** out);   // the stream's device int32 set by gather/scatter kernels on a bad index
-// Per-stream scratch buffer owned by the library (partials of two-pass reductions, block counts of compactions).
-// Kernels on one stream are ordered, so one buffer per stream is race-free; it grows on demand.
-int32_t workspace(hipStream_t stream, size_t bytes, void** out);
+// Per-stream scratch buffer owned by the library (partials of two-pass reductions and split products, block counts of
+// compactions); it grows on demand.  Kernels of one stream run in order, so the buffer is free again as soon as the kernels that
+// use it are queued; the lease keeps other host threads that enqueue on the same stream out until then.  Declare the lease in the
+// scope that issues every launch touching the buffer; asking twice with one lease is fine.
+class WorkspaceLease {
+public:
+    WorkspaceLease() = default;
+    WorkspaceLease(const WorkspaceLease&) = delete;
+    WorkspaceLease& operator=(const WorkspaceLease&) = delete;
+    ~WorkspaceLease() { release(); }
+    void release() {
+        if (held_) held_->unlock();
+        held_ = nullptr;
+    }
+
+private:
+    friend int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease);
+    std::mutex* held_ = nullptr;
+};
+int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease);
 
 // ---- dtypes -----------------------------------------------------------------------------------------------------------
 

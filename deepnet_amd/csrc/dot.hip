@@ -377,6 +377,7 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
     for (int d = 0; d < g.nbatch && fast; d++) fast = (g.bsa[d] % V) == 0 && (g.bsb[d] % V) == 0;
 
     const GemmArgs orig = g;
+    WorkspaceLease lease;   // covers the product and its finishing launch
     T* target = c;
     int64_t splits = 1;
     if (g.nbatch < DNH_MAX_DIMS && blocks <= 4 * (int64_t)device_cus()) {
@@ -386,7 +387,7 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         splits = (g.K + kchunk - 1) / kchunk;
         if (splits > 1) {
             T* ws = nullptr;
-            DNH_TRY(workspace(stream, sizeof(T) * (size_t)batch * splits * g.M * g.N, (void**)&ws));
+            DNH_TRY(workspace(stream, sizeof(T) * (size_t)batch * splits * g.M * g.N, (void**)&ws, lease));
             int64_t inner = splits * g.M * g.N;       // workspace layout [batch...][split][M][N]
             for (int d = g.nbatch - 1; d >= 0; d--) {
                 g.bsc[d] = inner;
@@ -571,6 +572,7 @@ bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t strea
     const int cus = device_cus();
     constexpr int V = 16 / (int)sizeof(T);
     T* partial = nullptr;
+    WorkspaceLease lease;
     if (g.sak == 1 || g.M == 1) {
         const bool vec = g.sak == 1 && g.sbk == 1 && (g.sam % V) == 0 && aligned_to(a, 16) && aligned_to(x, 16);
         const int v = vec ? V : 1;
@@ -589,7 +591,7 @@ bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t strea
                 splits = (uint32_t)((g.K + chunk - 1) / chunk);
             }
         }
-        if (splits > 1 && (*status = workspace(stream, sizeof(T) * (size_t)M * splits, (void**)&partial)) != DNH_OK) return true;
+        if (splits > 1 && (*status = workspace(stream, sizeof(T) * (size_t)M * splits, (void**)&partial, lease)) != DNH_OK) return true;
         const dim3 grid((unsigned)row_blocks, splits);
 #define DNH_GEMV(VV, TPR) hipLaunchKernelGGL((gemv_rows_kernel<T, VV, TPR>), grid, dim3(kBlock), 0, stream, y, partial, a, x, M, g.K, g.sam, g.sak, g.sbk, g.scm, chunk, splits)
         if (vec) { if (tpr == 256) DNH_GEMV(V, 256); else if (tpr == 64) DNH_GEMV(V, 64); else DNH_GEMV(V, 16); }
@@ -612,7 +614,7 @@ bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t strea
             }
         }
         if (splits > 65535) return false;
-        if (splits > 1 && (*status = workspace(stream, sizeof(T) * (size_t)M * splits, (void**)&partial)) != DNH_OK) return true;
+        if (splits > 1 && (*status = workspace(stream, sizeof(T) * (size_t)M * splits, (void**)&partial, lease)) != DNH_OK) return true;
         const int64_t total = mblocks * splits;
         if (total > 0x7FFFFFFF) return false;
         // measured: +4 % when the m blocks map one-to-one onto the XCDs (8 blocks), -2 % with 16 blocks, so only the former is re-numbered

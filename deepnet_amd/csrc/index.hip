@@ -404,7 +404,8 @@ int32_t run_compaction_fast(const uint8_t* mask, void* full, void* out, int64_t 
     const uint32_t nout = (uint32_t)(nout64 > (int64_t)kMaxItems ? kMaxItems : nout64);
     const uint32_t nb = cdiv(nvec, kFastJ * kBlock);
     uint32_t* counts;
-    DNH_TRY(workspace(stream, sizeof(uint32_t) * (size_t)nb, (void**)&counts));
+    WorkspaceLease lease;
+    DNH_TRY(workspace(stream, sizeof(uint32_t) * (size_t)nb, (void**)&counts, lease));
     hipLaunchKernelGGL(compact_count_fast_kernel<VEC>, dim3(nb), dim3(kBlock), 0, stream, mask, nvec, counts);
     DNH_LAUNCH_CHECK();
     if (nb <= 8192) {
@@ -443,7 +444,8 @@ int32_t run_compaction(const MaskArgs& m, void* full, void* out, const Lay& olay
     const uint32_t nout = (uint32_t)(nout64 > (int64_t)kMaxItems ? kMaxItems : nout64);
     const uint32_t nb = cdiv(n, kChunk);
     uint32_t* counts;
-    DNH_TRY(workspace(stream, sizeof(uint32_t) * (size_t)nb, (void**)&counts));
+    WorkspaceLease lease;
+    DNH_TRY(workspace(stream, sizeof(uint32_t) * (size_t)nb, (void**)&counts, lease));
     hipLaunchKernelGGL(compact_count_kernel, dim3(nb), dim3(kBlock), 0, stream, m, n, counts);
     DNH_LAUNCH_CHECK();
     hipLaunchKernelGGL(compact_scan_kernel, dim3(1), dim3(kBlock), 0, stream, counts, nb);

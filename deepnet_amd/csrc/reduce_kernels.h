@@ -335,7 +335,8 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
             }
         }
         State* partial = nullptr;
-        if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial));
+        WorkspaceLease lease;
+        if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial, lease));
         const dim3 grid((unsigned)row_blocks, splits);
 #define DNH_ROWS(V, TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, V, TPR, false>), grid, dim3(kBlock), 0, stream, r, (const void*)src, out, partial, o, nout, n, sr, chunk, splits)
         if (vec) {
@@ -398,7 +399,8 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         const int64_t total_blocks = base_blocks * splits;
         if (total_blocks <= 0x7FFFFFFF) {
             State* partial = nullptr;
-            if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial));
+            WorkspaceLease lease;
+            if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial, lease));
             const dim3 grid((unsigned)total_blocks);
             const uint32_t xcd_chunk = (total_blocks % 8 == 0 && total_blocks >= 64) ? (uint32_t)(total_blocks / 8) : 0u;
 #define DNH_COLS(V, W) hipLaunchKernelGGL((reduce_cols_kernel<R, V, W>), grid, dim3(kBlock), 0, stream, r, src, out, partial, oo, col_tiles, (uint32_t)base_blocks, xcd_chunk, nc, tc_stride, n, sr, chunk, splits)

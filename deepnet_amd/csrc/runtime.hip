@@ -19,6 +19,7 @@ int g_cus = 256;
 std::map<hipStream_t, int32_t*> g_error_flags;   // one index-error word per stream, so concurrent streams do not see each other's errors
 
 struct Workspace {
+    std::mutex in_use;   // held through a WorkspaceLease while an entry point queues the kernels that use the buffer
     void* ptr = nullptr;
     size_t bytes = 0;
 };
@@ -102,22 +103,30 @@ int32_t error_flag_ptr(hipStream_t stream, int32_t** out) {
     return DNH_OK;
 }
 
-int32_t workspace(hipStream_t stream, size_t bytes, void** out) {
-    std::lock_guard<std::mutex> lock(g_mu);
-    Workspace& w = g_ws[stream];
-    if (w.bytes < bytes) {
-        if (w.ptr) {
+int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease) {
+    Workspace* w;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        w = &g_ws[stream];   // map nodes do not move
+    }
+    if (lease.held_ != &w->in_use) {
+        lease.release();
+        w->in_use.lock();
+        lease.held_ = &w->in_use;
+    }
+    if (w->bytes < bytes) {
+        if (w->ptr) {
             // work that still reads the old buffer is ordered before the free by synchronising the stream
             DNH_HIP(hipStreamSynchronize(stream));
-            DNH_HIP(hipFree(w.ptr));
-            w.ptr = nullptr;
-            w.bytes = 0;
+            DNH_HIP(hipFree(w->ptr));
+            w->ptr = nullptr;
+            w->bytes = 0;
         }
         size_t want = bytes < (size_t)(4 << 20) ? (size_t)(4 << 20) : bytes + bytes / 2;
-        DNH_HIP(hipMalloc(&w.ptr, want));
-        w.bytes = want;
+        DNH_HIP(hipMalloc(&w->ptr, want));
+        w->bytes = want;
     }
-    *out = w.ptr;
+    *out = w->ptr;
     return DNH_OK;
 }
 

@@ -18,7 +18,8 @@
  *    DNH_ERR_INVALID_ARG on a mismatch;
  *  - `stream` is a hipStream_t passed as void* (NULL = the default stream); all ops are asynchronous with
  *    respect to the host unless stated otherwise;
- *  - all entry points may be called from any thread.
+ *  - all entry points may be called from any thread, also several threads on one stream at once: scratch memory
+ *    the library keeps per stream is held by one call until the kernels that use it are queued.
  */
 #ifndef TENSOR_HIP_H
 #define TENSOR_HIP_H

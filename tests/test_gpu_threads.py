@@ -61,6 +61,51 @@ def test_concurrent_threads_on_their_own_streams(G, H):
             np.testing.assert_array_equal(ref, g)
 
 
+def test_concurrent_threads_sharing_one_stream(G, H):
+    """Host threads that never set Cfg.Stream all enqueue on the default stream and so share its workspace: an entry point keeps
+    the buffer to itself until every kernel that uses it is queued, so split folds, compactions and split products of different
+    threads cannot read each other's partials."""
+    nthreads, rounds = 4, 8
+    rng = np.random.default_rng(11)
+    inputs = [(rng.integers(-1000, 1000, (512, 640)).astype(np.int32),
+               rng.standard_normal((96, 2048)).astype(np.float64)) for _ in range(nthreads)]
+
+    def chain(M, a, f):
+        x, y = M.ofNumpy(a), M.ofNumpy(f)
+        out = []
+        for r in range(rounds):
+            x = x + r
+            out.append(M.toNumpy(x.sumAxis(0)))                        # column fold, partials + finishing pass
+            out.append(M.toNumpy(x.flatten().maxAxis(0)))              # long row, split
+            out.append(M.toNumpy(x.flatten().M((x > 0).flatten())))    # compaction, block counts
+            out.append(M.toNumpy(y @ y.T))                             # 96 x 2048 x 96: one tile, K cut into chunks
+        return out
+
+    want = [chain(H, a, f) for a, f in inputs]
+    got = [None] * nthreads
+    errors = []
+
+    def worker(i):
+        try:
+            got[i] = chain(G, *inputs[i])
+        except Exception as e:  # noqa: BLE001
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(nthreads)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    for i in range(nthreads):
+        assert got[i] is not None
+        for k, (ref, g) in enumerate(zip(want[i], got[i])):
+            if k % 4 == 3:   # the fp64 product: summation order differs from the oracle's
+                np.testing.assert_allclose(g, ref, rtol=0, atol=1e-9)
+            else:
+                np.testing.assert_array_equal(ref, g)
+
+
 def test_index_error_flag_is_per_stream(G):
     """An out-of-range gather index on one stream is reported on that stream only."""
     lib = native.load()
