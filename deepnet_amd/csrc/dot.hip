@@ -37,8 +37,8 @@ struct GemmArgs {
     int64_t kchunk;                               // > 0: the innermost batch dimension walks K in chunks of this many (split K)
 };
 
-template <class T, bool FAST, bool ACC>
-__global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void gemm_kernel(T* __restrict__ c, const T* __restrict__ a, const T* __restrict__ b, GemmArgs g) {
+template <class T, bool FAST, bool ACC, bool SPLIT>
+__global__ __launch_bounds__(kBlock, (sizeof(T) == 4 && FAST ? 4 : 2)) void gemm_kernel(T* __restrict__ c, const T* __restrict__ a, const T* __restrict__ b, GemmArgs g) {
     constexpr int BK = kBK<T>;
     __shared__ __align__(16) T As[2][BK][BM + PAD];
     __shared__ __align__(16) T Bs[2][BK][BN + PAD];
@@ -53,7 +53,7 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
     const uint32_t tm = bid % g.tiles_m;
     bid /= g.tiles_m;
     int64_t oa = 0, ob = 0, oc = 0;
-    int64_t K = g.K;  // this block's extent along k: a chunk of it when K is split
+    uint32_t chunk_id = 0;
     for (int d = g.nbatch - 1; d >= 0; d--) {
         const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
         const uint32_t i = bid - q * g.bshape[d];
@@ -61,8 +61,10 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
         oa += (int64_t)i * g.bsa[d];
         ob += (int64_t)i * g.bsb[d];
         oc += (int64_t)i * g.bsc[d];
-        if (d == g.nbatch - 1 && g.kchunk > 0) K = min(g.kchunk, g.K - (int64_t)i * g.kchunk);
+        if (SPLIT && d == g.nbatch - 1) chunk_id = i;
     }
+    // this block's extent along k: the whole of K, or one chunk of it (SPLIT: the innermost batch dimension counts the chunks)
+    const int64_t K = SPLIT ? min(g.kchunk, g.K - (int64_t)chunk_id * g.kchunk) : g.K;
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     a += oa;
     b += ob;
@@ -72,6 +74,7 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
     // global -> register staging
     constexpr int SPT = BM * BK / kBlock;  // elements of each tile per thread
     T ra[SPT], rb[SPT];
+    uint32_t amask = 0, bmask = 0;  // element loads: bit i = ra[i] / rb[i] lies inside the matrix (else it is stored as zero)
 
     const bool full_mn = m0 + BM <= g.M && n0 + BN <= g.N;
     // load_tiles(k0, buf) fetches the tiles of K step k0 and says where they are: kVec / kScalar = in registers (ra/rb, in the
@@ -131,19 +134,41 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
                 }
             }
             return kDirect;
+        } else if (full_mn && k0 + BK <= K) {
+            // whole K step of an interior tile: every element exists
+            amask = ~0u;
+            bmask = ~0u;
+#pragma unroll
+            for (int i = 0; i < SPT; i++) {
+                const int idx = tid + i * kBlock;
+                ra[i] = a[(m0 + idx / BK) * g.sam + (k0 + idx % BK) * g.sak];
+                rb[i] = b[(k0 + idx / BN) * g.sbk + (n0 + idx % BN) * g.sbn];
+            }
+            return kScalar;
         } else {
+            amask = 0;
+            bmask = 0;
 #pragma unroll
             for (int i = 0; i < SPT; i++) {
                 const int idx = tid + i * kBlock;
                 {
                     const int row = idx / BK, kk = idx % BK;
                     const int64_t m = m0 + row, k = k0 + kk;
-                    ra[i] = (m < g.M && k < K) ? a[m * g.sam + k * g.sak] : T(0);
+                    // Unconditional load from an address clamped to element (0, 0); whether the element counts is kept as one
+                    // bit and applied when the registers go to LDS, after the MFMAs of the current step.  The loads of a thread
+                    // are then issued back to back and nothing waits for them before the MFMA chain (`cond ? load : 0` leaves
+                    // the compiler free to branch around every load or to select right after it, and which one it picked
+                    // changed with unrelated edits: fp64 edge tiles ran 20 % slower when it did).
+                    const bool ok = m < g.M && k < K;
+                    ra[i] = a[ok ? m * g.sam + k * g.sak : 0];
+                    amask |= (uint32_t)ok << i;
                 }
                 {
                     const int kk = idx / BN, col = idx % BN;
                     const int64_t k = k0 + kk, n = n0 + col;
-                    rb[i] = (k < K && n < g.N) ? b[k * g.sbk + n * g.sbn] : T(0);
+                    const bool ok = k < K && n < g.N;
+                    rb[i] = b[ok ? k * g.sbk + n * g.sbn : 0];
+                    bmask |= (uint32_t)ok << i;
                 }
             }
             return kScalar;
@@ -178,8 +203,8 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
 #pragma unroll
             for (int i = 0; i < SPT; i++) {
                 const int idx = tid + i * kBlock;
-                As[buf][idx % BK][idx / BK] = ra[i];
-                Bs[buf][idx / BN][idx % BN] = rb[i];
+                As[buf][idx % BK][idx / BK] = ((amask >> i) & 1u) ? ra[i] : T(0);
+                Bs[buf][idx / BN][idx % BN] = ((bmask >> i) & 1u) ? rb[i] : T(0);
             }
         }
     };
@@ -196,8 +221,11 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
 #pragma unroll
                 for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
 
-        int vl = load_tiles(0, 0);
-        store_tiles(0, vl);
+        int vl = kDirect;
+        if (FAST || K > 0) {  // (the fast kernel is only launched with K > 0) an empty inner dimension has no element to fetch (not even the clamped one): the target becomes zeros
+            vl = load_tiles(0, 0);
+            store_tiles(0, vl);
+        }
         __syncthreads();
         int cur = 0;
         const int lk = lane >> 5, lm = lane & 31;
@@ -253,8 +281,11 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 ? (FAST ? 4 : 3) : 2)) void
             for (int j = 0; j < 4; j++)
 #pragma unroll
                 for (int r = 0; r < 4; r++) acc[i][j][r] = 0.0;
-        int vl = load_tiles(0, 0);
-        store_tiles(0, vl);
+        int vl = kDirect;
+        if (FAST || K > 0) {  // (the fast kernel is only launched with K > 0) an empty inner dimension has no element to fetch (not even the clamped one): the target becomes zeros
+            vl = load_tiles(0, 0);
+            store_tiles(0, vl);
+        }
         __syncthreads();
         int cur = 0;
         const int lk = lane >> 4, lm = lane & 15;
@@ -312,6 +343,7 @@ int64_t choose_k_splits(int64_t blocks, int64_t steps, int64_t out_elems) {
     constexpr int64_t kMinSteps = 4;
     const int64_t cus = device_cus();
     const int64_t max_splits = steps / kMinSteps;
+    if (max_splits < 2) return 1;                                  // also the empty inner dimension (no steps)
     auto cost = [&](int64_t sp) {
         const int64_t chunk = (steps + sp - 1) / sp;
         const int64_t real = (steps + chunk - 1) / chunk;          // chunks that are not empty
@@ -380,9 +412,9 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
     WorkspaceLease lease;   // covers the product and its finishing launch
     T* target = c;
     int64_t splits = 1;
-    if (g.nbatch < DNH_MAX_DIMS && blocks <= 4 * (int64_t)device_cus()) {
-        const int64_t steps = (g.K + kBK<T> - 1) / kBK<T>;
-        const int64_t want = choose_k_splits<T>(blocks, steps, batch * g.M * g.N);
+    const int64_t steps = (g.K + kBK<T> - 1) / kBK<T>;
+    const int64_t want = (g.nbatch < DNH_MAX_DIMS && blocks <= 4 * (int64_t)device_cus()) ? choose_k_splits<T>(blocks, steps, batch * g.M * g.N) : 1;
+    if (want > 1) {   // implies steps >= 8: the chunk below is not empty
         const int64_t kchunk = ((steps + want - 1) / want) * kBK<T>;
         splits = (g.K + kchunk - 1) / kchunk;
         if (splits > 1) {
@@ -407,13 +439,15 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         }
     }
     g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
-    if (g.accumulate) {
-        if (fast) hipLaunchKernelGGL((gemm_kernel<T, true, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
-        else hipLaunchKernelGGL((gemm_kernel<T, false, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+#define DNH_GEMM(FASTF, ACCF, SPLITF) hipLaunchKernelGGL((gemm_kernel<T, FASTF, ACCF, SPLITF>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g)
+    if (splits > 1) {
+        if (fast) DNH_GEMM(true, false, true); else DNH_GEMM(false, false, true);
+    } else if (g.accumulate) {
+        if (fast) DNH_GEMM(true, true, false); else DNH_GEMM(false, true, false);
     } else {
-        if (fast) hipLaunchKernelGGL((gemm_kernel<T, true, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
-        else hipLaunchKernelGGL((gemm_kernel<T, false, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+        if (fast) DNH_GEMM(true, false, false); else DNH_GEMM(false, false, false);
     }
+#undef DNH_GEMM
     DNH_LAUNCH_CHECK();
     if (splits > 1) {
         const uint32_t total = (uint32_t)(batch * orig.M * orig.N);   // at most 4 tiles per CU: fits 32 bits

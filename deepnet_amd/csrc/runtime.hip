@@ -12,7 +12,7 @@ namespace dnh {
 
 namespace {
 std::mutex g_mu;
-std::atomic<uint64_t> g_epoch{1};   // bumped whenever the active device changes
+std::atomic<uint64_t> g_epoch{1};   // bumped when the device is chosen
 bool g_init = false;
 int g_device = 0;
 int g_cus = 256;
@@ -63,6 +63,7 @@ std::string& last_error() {
 
 static int32_t init_locked(int device) {
     if (g_init && device == g_device) return DNH_OK;
+    if (g_init) return fail(DNH_ERR_INVALID_ARG, "dnh_init: the library already runs on device %d; it cannot move to device %d", g_device, device);
     int count = 0;
     hipError_t e = hipGetDeviceCount(&count);
     if (e != hipSuccess || count == 0) return fail(DNH_ERR_HIP, "no HIP device available (%s)", hipGetErrorString(e));
@@ -78,8 +79,8 @@ static int32_t init_locked(int device) {
 }
 
 int32_t ensure_init() {
-    // HIP's current device is per host thread: the first call of a thread (and the first after dnh_init selected another
-    // device) binds the thread to our device; later calls cost one thread-local compare.
+    // HIP's current device is per host thread: the first call of a thread binds the thread to the library's device; later
+    // calls cost one thread-local compare.
     thread_local int t_bound_device = -1;
     thread_local uint64_t t_bound_epoch = 0;
     if (t_bound_device >= 0 && t_bound_epoch == g_epoch.load(std::memory_order_acquire)) return DNH_OK;
@@ -315,6 +316,7 @@ int32_t dnh_host_alloc(size_t bytes, void** out) {
 
 int32_t dnh_host_free(void* ptr) {
     if (!ptr) return DNH_OK;
+    DNH_TRY(ensure_init());
     DNH_HIP(hipHostFree(ptr));
     return DNH_OK;
 }
@@ -356,6 +358,7 @@ int32_t dnh_stream_create(void** stream) {
 
 int32_t dnh_stream_destroy(void* stream) {
     if (!stream) return DNH_OK;
+    DNH_TRY(ensure_init());
     DNH_HIP(hipStreamSynchronize((hipStream_t)stream));
     drop_workspace((hipStream_t)stream);
     {
@@ -395,19 +398,23 @@ int32_t dnh_event_create(void** event) {
 }
 int32_t dnh_event_destroy(void* event) {
     if (!event) return DNH_OK;
+    DNH_TRY(ensure_init());
     DNH_HIP(hipEventDestroy((hipEvent_t)event));
     return DNH_OK;
 }
 int32_t dnh_event_record(void* event, void* stream) {
+    DNH_TRY(ensure_init());
     DNH_HIP(hipEventRecord((hipEvent_t)event, (hipStream_t)stream));
     return DNH_OK;
 }
 int32_t dnh_event_sync(void* event) {
+    DNH_TRY(ensure_init());
     DNH_HIP(hipEventSynchronize((hipEvent_t)event));
     return DNH_OK;
 }
 int32_t dnh_event_elapsed_ms(void* start, void* stop, float* ms) {
     if (!ms) return fail(DNH_ERR_INVALID_ARG, "dnh_event_elapsed_ms: null argument");
+    DNH_TRY(ensure_init());
     DNH_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
     return DNH_OK;
 }

@@ -131,6 +131,10 @@ typedef enum DnhArgReduceOp { DNH_ARG_MIN = 0, DNH_ARG_MAX = 1 } DnhArgReduceOp;
 /* ---------------------------------------------------------------------------------------------------
  * Device, errors                                     (replaces Cuda/CudaUtils.fs:36-60 context creation)
  * ------------------------------------------------------------------------------------------------- */
+/* Selects the device every later call of this process runs on (the reference likewise creates one context on the
+ * first device it finds, Cuda/CudaUtils.fs:36-60).  Optional: the first other call initialises device 0.  Calling it
+ * again with the same device is a no-op; another device is refused with DNH_ERR_INVALID_ARG, since buffers, cached
+ * blocks and workspaces already belong to the first one. */
 int32_t dnh_init(int32_t device);
 int32_t dnh_device_info(DnhDeviceInfo* info);
 /* Copies the calling thread's last error message (NUL terminated, truncated to n). */

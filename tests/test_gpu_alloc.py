@@ -108,3 +108,16 @@ def test_storage_used_on_two_streams_takes_the_synchronising_free(G):
         del y
     finally:
         native.check(lib.dnh_stream_destroy(s))
+
+
+def test_device_is_chosen_once(G):
+    """dnh_init with the device in use is a no-op; any other device is refused, since buffers, cached blocks and workspaces
+    already live on the first one."""
+    lib = native.load()
+    assert lib.dnh_init(0) == abi.DNH_OK
+    assert lib.dnh_init(1) == abi.DNH_ERR_INVALID_ARG
+    buf = C.create_string_buffer(256)
+    lib.dnh_last_error(buf, 256)
+    assert b"device" in buf.value
+    x = G.ofNumpy(np.arange(6, dtype=np.int32))
+    assert G.toNumpy(x + x).tolist() == [0, 2, 4, 6, 8, 10]

@@ -34,6 +34,25 @@ def test_matmat(H, G, rng, dt, m, k, n):
     check_dot(ref, got, a, b)
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_empty_dimensions(H, G, dt):
+    """An empty inner dimension gives zeros (an empty sum), empty outer dimensions give an empty result; nothing is fetched."""
+    for m, k, n in [(5, 0, 7), (130, 0, 129), (0, 4, 3), (3, 4, 0)]:
+        a = np.zeros((m, k), dt)
+        b = np.zeros((k, n), dt)
+        ref, got = both(H, G, lambda a, b: a @ b, a, b)
+        assert got.shape == (m, n) and ref.shape == (m, n)
+        assert np.array_equal(got, np.zeros((m, n), dt)) and np.array_equal(ref, got)
+    a = np.zeros((2, 3, 0), dt)
+    b = np.zeros((2, 0, 4), dt)
+    ref, got = both(H, G, lambda a, b: a @ b, a, b)
+    assert np.array_equal(got, np.zeros((2, 3, 4), dt)) and np.array_equal(ref, got)
+    av = np.zeros((6, 0), dt)
+    v = np.zeros((0,), dt)
+    ref, got = both(H, G, lambda a, b: a @ b, av, v)
+    assert np.array_equal(got, np.zeros((6,), dt)) and np.array_equal(ref, got)
+
+
 def test_doc_vector(H, G):
     # Guide-Operations.md:129-148
     h = 3.0 * np.arange(5.0)[:, None] + np.arange(3.0)[None, :]
