@@ -9,6 +9,7 @@ import numpy as np
 
 HBM_PEAK_GBS = 8000.0
 FP32_MFMA_PEAK_TFLOPS = 157.3
+FP64_MFMA_PEAK_TFLOPS = 78.6
 
 
 class Timer:
@@ -47,11 +48,12 @@ def nsets_for(nbytes):
     return max(1, min(40, math.ceil(600e6 / max(nbytes, 1))))
 
 
-def report(log, cfg, name, ms, nbytes=None, flops=None):
+def report(log, cfg, name, ms, nbytes=None, flops=None, fp64=False):
     if flops:
         tf = flops / (ms * 1e-3) / 1e12
-        log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {tf:8.2f} TFLOP/s  {100 * tf / FP32_MFMA_PEAK_TFLOPS:5.1f}% of fp32 MFMA peak")
-        return {"cfg": cfg, "op": name, "ms": ms, "TFLOPs": tf, "frac": tf / FP32_MFMA_PEAK_TFLOPS}
+        peak = FP64_MFMA_PEAK_TFLOPS if fp64 else FP32_MFMA_PEAK_TFLOPS
+        log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {tf:8.2f} TFLOP/s  {100 * tf / peak:5.1f}% of {'fp64' if fp64 else 'fp32'} MFMA peak")
+        return {"cfg": cfg, "op": name, "ms": ms, "TFLOPs": tf, "frac": tf / peak}
     gb = nbytes / (ms * 1e-3) / 1e9
     log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {gb:8.1f} GB/s  {100 * gb / HBM_PEAK_GBS:5.1f}% of HBM peak  ({nbytes / 1e6:.1f} MB)")
     return {"cfg": cfg, "op": name, "ms": ms, "GBps": gb, "frac": gb / HBM_PEAK_GBS}
@@ -74,11 +76,11 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6)):
     def new(shape, dt):
         return Tensor.new(shape, G.Dev, dt)
 
-    def timed(cfg, name, nbytes, build, flops=None, reps=20):
+    def timed(cfg, name, nbytes, build, flops=None, reps=20, fp64=False):
         ns = nsets_for(nbytes)
         sets = [build(i) for i in range(ns)]
         ms = T.time(sets, reps=max(reps, ns))
-        results.append(report(log, cfg, name, ms, nbytes, flops))
+        results.append(report(log, cfg, name, ms, nbytes, flops, fp64))
         keep.clear()
 
     f32 = np.float32
@@ -222,6 +224,15 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6)):
             sm.Backend.SumLastAxis(sm, a)
             return [("binary", (abi.DNH_DIVIDE, D(c), D(a), D(sm[:, :, None].broadcastTo([Bn, n, n]))))]
         timed(5, "Divide e / rowsum (broadcast)", 2 * N * 4 + R * 4, div5)
+        # the matrix sizes of the reference's own benchmark (Tensor.Benchmark/Benchmark.fs:216): few output tiles, K is split
+        for sq in (1000, 2000, 4000):
+            for dt, sz in ((np.float32, 4), (np.float64, 8)):
+                sa = G.ofNumpy(rng.standard_normal((sq, sq)).astype(dt))
+                sb = G.ofNumpy(rng.standard_normal((sq, sq)).astype(dt))
+                sc = new([sq, sq], dt)
+                timed(5, f"MatMatDot {sq}^3 {np.dtype(dt).name}", 3 * sq * sq * sz, lambda i: [("dot", (D(sc), D(sa), D(sb)))],
+                      flops=2.0 * sq ** 3, fp64=dt is np.float64)
+                del sa, sb, sc
     if 6 in which:
         # the vector forms of dot (not one of the five configurations; bandwidth-bound)
         n = 8192

@@ -368,34 +368,50 @@ int64_t choose_k_splits(int64_t blocks, int64_t steps, int64_t out_elems) {
     return best;
 }
 
-// One wavefront covers 64 consecutive output elements (coalesced along n); the SG wavefronts of a block take the chunks
-// s = w, w + SG, ... of those elements, and wavefront 0 adds the SG sums in index order: the result depends on (splits, SG) only.
-template <class T, bool ACC, int SG>
-__global__ __launch_bounds__(64 * SG) void gemm_split_finish_kernel(T* __restrict__ c, const T* __restrict__ ws, GemmArgs g, uint32_t splits, uint32_t total) {
-    __shared__ T red[SG][64];
+// One wavefront covers 64 consecutive output vectors of VEC elements (coalesced along n); the SG wavefronts of a block take the
+// chunks s = w, w + SG, ... of those outputs, and wavefront 0 adds the SG sums in index order: the result depends on
+// (splits, SG) only.  VEC > 1 needs N % VEC == 0 and a target whose rows are contiguous and 16-byte aligned.
+template <class T, bool ACC, int SG, int VEC>
+__global__ __launch_bounds__(64 * SG) void gemm_split_finish_kernel(T* __restrict__ c, const T* __restrict__ ws, GemmArgs g, uint32_t splits, uint32_t total_vecs) {
+    __shared__ Pack<T, VEC> red[SG][64];
     const uint32_t lane = threadIdx.x % 64u, w = threadIdx.x / 64u;
     const uint32_t e = blockIdx.x * 64u + lane;
-    const uint32_t N = (uint32_t)g.N, M = (uint32_t)g.M;
-    const uint32_t n = e % N, r = e / N, m = r % M;
+    const uint32_t NV = (uint32_t)g.N / VEC, M = (uint32_t)g.M;
+    const uint32_t n = (e % NV) * VEC, r = e / NV, m = r % M;
     uint32_t bl = r / M;
-    T sum = T(0);
-    if (e < total) {
-        const size_t mn = (size_t)M * N;
-        const T* p = ws + ((size_t)bl * splits * M + m) * N + n;
-        for (uint32_t s = w; s < splits; s += SG) sum += p[s * mn];
+    Pack<T, VEC> sum = splat_pack<T, VEC>(T(0));
+    if (e < total_vecs) {
+        const size_t mn = (size_t)M * (size_t)g.N;
+        const T* p = ws + ((size_t)bl * splits * M + m) * (size_t)g.N + n;
+        for (uint32_t s = w; s < splits; s += SG) {
+            const Pack<T, VEC> v = load_pack<T, VEC>(p + s * mn);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) sum.v[k] += v.v[k];
+        }
     }
     red[w][lane] = sum;
     __syncthreads();
-    if (w != 0 || e >= total) return;
+    if (w != 0 || e >= total_vecs) return;
 #pragma unroll
-    for (int i = 1; i < SG; i++) sum += red[i][lane];
+    for (int i = 1; i < SG; i++)
+#pragma unroll
+        for (int k = 0; k < VEC; k++) sum.v[k] += red[i][lane].v[k];
     int64_t oc = (int64_t)m * g.scm + (int64_t)n * g.scn;
     for (int d = g.nbatch - 1; d >= 0; d--) {
         const uint32_t q = (d == 0) ? 0u : bl / g.bshape[d];
         oc += (int64_t)(bl - q * g.bshape[d]) * g.bsc[d];
         bl = q;
     }
-    c[oc] = ACC ? c[oc] + sum : sum;
+    if constexpr (VEC > 1) {
+        if (ACC) {
+            const Pack<T, VEC> old = load_pack<T, VEC>(c + oc);
+#pragma unroll
+            for (int k = 0; k < VEC; k++) sum.v[k] = old.v[k] + sum.v[k];
+        }
+        store_pack<T, VEC>(c + oc, sum);
+    } else {
+        c[oc] = ACC ? c[oc] + sum.v[0] : sum.v[0];
+    }
 }
 
 template <class T>
@@ -450,14 +466,19 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
 #undef DNH_GEMM
     DNH_LAUNCH_CHECK();
     if (splits > 1) {
-        const uint32_t total = (uint32_t)(batch * orig.M * orig.N);   // at most 4 tiles per CU: fits 32 bits
+        constexpr int FV = 16 / (int)sizeof(T);
+        bool vec = orig.scn == 1 && (orig.N % FV) == 0 && (orig.scm % FV) == 0 && aligned_to(target, 16);
+        for (int d = 0; d < orig.nbatch && vec; d++) vec = (orig.bsc[d] % FV) == 0;
+        const uint32_t total = (uint32_t)(batch * orig.M * orig.N / (vec ? FV : 1));   // at most 4 tiles per CU: fits 32 bits
         const unsigned fb = (unsigned)cdiv((int64_t)total, 64);
-#define DNH_FINISH(ACCF, SGV) hipLaunchKernelGGL((gemm_split_finish_kernel<T, ACCF, SGV>), dim3(fb), dim3(64 * SGV), 0, stream, target, (const T*)c, orig, (uint32_t)splits, total)
+#define DNH_FINISH(ACCF, SGV, VV) hipLaunchKernelGGL((gemm_split_finish_kernel<T, ACCF, SGV, VV>), dim3(fb), dim3(64 * SGV), 0, stream, target, (const T*)c, orig, (uint32_t)splits, total)
+#define DNH_FINISH_V(ACCF, SGV) do { if (vec) DNH_FINISH(ACCF, SGV, FV); else DNH_FINISH(ACCF, SGV, 1); } while (0)
         if (splits >= 32) {
-            if (orig.accumulate) DNH_FINISH(true, 16); else DNH_FINISH(false, 16);
+            if (orig.accumulate) DNH_FINISH_V(true, 16); else DNH_FINISH_V(false, 16);
         } else {
-            if (orig.accumulate) DNH_FINISH(true, 4); else DNH_FINISH(false, 4);
+            if (orig.accumulate) DNH_FINISH_V(true, 4); else DNH_FINISH_V(false, 4);
         }
+#undef DNH_FINISH_V
 #undef DNH_FINISH
         DNH_LAUNCH_CHECK();
     }
