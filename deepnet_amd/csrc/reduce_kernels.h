@@ -318,6 +318,9 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         // threads per row: at least four vectors per thread (measured on 16 Mi fp32: rows of 256-512 elements run 15-30 % faster
         // with 16 threads than with 64, rows of 1024-2048 fastest with 64, 4096 and longer with 256)
         int tpr = (n >= (int64_t)256 * v * 4) ? 256 : (n >= (int64_t)64 * v * 4 ? 64 : 16);
+        // few rows (1000 x 1000: 63 blocks of 16 rows for 256 CUs): widen the rows' thread groups while that leaves every thread
+        // a vector, until each CU has a block
+        while (tpr < 256 && (int64_t)nout * tpr < (int64_t)cus * kBlock && n >= (int64_t)tpr * 4 * v) tpr *= 4;
         const int rpb = kBlock / tpr;
         const int64_t row_blocks = (nout + rpb - 1) / rpb;
         uint32_t splits = 1;
