@@ -32,3 +32,22 @@ def test_cpp_frontend_against_oracle():
     out = _run("gpu")
     assert "0 failed" in out
     assert out.count("PASS parity.") >= 30 and out.count("PASS doc.") >= 40
+
+
+@pytest.mark.gpu
+def test_cpp_reference_benchmark_loop_runs():
+    """deepnet_amd/cpp/bench_suite.cpp (the reference's benchmark loop through the compiled host layer) runs every method at every
+    shape and type and prints the reference's CSV columns."""
+    exe = os.path.join(ROOT, "deepnet_amd", "cpp", "_build", "bench_suite")
+    if not os.path.exists(exe):
+        import __graft_entry__
+        __graft_entry__.build_cpp_bench()
+    p = subprocess.run([exe, "1", "0"], capture_output=True, text=True, timeout=110)
+    assert p.returncode == 0, p.stderr[-2000:]
+    lines = p.stdout.strip().splitlines()
+    assert lines[0] == "Method,Shape,Type,Dev,Mean [ms],StdDev [ms]"
+    rows = [l.split(",") for l in lines[1:]]
+    assert all(len(r) == 6 and r[3] == "Hip" and float(r[4]) > 0 for r in rows)
+    assert {r[1] for r in rows} == {"1000x1000", "2000x2000", "4000x4000"}
+    assert {r[2] for r in rows} == {"single", "double", "int32"}
+    assert {"Add", "SumAxis", "ArgMaxAxis", "MaskedGet", "Dot", "Invert"} <= {r[0] for r in rows}
