@@ -130,6 +130,40 @@ __global__ __launch_bounds__(kMaxPanelThreads) void invert_panel_kernel(T* __res
             G[(int64_t)r * NB + jj] = P[(int64_t)r * ld + kb + jj] - ((r == kb + jj) ? T(1) : T(0));
 }
 
+// Replays the row exchanges of the block of rows [kb, kb + wc), wc <= NB, on row numbers: entry i of the result says that row pos[i]
+// ends up with the content of row src[i] (the block's own rows first, then their partners outside the block; at most 2 * wc = 64
+// rows take part).  A column then needs one round of independent loads and one round of stores instead of wc dependent round
+// trips.  Run by one whole wavefront: lane j < wc passes the pivot of step j and every lane keeps entry `lane` in registers, so a
+// step is a ballot and two lane reads instead of a search through LDS (which took 40 us of a 49 us exchange kernel).
+// Writes the entries to pos[] / src[] and returns their number.
+__device__ inline int replay_exchanges_wave(int my_pivot, int kb, int wc, int lane, int* pos, int* src) {
+    int ps = lane < wc ? kb + lane : -1, sr = ps;
+    int m = wc;
+    for (int j = 0; j < wc; j++) {
+        const int p = __builtin_amdgcn_readlane(my_pivot, j);
+        if (p == kb + j) continue;
+        int ip;
+        if (p < kb + wc) {
+            ip = p - kb;
+        } else {
+            const unsigned long long hit = __ballot(lane >= wc && lane < m && ps == p);
+            if (hit) {
+                ip = __builtin_ctzll(hit);
+            } else {
+                ip = m;
+                if (lane == m) { ps = p; sr = p; }
+                m++;
+            }
+        }
+        const int sj = __builtin_amdgcn_readlane(sr, j), sip = __builtin_amdgcn_readlane(sr, ip);
+        if (lane == j) sr = sip;
+        if (lane == ip) sr = sj;
+    }
+    pos[lane] = ps;
+    src[lane] = sr;
+    return m;
+}
+
 // The same Gauss-Jordan steps on a sub-panel of sw <= CW columns held in LDS, so that the dependent chain pivot search ->
 // exchange -> pivot row -> update runs at LDS latency instead of cache round trips.  Element (r, c) of the sub-panel lives at
 // L[r * CW + c] and is owned by thread (r % rows_per_pass) * CW + c: every access of the update is linear in the thread index,
@@ -139,7 +173,8 @@ __global__ __launch_bounds__(kMaxPanelThreads) void invert_panel_kernel(T* __res
 template <class T, int CW>
 __global__ __launch_bounds__(kMaxPanelThreads) void invert_subpanel_lds_kernel(T* __restrict__ w, T* __restrict__ gsub, int32_t* __restrict__ ipiv,
                                                                                int32_t* singular, int n, int ld, int cs, int sw, int gld,
-                                                                               int64_t bs_w, int64_t bs_gs) {
+                                                                               int64_t bs_w, int64_t bs_gs, T* __restrict__ tbuf, int kb, int wc,
+                                                                               int64_t bs_t) {
     extern __shared__ __align__(16) unsigned char lds_raw[];
     T* P = w + (int64_t)blockIdx.x * bs_w;
     T* Gs = gsub + (int64_t)blockIdx.x * bs_gs;
@@ -232,6 +267,56 @@ __global__ __launch_bounds__(kMaxPanelThreads) void invert_subpanel_lds_kernel(T
             P[(int64_t)r * ld + cs + c] = v;
             Gs[(int64_t)r * gld + c] = v - ((r == cs + c) ? T(1) : T(0));
         }
+    // The sub-panel's row exchanges applied to the other columns of its panel [kb, kb + wc), and the exchanged rows cs .. cs + sw
+    // of those columns copied to T (zeros in the sub-panel's own columns) for invert_panel_update_kernel.  One thread per column:
+    // all its loads, then all its stores, so no thread reads what another one writes.
+    if (wc > sw) {
+        __shared__ int pos[2 * NB], src[2 * NB], cnt;
+        if (tid < 64) {
+            const int m = replay_exchanges_wave(tid < sw ? piv_s[tid] : 0, cs, sw, tid, pos, src);
+            if (tid == 0) cnt = m;
+        }
+        __syncthreads();
+        if (tid < wc) {
+            const int col = kb + tid;
+            T* Tb = tbuf + (int64_t)blockIdx.x * bs_t;
+            if (col >= cs && col < cs + sw) {
+                for (int j = 0; j < sw; j++) Tb[(int64_t)j * ld + col] = T(0);
+            } else {
+                const int m = cnt;
+                T val[2 * CW];
+#pragma unroll
+                for (int i = 0; i < 2 * CW; i++)
+                    if (i < m) val[i] = P[(int64_t)src[i] * ld + col];
+#pragma unroll
+                for (int i = 0; i < 2 * CW; i++)
+                    if (i < m) {
+                        if (src[i] != pos[i]) P[(int64_t)pos[i] * ld + col] = val[i];
+                        if (i < sw) Tb[(int64_t)i * ld + col] = val[i];
+                    }
+            }
+        }
+    }
+}
+
+// W[r, c] += sum_j Gs[r, j] * T[j, c] for the columns c of a panel [kb, kb + wc) outside the sub-panel [cs, cs + sw) that was just
+// eliminated (T is zero in the sub-panel's own columns, which therefore stay as they are).  One thread per row and column.
+template <class T>
+__global__ __launch_bounds__(256) void invert_panel_update_kernel(T* __restrict__ w, const T* __restrict__ gsub, const T* __restrict__ tbuf, int n,
+                                                                  int ld, int gld, int kb, int wc, int cs, int sw, int64_t bs_w, int64_t bs_gs,
+                                                                  int64_t bs_t) {
+    __shared__ T ts[NB][NB + 1];
+    const T* Tb = tbuf + (int64_t)blockIdx.y * bs_t;
+    for (int i = threadIdx.x; i < sw * wc; i += 256) ts[i / wc][i % wc] = Tb[(int64_t)(i / wc) * ld + kb + i % wc];
+    __syncthreads();
+    const int cc = threadIdx.x % NB, r = blockIdx.x * (256 / NB) + threadIdx.x / NB;
+    const int col = kb + cc;
+    if (r >= n || cc >= wc || (col >= cs && col < cs + sw)) return;
+    const T* g = gsub + (int64_t)blockIdx.y * bs_gs + (int64_t)r * gld;
+    T acc = T(0);
+    for (int j = 0; j < sw; j++) acc += g[j] * ts[j][cc];
+    T* dst = w + (int64_t)blockIdx.y * bs_w + (int64_t)r * ld + col;
+    *dst += acc;
 }
 
 // G - I_block of a panel that was processed in sub-panels.
@@ -256,28 +341,11 @@ __global__ __launch_bounds__(kSwapThreads) void invert_swap_kernel(T* __restrict
                                                                    int64_t bs_t) {
     __shared__ int pos[2 * NB];   // affected row positions: the block's rows first, then partners outside the block
     __shared__ int src[2 * NB];   // the row whose content ends up at pos[i]
-    __shared__ int pv[NB];
     __shared__ int cnt;
     const int32_t* piv = ipiv + (int64_t)blockIdx.y * n;
-    if (threadIdx.x < wc) pv[threadIdx.x] = piv[kb + threadIdx.x];
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int m = wc;
-        for (int j = 0; j < wc; j++) { pos[j] = kb + j; src[j] = kb + j; }
-        for (int j = 0; j < wc; j++) {
-            const int p = pv[j];
-            if (p == kb + j) continue;
-            int ip = -1;
-            if (p < kb + wc) {
-                ip = p - kb;
-            } else {
-                for (int q = wc; q < m; q++)
-                    if (pos[q] == p) { ip = q; break; }
-                if (ip < 0) { ip = m; pos[m] = p; src[m] = p; m++; }
-            }
-            const int t = src[j]; src[j] = src[ip]; src[ip] = t;
-        }
-        cnt = m;
+    {
+        const int m = replay_exchanges_wave(threadIdx.x < wc ? piv[kb + threadIdx.x] : 0, kb, wc, threadIdx.x, pos, src);
+        if (threadIdx.x == 0) cnt = m;
     }
     __syncthreads();
     const int c = c_begin + blockIdx.x * kSwapThreads + threadIdx.x;
@@ -392,8 +460,8 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
         auto lds_need = [&](int cw) { return (size_t)n * cw * sizeof(T); };
         int sb = 0;
         for (int cand = NB; cand >= 1; cand >>= 1)
-            if (lds_need(cand) + 1024 <= (size_t)lds_limit) { sb = cand; break; }
-        auto launch_subpanel = [&](int cw, T* g, int cs, int sw, int gld) -> int32_t {
+            if (lds_need(cand) + 2048 <= (size_t)lds_limit) { sb = cand; break; }   // 2 KB for the kernel's static arrays
+        auto launch_subpanel = [&](int cw, T* g, int cs, int sw, int gld, int pkb, int pwc) -> int32_t {
             const size_t lds = lds_need(cw);
 #define DNH_SUBPANEL(CWV)                                                                                                              \
     case CWV:                                                                                                                          \
@@ -401,7 +469,7 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
             DNH_HIP(hipFuncSetAttribute((const void*)invert_subpanel_lds_kernel<T, CWV>, hipFuncAttributeMaxDynamicSharedMemorySize,  \
                                         (int)lds));                                                                                    \
         hipLaunchKernelGGL((invert_subpanel_lds_kernel<T, CWV>), dim3((unsigned)batch), dim3(threads), lds, stream, W, g, ipiv, flag, n, ld, \
-                           cs, sw, gld, bs_w, bs_g);                                                                                   \
+                           cs, sw, gld, bs_w, bs_g, Tb, pkb, pwc, bs_t);                                                               \
         break;
             switch (cw) {
                 DNH_SUBPANEL(32) DNH_SUBPANEL(16) DNH_SUBPANEL(8) DNH_SUBPANEL(4) DNH_SUBPANEL(2) DNH_SUBPANEL(1)
@@ -412,17 +480,14 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
         for (int kb = 0; kb < n; kb += NB) {
             const int wc = (n - kb < NB) ? n - kb : NB;
             if (sb == NB) {
-                DNH_TRY(launch_subpanel(NB, G, kb, wc, NB));
+                DNH_TRY(launch_subpanel(NB, G, kb, wc, NB, kb, wc));
             } else if (sb > 0) {
                 for (int cs = kb; cs < kb + wc; cs += sb) {
                     const int sw = (kb + wc - cs < sb) ? kb + wc - cs : sb;
-                    DNH_TRY(launch_subpanel(sb, Gs, cs, sw, sb));
-                    if (wc > sw) {
-                        // the sub-panel's steps applied to the panel's other columns
-                        hipLaunchKernelGGL((invert_swap_kernel<T>), dim3(1, (unsigned)batch), dim3(kSwapThreads), 0, stream, W, Tb, ipiv, n, ld,
-                                           cs, sw, kb, kb + wc, bs_w, bs_t);
-                        DNH_TRY(gemm_accumulate(t->dtype, W + kb, Gs, Tb + kb, n, wc, sw, sb, ld, ld, batch, bs_g, bs_t, bs_w, stream));
-                    }
+                    DNH_TRY(launch_subpanel(sb, Gs, cs, sw, sb, kb, wc));   // also exchanges the panel's other columns and fills T
+                    if (wc > sw)                                             // the sub-panel's steps applied to those columns
+                        hipLaunchKernelGGL((invert_panel_update_kernel<T>), dim3((unsigned)cdiv(n, 256 / NB), (unsigned)batch), dim3(256), 0, stream,
+                                           W, Gs, Tb, n, ld, sb, kb, wc, cs, sw, bs_w, bs_g, bs_t);
                 }
                 hipLaunchKernelGGL((invert_extract_g_kernel<T>), dim3((unsigned)cdiv((int64_t)n * wc, 256), (unsigned)batch), dim3(256), 0, stream,
                                    W, G, n, ld, kb, wc, bs_w, bs_g);
