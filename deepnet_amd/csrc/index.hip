@@ -397,6 +397,61 @@ __global__ __launch_bounds__(kBlock) void compact_move_fast_kernel(const uint8_t
     }
 }
 
+// TrueIndices of a mask whose elements lie in row-major order in memory: the block counts of compact_count_fast_kernel<16>, then
+// every thread ranks the selected elements of its four 16-byte mask vectors and notes their positions inside the block's region
+// (16 Ki elements, so 16 bits each) in LDS at their rank; the block then writes the coordinates rank by rank, so a wavefront's
+// store instruction covers 64 consecutive rows of the target (per-thread runs straight from registers measured 1.6x slower than
+// the general kernel: every store instruction touched 64 different cache lines).
+template <bool PREFIXED, bool PAIR>
+__global__ __launch_bounds__(kBlock) void true_indices_fast_kernel(const uint8_t* mask, int64_t* out, Lay shp, uint32_t nvec, uint32_t nout,
+                                                                   const uint32_t* block_base) {
+    constexpr int VEC = 16;
+    __shared__ uint16_t stage[kFastJ * kBlock * VEC];
+    uint32_t flags[kFastJ];
+    uint64_t packed = 0;
+#pragma unroll
+    for (int j = 0; j < kFastJ; j++) {
+        const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+        flags[j] = v < nvec ? mask_flags<VEC>(mask + (size_t)v * VEC) : 0u;
+        packed |= (uint64_t)__popc(flags[j]) << (16 * j);
+    }
+    uint64_t total;
+    const uint64_t pre = block_exclusive_scan64(packed, &total);
+    const uint32_t seg_base = PREFIXED ? block_base[blockIdx.x] : block_sum_before(block_base, blockIdx.x);
+    uint32_t lbase = 0;
+#pragma unroll
+    for (int j = 0; j < kFastJ; j++) {
+        uint32_t k = lbase + (uint32_t)((pre >> (16 * j)) & 0xFFFF);
+        lbase += (uint32_t)((total >> (16 * j)) & 0xFFFF);
+        uint32_t f = flags[j];
+        while (f) {
+            const int e = __ffs((int)f) - 1;
+            f &= f - 1;
+            stage[k++] = (uint16_t)((j * kBlock + threadIdx.x) * VEC + e);
+        }
+    }
+    __syncthreads();
+    const uint32_t region = blockIdx.x * (uint32_t)(kFastJ * kBlock * VEC);
+    for (uint32_t r = threadIdx.x; r < lbase; r += kBlock) {
+        const uint32_t k = seg_base + r;
+        if (k >= nout) break;
+        uint32_t i = region + stage[r];
+        if constexpr (PAIR) {   // two coordinates: one 16-byte store
+            const uint32_t q = i / shp.shape[1];
+            Pack<int64_t, 2> pr;
+            pr.v[0] = (int64_t)q;
+            pr.v[1] = (int64_t)(i - q * shp.shape[1]);
+            store_pack<int64_t, 2>(out + (size_t)k * 2, pr);
+        } else {
+            for (int d = shp.nd - 1; d >= 0; d--) {
+                const uint32_t q = (d == 0) ? 0u : i / shp.shape[d];
+                out[(size_t)k * shp.nd + d] = (int64_t)(i - q * shp.shape[d]);
+                i = q;
+            }
+        }
+    }
+}
+
 template <class W, bool SET>
 int32_t run_compaction_fast(const uint8_t* mask, void* full, void* out, int64_t n, int64_t nout64, hipStream_t stream) {
     constexpr int VEC = 16 / (int)sizeof(W);
@@ -561,5 +616,40 @@ extern "C" int32_t dnh_true_indices(const DnhTensor* t, const DnhTensor* src, vo
         // a 0-d source has one element and no coordinates: nothing to write
         return DNH_OK;
     }
-    return run_compaction<kTrueIndices>(m, nullptr, elem_ptr(t), lay_of(t), 8, nelems(src), t->shape[0], (hipStream_t)stream);
+    const int64_t n = nelems(src), nout = t->shape[0];
+    // fast path: the mask's elements lie in row-major order (extent-1 dimensions aside), whole 16-byte vectors, a dense target
+    bool dense = n > 0 && nout > 0 && n <= (int64_t)kMaxItems && (n % 16) == 0 && aligned_to(elem_ptr(src), 16) &&
+                 t->stride[1] == 1 && t->stride[0] == t->shape[1];
+    int64_t expect = 1;
+    for (int d = src->ndims - 1; d >= 0 && dense; d--) {
+        if (src->shape[d] != 1 && src->stride[d] != expect) dense = false;
+        expect *= src->shape[d];
+    }
+    if (dense) {
+        hipStream_t s = (hipStream_t)stream;
+        const uint8_t* mask = (const uint8_t*)elem_ptr(src);
+        int64_t* out = (int64_t*)elem_ptr(t);
+        const uint32_t nvec = (uint32_t)(n / 16);
+        const uint32_t no = (uint32_t)(nout > (int64_t)kMaxItems ? kMaxItems : nout);
+        const uint32_t nb = cdiv(nvec, kFastJ * kBlock);
+        const bool pair = src->ndims == 2 && aligned_to(out, 16);
+        uint32_t* counts;
+        WorkspaceLease lease;
+        DNH_TRY(workspace(s, sizeof(uint32_t) * (size_t)nb, (void**)&counts, lease));
+        hipLaunchKernelGGL(compact_count_fast_kernel<16>, dim3(nb), dim3(kBlock), 0, s, mask, nvec, counts);
+        DNH_LAUNCH_CHECK();
+        const Lay shp = lay_of(src);
+        if (nb <= 8192) {
+            if (pair) hipLaunchKernelGGL((true_indices_fast_kernel<false, true>), dim3(nb), dim3(kBlock), 0, s, mask, out, shp, nvec, no, counts);
+            else hipLaunchKernelGGL((true_indices_fast_kernel<false, false>), dim3(nb), dim3(kBlock), 0, s, mask, out, shp, nvec, no, counts);
+        } else {
+            hipLaunchKernelGGL(compact_scan_kernel, dim3(1), dim3(kBlock), 0, s, counts, nb);
+            DNH_LAUNCH_CHECK();
+            if (pair) hipLaunchKernelGGL((true_indices_fast_kernel<true, true>), dim3(nb), dim3(kBlock), 0, s, mask, out, shp, nvec, no, counts);
+            else hipLaunchKernelGGL((true_indices_fast_kernel<true, false>), dim3(nb), dim3(kBlock), 0, s, mask, out, shp, nvec, no, counts);
+        }
+        DNH_LAUNCH_CHECK();
+        return DNH_OK;
+    }
+    return run_compaction<kTrueIndices>(m, nullptr, elem_ptr(t), lay_of(t), 8, n, nout, (hipStream_t)stream);
 }

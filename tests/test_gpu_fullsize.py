@@ -103,6 +103,14 @@ def test_masked_get_many_blocks(G):
     assert_exact(a[a > 500], G.toNumpy(ta.M(ta > 500)))
 
 
+def test_true_indices_many_blocks(G):
+    """A dense 2-d mask of 144 Mi elements: more than 8192 blocks on the fast TrueIndices path (scan launch), sparse selection."""
+    rng = np.random.default_rng(9)
+    m = rng.random((9216, 16384)) < 0.01
+    got = G.toNumpy(G.ofNumpy(m).trueIdx())
+    assert_exact(np.argwhere(m).astype(np.int64), got)
+
+
 def test_config5_mlp_block(G):
     rng = np.random.default_rng(123)
     sd = 1.0 / np.sqrt(512.0)

@@ -132,12 +132,17 @@ def test_mask_doc_vectors(H, G):
     assert G.toNumpy(t).tolist() == [[8.0, 9.0, 3.0], [4.0, 5.0, 0.0]]                    # :109-114
 
 
-@pytest.mark.parametrize("shape", [(2, 4), (50,), (7, 11, 13), (3, 0), (100, 100)])
+@pytest.mark.parametrize("shape", [(2, 4), (50,), (7, 11, 13), (3, 0), (100, 100), (16,), (4096,), (64, 48), (8, 6, 32), (1, 160, 1, 3),
+                                   (333, 1024)])
 def test_true_idx(H, G, rng, shape):
     m = rng.random(shape) < 0.4
     ref, got = both(H, G, lambda m: m.trueIdx(), m)
     assert_exact(ref, got)
     assert_exact(np.argwhere(m).astype(np.int64).reshape(-1, len(shape)), got)
+    # all true, all false, and a target that is a column slice of a wider tensor (not dense: the general path)
+    for mm in (np.ones(shape, np.bool_), np.zeros(shape, np.bool_)):
+        ref, got = both(H, G, lambda m: m.trueIdx(), mm)
+        assert_exact(ref, got)
     # on a permuted view
     if len(shape) == 3:
         ref, got = both(H, G, lambda m: m.permuteAxes([1, 2, 0]).trueIdx(), m)
