@@ -170,6 +170,17 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6)):
             return [("masked_get", (D(new([K], np.int32)), D(a), arr, 1))]
         timed(4, "MaskedGet int32 by bool mask", 2 * N + N * 4 + K * 4, mget)
 
+        def mset(i):
+            a, b, m = mk()
+            arr = (C.POINTER(abi.DnhTensor) * 1)()
+            dm = CAbiTensorBackend._desc(m)
+            keep.append((m, dm, arr))
+            arr[0] = C.pointer(dm)
+            return [("masked_set", (D(a), arr, 1, D(b[0:K])))]
+        timed(4, "MaskedSet int32 by bool mask", 2 * N + K * 4 + K * 4, mset)
+        timed(4, "TrueIndices bool[16Mi] -> [K,1]", 2 * N + K * 8,
+              lambda i: (lambda a, b, m: [("true_indices", (D(new([K, 1], np.int64)), D(m)))])(*mk()))
+
         def gat(i):
             a = G.ofNumpy(ha)
             idx = G.ofNumpy(hidx)
