@@ -219,7 +219,16 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 && FAST ? 4 : 2)) void gemm
 #pragma unroll
             for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+                for (int r = 0; r < 16; r++) {
+                    // accumulate mode starts from the target's values, fetched while the first tiles arrive: the epilogue is then a
+                    // plain store instead of 64 read-modify-write round trips per lane
+                    acc[i][j][r] = 0.f;
+                    if constexpr (ACC) {
+                        const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + (lane >> 5) * 4 + (r & 3);
+                        const int64_t n = n0 + wn + j * 32 + (lane & 31);
+                        if (full_mn || (m < g.M && n < g.N)) acc[i][j][r] = c[m * g.scm + n * g.scn];
+                    }
+                }
 
         int vl = kDirect;
         if (FAST || K > 0) {  // (the fast kernel is only launched with K > 0) an empty inner dimension has no element to fetch (not even the clamped one): the target becomes zeros
@@ -268,7 +277,7 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 && FAST ? 4 : 2)) void gemm
                     const int64_t n = n0 + wn + j * 32 + lm;
                     if (full_mn || (m < g.M && n < g.N)) {
                         T* dst = c + m * g.scm + n * g.scn;
-                        *dst = ACC ? *dst + acc[i][j][r] : acc[i][j][r];
+                        *dst = acc[i][j][r];
                     }
                 }
     } else {
@@ -280,7 +289,13 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 && FAST ? 4 : 2)) void gemm
 #pragma unroll
             for (int j = 0; j < 4; j++)
 #pragma unroll
-                for (int r = 0; r < 4; r++) acc[i][j][r] = 0.0;
+                for (int r = 0; r < 4; r++) {
+                    acc[i][j][r] = 0.0;
+                    if constexpr (ACC) {   // as for single precision: start from the target's values
+                        const int64_t m = m0 + wm + i * 16 + 4 * r + (lane >> 4), n = n0 + wn + j * 16 + (lane & 15);
+                        if (full_mn || (m < g.M && n < g.N)) acc[i][j][r] = c[m * g.scm + n * g.scn];
+                    }
+                }
         int vl = kDirect;
         if (FAST || K > 0) {  // (the fast kernel is only launched with K > 0) an empty inner dimension has no element to fetch (not even the clamped one): the target becomes zeros
             vl = load_tiles(0, 0);
@@ -319,7 +334,7 @@ __global__ __launch_bounds__(kBlock, (sizeof(T) == 4 && FAST ? 4 : 2)) void gemm
                     const int64_t m = m0 + wm + i * 16 + 4 * r + lk, n = n0 + wn + j * 16 + lm;
                     if (full_mn || (m < g.M && n < g.N)) {
                         T* dst = c + m * g.scm + n * g.scn;
-                        *dst = ACC ? *dst + acc[i][j][r] : acc[i][j][r];
+                        *dst = acc[i][j][r];
                     }
                 }
     }
