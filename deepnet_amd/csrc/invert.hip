@@ -186,6 +186,7 @@ __global__ __launch_bounds__(kMaxPanelThreads) void invert_subpanel_lds_kernel(T
     __shared__ T red_v[2][kMaxPanelThreads / 64];
     __shared__ int red_i[2][kMaxPanelThreads / 64];
     __shared__ int piv_s[NB];   // pivots go to memory once, at the end: a barrier waits for the stores issued before it
+    __shared__ T prow[2][NB];
     {
         // sixteen loads in flight per thread: a single workgroup fetches the whole sub-panel, so the fetch is latency-bound
         constexpr int UL = 16;
@@ -219,14 +220,18 @@ __global__ __launch_bounds__(kMaxPanelThreads) void invert_subpanel_lds_kernel(T
             if (tid == 0) *singular = 1;
         }
         if (tid == 0) piv_s[j] = p;
-        if (p != col && tid < CW) {
-            const T t = L[col * CW + tid];
-            L[col * CW + tid] = L[p * CW + tid];
-            L[p * CW + tid] = t;
+        if (tid < CW) {
+            // exchange rows col and p; the pivot row also goes to a side buffer (one per step parity), so that nobody reads it
+            // from L while its owners rewrite it below and the step needs no barrier between the two
+            const T a = L[p * CW + tid];
+            if (p != col) {
+                L[p * CW + tid] = L[col * CW + tid];
+                L[col * CW + tid] = a;
+            }
+            prow[j & 1][tid] = a;
         }
         __syncthreads();
-        const T sj = (c == j ? T(1) : L[col * CW + c]) / L[col * CW + j];   // my column's entry of the scaled pivot row
-        __syncthreads();                                                    // everyone has read the pivot row before it changes
+        const T sj = (c == j ? T(1) : prow[j & 1][c]) / prow[j & 1][j];   // my column's entry of the scaled pivot row
         const bool is_pivot_col = c == j;
         // The update is bound by the instruction issue rate of the one CU that runs it, so the loop body is kept minimal: every
         // row is treated alike (the pivot row is rewritten by its owners afterwards, the next column's pivot search is a separate
