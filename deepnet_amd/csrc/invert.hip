@@ -14,6 +14,7 @@
 // A pivot that is exactly zero marks the matrix singular (LAPACK's info > 0), reported as DNH_ERR_SINGULAR_MATRIX.
 // Floating point only; the work is 2 n^3 flops per matrix, nearly all of it in step 3.
 #include "common.h"
+#include "wave_argmax.h"
 
 namespace dnh {
 int32_t gemm_accumulate(int32_t dtype, void* c, const void* a, const void* b, int64_t M, int64_t N, int64_t K, int64_t lda,
@@ -34,21 +35,12 @@ __device__ inline T abs_of(T x) { return x < T(0) ? -x : x; }
 template <class T>
 __device__ inline void block_arg_max(T& best, int& bi, T* red_v, int* red_i) {
     const int tid = threadIdx.x, nwaves = blockDim.x >> 6;
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        const T ov = __shfl_xor(best, off, 64);
-        const int oi = __shfl_xor(bi, off, 64);
-        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
-    }
-    if ((tid & 63) == 0) { red_v[tid >> 6] = best; red_i[tid >> 6] = bi; }
+    wave_arg_max_to_lane63(best, bi);
+    if ((tid & 63) == 63) { red_v[tid >> 6] = best; red_i[tid >> 6] = bi; }
     __syncthreads();
-    best = red_v[0];
-    bi = red_i[0];
-    for (int k = 1; k < nwaves; k++) {
-        const T ov = red_v[k];
-        const int oi = red_i[k];
-        if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
-    }
+    // the wavefronts' candidates (at most 16) are combined by every wavefront for itself: one LDS read per lane and four lane
+    // shifts (a loop over the entries cost 0.9 us of a 5 us elimination step, rolled or unrolled)
+    arg_max_of_entries(red_v, red_i, nwaves, tid & 63, best, bi);
 }
 
 // Thread layout of the panel kernel: lane l of a wavefront works on panel column l % 32 of row l / 32 + 2 * (wavefront, pass),
