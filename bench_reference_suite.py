@@ -101,9 +101,9 @@ class Worker:
     def MaskedGet(self): self.a.M(self.p)
     def MaskedSet(self): self.maskedSetTarget.setM([self.p], self.maskedSetElems)
     def Invert(self): self.T.invert(self.a)
-    def PseudoInvert(self): raise NotImplementedError("PseudoInvert needs SVD, which no device backend provides")
-    def SVD(self): raise NotImplementedError("SVD is not supported by the device backends (CudaBackend.fs:486-488)")
-    def SymEigDec(self): raise NotImplementedError("SymmetricEigenDecomposition is not supported by the device backends")
+    def PseudoInvert(self): self.T.pseudoInvert(self.a)
+    def SVD(self): self.T.SVD(self.a)
+    def SymEigDec(self): self.T.symmetricEigenDecomposition("Upper", self.a)
     def Not(self): self._ensure_bool(); ~self.p
     def And(self): self._ensure_bool(); self.p & self.q
     def Or(self): self._ensure_bool(); self.p | self.q

@@ -19,6 +19,7 @@ DNH_ERR_HIP = 4
 DNH_ERR_INDEX_OUT_OF_RANGE = 5
 DNH_ERR_NOT_INITIALIZED = 6
 DNH_ERR_SINGULAR_MATRIX = 7
+DNH_ERR_NO_CONVERGENCE = 8
 
 # DnhDType
 DNH_BOOL, DNH_U8, DNH_I8, DNH_I32, DNH_U32, DNH_I64, DNH_U64, DNH_F32, DNH_F64 = range(9)
@@ -136,6 +137,12 @@ OP_SIGNATURES = {
     "batched_invert": [_T, _T],
 }
 
+# entry points the CPU oracle does not restate in C (it uses numpy's LAPACK, which is what the reference's host backend calls)
+LAPACK_OP_SIGNATURES = {
+    "batched_svd": [_T, _T, _T, _T],          # s, u (or NULL), v (or NULL), src
+    "symmetric_eig": [C.c_int32, _T, _T, _T],  # part (0 upper, 1 lower), eigvals, eigvecs, src
+}
+
 # every symbol include/tensor_hip.h declares
 EXPORTED_SYMBOLS = [
     "dnh_init", "dnh_device_info", "dnh_last_error", "dnh_async_error",
@@ -144,4 +151,4 @@ EXPORTED_SYMBOLS = [
     "dnh_memcpy_h2d", "dnh_memcpy_d2h", "dnh_memcpy_d2d",
     "dnh_stream_create", "dnh_stream_destroy", "dnh_stream_sync", "dnh_device_sync",
     "dnh_event_create", "dnh_event_destroy", "dnh_event_record", "dnh_event_sync", "dnh_event_elapsed_ms",
-] + ["dnh_" + k for k in OP_SIGNATURES]
+] + ["dnh_" + k for k in OP_SIGNATURES] + ["dnh_" + k for k in LAPACK_OP_SIGNATURES]

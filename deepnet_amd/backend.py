@@ -16,6 +16,9 @@ from . import abi
 from .layout import TensorLayout
 
 
+MatrixPart = ("Upper", "Lower")   # Tensor/Tensor/TensorBackend.fs: which triangle a symmetric operation reads
+
+
 class SingularMatrixException(ArithmeticError):
     """Raised when a matrix that is not invertible is inverted (Tensor/Tensor/Tensor.fs:2831-2834)."""
 
@@ -214,10 +217,12 @@ class CAbiTensorBackend:
 
     # the reference's CUDA backend also leaves SVD/eigen unsupported (CudaBackend.fs:486-492)
     def BatchedSVD(self, trgtS, trgtUV, src1):
-        raise NotImplementedError("BatchedSVD is not supported by this backend")
+        u, v = (None, None) if trgtUV is None else (C.byref(self._desc(trgtUV[0])), C.byref(self._desc(trgtUV[1])))
+        self._call("batched_svd", C.byref(self._desc(trgtS)), u, v, C.byref(self._desc(src1)))
 
     def BatchedInvert(self, trgt, src1):
         self._call("batched_invert", C.byref(self._desc(trgt)), C.byref(self._desc(src1)))
 
     def SymmetricEigenDecomposition(self, part, trgtEigVals, trgtEigVecs, src):
-        raise NotImplementedError("SymmetricEigenDecomposition is not supported by this backend")
+        self._call("symmetric_eig", MatrixPart.index(part), C.byref(self._desc(trgtEigVals)), C.byref(self._desc(trgtEigVecs)),
+                   C.byref(self._desc(src)))

@@ -625,6 +625,86 @@ class Tensor:
         trgt.FillInvert(a)
         return trgt
 
+    # ---- SVD, pseudo-inverse, symmetric eigendecomposition (Tensor.fs:2841-2977) -------------------------------------------------------
+    @staticmethod
+    def SVDSizes(a: "Tensor"):
+        if a.NDims < 2:
+            raise ValueError(f"Need at least a matrix to SVD but got shape {a.Shape}.")
+        batchShp = list(a.Shape[:a.NDims - 2])
+        M, N = a.Shape[a.NDims - 2], a.Shape[a.NDims - 1]
+        return batchShp, M, N, min(M, N)
+
+    def FillSVD(self, a: "Tensor", trgtUV=None):
+        """Fills this tensor with the (batched) singular values of `a`; trgtUV = (U, V) also receives the transformation matrices."""
+        batchShp, M, N, K = Tensor.SVDSizes(a)
+        _same_storage([self, a])
+        if list(self.Shape) != batchShp + [K]:
+            raise ValueError(f"Need a tensor of shape {batchShp + [K]} for SVD singular values but got shape {self.Shape}.")
+        if trgtUV is not None:
+            trgtU, trgtV = trgtUV
+            _same_storage([self, a, trgtU, trgtV])
+            if list(trgtU.Shape) != batchShp + [M, M]:
+                raise ValueError(f"Need a tensor of shape {batchShp + [M, M]} for SVD left unitary matrices but got shape {trgtU.Shape}.")
+            if list(trgtV.Shape) != batchShp + [N, N]:
+                raise ValueError(f"Need a tensor of shape {batchShp + [N, N]} for SVD right unitary matrices but got shape {trgtV.Shape}.")
+        self.Backend.BatchedSVD(self, trgtUV, a)
+
+    @staticmethod
+    def SVD(a: "Tensor"):
+        """(U, S, V) with a = U .* diagMat(S) .* V.T, batched over the leading dimensions."""
+        batchShp, M, N, K = Tensor.SVDSizes(a)
+        U = Tensor.new(batchShp + [M, M], a.Dev, a.DataType, order=ColumnMajor)
+        S = Tensor.new(batchShp + [K], a.Dev, a.DataType, order=ColumnMajor)
+        V = Tensor.new(batchShp + [N, N], a.Dev, a.DataType, order=RowMajor)
+        S.FillSVD(a, trgtUV=(U, V))
+        return U, S, V
+
+    @staticmethod
+    def SVDWithoutUV(a: "Tensor") -> "Tensor":
+        batchShp, M, N, K = Tensor.SVDSizes(a)
+        S = Tensor.new(batchShp + [K], a.Dev, a.DataType, order=ColumnMajor)
+        S.FillSVD(a)
+        return S
+
+    def FillPseudoInvert(self, a: "Tensor", rCond=1e-15):
+        """Moore-Penrose pseudo-inverse through the SVD; singular values below rCond count as zero (Tensor.fs:2911-2924)."""
+        _same_storage([self, a])
+        if a.NDims < 2:
+            raise ValueError(f"Need at least a matrix to pseudo invert but got shape {a.Shape}.")
+        a = a.broadcastTo(self.Shape)
+        u, s, v = Tensor.SVD(a)
+        dt = np.dtype(a.DataType).type
+        rc, zero, one = s.scalarLike(dt(rCond)), s.scalarLike(dt(0)), s.scalarLike(dt(1))
+        sinv = Tensor.ifThenElse(s >= rc, one / s, zero)
+        self.FillDot(v, sinv.padRight() * u.T)
+
+    @staticmethod
+    def pseudoInvert(a: "Tensor", rCond=1e-15) -> "Tensor":
+        trgt = Tensor.new(a.Shape, a.Dev, a.DataType)
+        trgt.FillPseudoInvert(a, rCond)
+        return trgt
+
+    @staticmethod
+    def FillSymmetricEigenDecomposition(part, trgtEigVals: "Tensor", trgtEigVecs: "Tensor", a: "Tensor"):
+        _same_storage([trgtEigVals, trgtEigVecs, a])
+        if a.NDims != 2 or a.Shape[0] != a.Shape[1]:
+            raise ValueError(f"Require a square matrix for symmetric eigen-decomposition but got {a.Shape}.")
+        if list(trgtEigVecs.Shape) != list(a.Shape):
+            raise ValueError(f"trgtEigVecs and src must have the same shapes but got {trgtEigVecs.Shape} and {a.Shape}.")
+        if trgtEigVals.NDims != 1 or trgtEigVals.Shape[0] != a.Shape[0]:
+            raise ValueError(f"trgtEigVals must be a vector of length {a.Shape[0]} but it has shape {trgtEigVals.Shape}.")
+        trgtEigVals.Backend.SymmetricEigenDecomposition(part, trgtEigVals, trgtEigVecs, a)
+
+    @staticmethod
+    def symmetricEigenDecomposition(part, a: "Tensor"):
+        """(vals, vecs): ascending eigenvalues, column k of vecs the eigenvector of vals[k]; only the `part` triangle is read."""
+        if a.NDims != 2:
+            raise ValueError("require a square matrix for symmetric eigen-decomposition")
+        trgtEigVals = Tensor.new([a.Shape[0]], a.Dev, a.DataType)
+        trgtEigVecs = Tensor.new(a.Shape, a.Dev, a.DataType, order=ColumnMajor)
+        Tensor.FillSymmetricEigenDecomposition(part, trgtEigVals, trgtEigVecs, a)
+        return trgtEigVals, trgtEigVecs
+
     def __matmul__(self, b: "Tensor") -> "Tensor":
         a = self
         _same_storage([a, b])

@@ -41,7 +41,8 @@ typedef enum DnhStatus {
     DNH_ERR_HIP = 4,              /* -> CudaException analogue                                  */
     DNH_ERR_INDEX_OUT_OF_RANGE = 5, /* -> IndexOutOfRangeException (Host/FastAccess.fs:51-61)   */
     DNH_ERR_NOT_INITIALIZED = 6,
-    DNH_ERR_SINGULAR_MATRIX = 7   /* -> SingularMatrixException (Tensor.fs:2831-2834)               */
+    DNH_ERR_SINGULAR_MATRIX = 7,  /* -> SingularMatrixException (Tensor.fs:2831-2834)               */
+    DNH_ERR_NO_CONVERGENCE = 8    /* -> "SVD did not converge" (Host/HostBackend.fs:598)             */
 } DnhStatus;
 
 /* Element types: the set the reference marshals to kernels (Cuda/NativeTensor.fs:22-34). bool is one byte 0/1. */
@@ -243,6 +244,19 @@ int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void
  * t's shape by the frontend, Tensor.fs:2811-2815), single or double; any strides; t may be src.  Partial pivoting; a pivot
  * that is exactly zero gives DNH_ERR_SINGULAR_MATRIX (LAPACK info > 0).  Synchronises the stream to read that flag. */
 int32_t dnh_batched_invert(const DnhTensor* t, const DnhTensor* src, void* stream);
+
+/* ITensorBackend.BatchedSVD (TensorBackend.fs:143; Host/HostBackend.fs:579-606 LAPACK gesdd with job 'A' or 'N'; not implemented
+ * by the reference's CUDA backend, Cuda/CudaBackend.fs:486-488).  src [b_1..b_k; M; N], single or double, any strides.
+ * s [b..; min(M, N)] receives the singular values in descending order.  u [b..; M; M] and v [b..; N; N] are both given (then
+ * src = u diag(s) v^T with u, v orthogonal) or both NULL (singular values only).  One-sided Jacobi rotations; synchronises
+ * the stream once per sweep; DNH_ERR_NO_CONVERGENCE if a matrix is not diagonal after 60 sweeps. */
+int32_t dnh_batched_svd(const DnhTensor* s, const DnhTensor* u, const DnhTensor* v, const DnhTensor* src, void* stream);
+
+/* ITensorBackend.SymmetricEigenDecomposition (TensorBackend.fs:145; Host/HostBackend.fs:608-628 LAPACK syevd 'V'; not implemented
+ * by the reference's CUDA backend, Cuda/CudaBackend.fs:490-492).  src [n; n]; only the triangle named by part (0 = upper,
+ * 1 = lower, MatrixPart in Tensor/Tensor/TensorBackend.fs) is read.  eigvals [n] receives the eigenvalues in ascending order,
+ * column k of eigvecs [n; n] the unit eigenvector of eigenvalue k.  eigvecs may be src. */
+int32_t dnh_symmetric_eig(int32_t part, const DnhTensor* eigvals, const DnhTensor* eigvecs, const DnhTensor* src, void* stream);
 
 #ifdef __cplusplus
 }

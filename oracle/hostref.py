@@ -80,6 +80,29 @@ class TensorHostRefBackend(CAbiTensorBackend):
     def Transfer(self, trgt, src) -> bool:
         return False  # HostBackend.fs:210-211: the device backends implement transfers
 
+    # The reference's host backend hands these two to LAPACK (HostBackend.fs:579-628: gesdd with job 'A' / 'N', syevd with job 'V');
+    # numpy.linalg.svd and numpy.linalg.eigh call the same routines, so they are the restatement.  Bit-level parity with MKL is
+    # unpinned (library build and threading), and vectors are only defined up to sign: the tests compare through properties.
+    def BatchedSVD(self, trgtS, trgtUV, src1):
+        a = toNumpy(src1)
+        if a.dtype.kind != "f":
+            raise NotImplementedError("this operation is only supported for floating point numbers")
+        if trgtUV is None:
+            _assign(trgtS, np.linalg.svd(a, compute_uv=False))
+        else:
+            u, s, vt = np.linalg.svd(a, full_matrices=True)
+            _assign(trgtS, s)
+            _assign(trgtUV[0], u)
+            _assign(trgtUV[1], np.swapaxes(vt, -1, -2))
+
+    def SymmetricEigenDecomposition(self, part, trgtEigVals, trgtEigVecs, src):
+        a = toNumpy(src)
+        if a.dtype.kind != "f":
+            raise NotImplementedError("this operation is only supported for floating point numbers")
+        w, v = np.linalg.eigh(a, UPLO="U" if part == "Upper" else "L")
+        _assign(trgtEigVals, w)
+        _assign(trgtEigVecs, v)
+
 
 class TensorHostRefDevice(ITensorDevice):
     Id = "HostRef"
@@ -112,6 +135,15 @@ def toNumpy(t: Tensor) -> np.ndarray:
         view = np.lib.stride_tricks.as_strided(t.Storage.HostArray[lay.Offset:], shape=lay.Shape, strides=[s * isz for s in lay.Stride])
         out[...] = view
     return out
+
+
+def _assign(t: Tensor, values: np.ndarray):
+    """Writes `values` into the (possibly strided) host tensor t."""
+    lay = t.Layout
+    if lay.NElems:
+        isz = t.DataType.itemsize
+        view = np.lib.stride_tricks.as_strided(t.Storage.HostArray[lay.Offset:], shape=lay.Shape, strides=[s * isz for s in lay.Stride])
+        view[...] = np.asarray(values, dtype=t.DataType).reshape(lay.Shape)
 
 
 def transfer(t: Tensor) -> Tensor:
