@@ -13,6 +13,7 @@
 #pragma once
 
 #include <cstdint>
+#include <algorithm>
 #include <cstring>
 #include <memory>
 #include <new>
@@ -31,6 +32,7 @@ using Shape = std::vector<int64_t>;
 struct NotSupportedException : std::runtime_error { using std::runtime_error::runtime_error; };
 struct HipException : std::runtime_error { using std::runtime_error::runtime_error; };
 struct SingularMatrixException : std::runtime_error { using std::runtime_error::runtime_error; };   // Tensor.fs:2831-2834
+enum class MatrixPart { Upper, Lower };   // which triangle a symmetric operation reads (TensorBackend.fs)
 
 constexpr int64_t NotFound = DNH_NOT_FOUND;                         // SpecialIdx.NotFound, TensorRng.fs:24
 constexpr int64_t Remainder = (-9223372036854775807LL - 1LL) + 3;   // SpecialIdx.Remainder, TensorRng.fs:21
@@ -170,6 +172,7 @@ inline void check(int32_t status) {
         case DNH_ERR_OUT_OF_MEMORY: throw std::bad_alloc();
         case DNH_ERR_INDEX_OUT_OF_RANGE: throw std::out_of_range(buf);
         case DNH_ERR_SINGULAR_MATRIX: throw SingularMatrixException(buf);
+        case DNH_ERR_NO_CONVERGENCE: throw std::runtime_error(buf);                  // "SVD did not converge" (HostBackend.fs:598)
         default: throw HipException(buf);
     }
 }
@@ -328,6 +331,16 @@ struct TensorHipBackend {
     static void MatMatDot(const Tensor<T>& t, const Tensor<T>& a, const Tensor<T>& b) { dot(t, a, b); }
     static void BatchedMatMatDot(const Tensor<T>& t, const Tensor<T>& a, const Tensor<T>& b) { dot(t, a, b); }
     static void BatchedInvert(const Tensor<T>& trgt, const Tensor<T>& src) { auto t = desc(trgt); auto s = desc(src); check(dnh_batched_invert(&t, &s, Cfg::Stream())); }
+    // trgtU / trgtV both null: singular values only (the reference's `trgtUV: (U, V) option`)
+    static void BatchedSVD(const Tensor<T>& trgtS, const Tensor<T>* trgtU, const Tensor<T>* trgtV, const Tensor<T>& src) {
+        auto s = desc(trgtS); auto a = desc(src);
+        if (trgtU && trgtV) { auto u = desc(*trgtU); auto v = desc(*trgtV); check(dnh_batched_svd(&s, &u, &v, &a, Cfg::Stream())); }
+        else check(dnh_batched_svd(&s, nullptr, nullptr, &a, Cfg::Stream()));
+    }
+    static void SymmetricEigenDecomposition(MatrixPart part, const Tensor<T>& eigVals, const Tensor<T>& eigVecs, const Tensor<T>& src) {
+        auto w = desc(eigVals); auto v = desc(eigVecs); auto a = desc(src);
+        check(dnh_symmetric_eig(part == MatrixPart::Upper ? 0 : 1, &w, &v, &a, Cfg::Stream()));
+    }
 };
 
 // ---- Tensor<'T> frontend (Tensor.fs), the part that drives the backend path -----------------------------------------------------------
@@ -516,6 +529,34 @@ class Tensor {
         Backend::BatchedInvert(*this, a.broadcastTo(Shape_()));
     }
     static Tensor invert(const Tensor& a) { Tensor t(a.Shape_()); t.FillInvert(a); return t; }
+
+    // SVD and symmetric eigendecomposition (Tensor.fs:2841-2977); U is column-major, V row-major as in the reference
+    struct SVDResult { Tensor U, S, V; };
+    static SVDResult SVD(const Tensor& a) {
+        if (a.NDims() < 2) throw std::invalid_argument("Need at least a matrix to SVD.");
+        Shape batch(a.Shape_().begin(), a.Shape_().end() - 2);
+        const int64_t M = a.Shape_()[a.NDims() - 2], N = a.Shape_()[a.NDims() - 1];
+        Shape su = batch, ss = batch, sv = batch;
+        su.push_back(M); su.push_back(M); ss.push_back(M < N ? M : N); sv.push_back(N); sv.push_back(N);
+        SVDResult r{Tensor(su), Tensor(ss), Tensor(sv)};
+        Backend::BatchedSVD(r.S, &r.U, &r.V, a);
+        return r;
+    }
+    static Tensor SVDWithoutUV(const Tensor& a) {
+        if (a.NDims() < 2) throw std::invalid_argument("Need at least a matrix to SVD.");
+        Shape ss(a.Shape_().begin(), a.Shape_().end() - 2);
+        ss.push_back(std::min(a.Shape_()[a.NDims() - 2], a.Shape_()[a.NDims() - 1]));
+        Tensor s(ss);
+        Backend::BatchedSVD(s, nullptr, nullptr, a);
+        return s;
+    }
+    struct EigResult { Tensor vals, vecs; };
+    static EigResult symmetricEigenDecomposition(MatrixPart part, const Tensor& a) {
+        if (a.NDims() != 2 || a.Shape_()[0] != a.Shape_()[1]) throw std::invalid_argument("Require a square matrix for symmetric eigen-decomposition.");
+        EigResult r{Tensor(Shape{a.Shape_()[0]}), Tensor(a.Shape_())};
+        Backend::SymmetricEigenDecomposition(part, r.vals, r.vecs, a);
+        return r;
+    }
 
     // dot, dispatched by rank as Tensor.(.*) / FillDot (Tensor.fs:2714-2797)
     Tensor dot(const Tensor& b) const {

@@ -229,13 +229,22 @@ and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> Valu
         member this.MatMatDot (t, a, b) = dot t a b
         member this.BatchedMatMatDot (t, a, b) = dot t a b
 
-        // not on the accelerated path; the CUDA backend leaves SVD and the eigen-decomposition unsupported too (CudaBackend.fs:486-492)
+        // LAPACK-type members; the CUDA backend leaves SVD and the eigen-decomposition unsupported (CudaBackend.fs:486-492)
         member this.BatchedInvert (trgt, src) =
             let mutable t, s = desc trgt, desc src
             Native.check (Native.dnh_batched_invert (&t, &s, Cfg.Stream))
-        member this.BatchedSVD (trgtS, trgtUV, src) = raise (NotSupportedException "BatchedSVD is not supported by the HIP backend")
+        member this.BatchedSVD (trgtS, trgtUV, src) =
+            let mutable s, a = desc trgtS, desc src
+            match trgtUV with
+            | Some (trgtU, trgtV) ->
+                let mutable u, v = desc trgtU, desc trgtV
+                Native.check (Native.dnh_batched_svd (&s, &u, &v, &a, Cfg.Stream))
+            | None ->
+                Native.check (Native.dnh_batched_svd_values (&s, IntPtr.Zero, IntPtr.Zero, &a, Cfg.Stream))
         member this.SymmetricEigenDecomposition (part, eigVals, eigVecs, src) =
-            raise (NotSupportedException "SymmetricEigenDecomposition is not supported by the HIP backend")
+            let mutable w, v, a = desc eigVals, desc eigVecs, desc src
+            let part = match part with | MatrixPart.Upper -> 0 | MatrixPart.Lower -> 1
+            Native.check (Native.dnh_symmetric_eig (part, &w, &v, &a, Cfg.Stream))
 
 /// Host <-> device copies: the source is made row-major first, a non-row-major target goes through a device temporary
 /// (CudaBackend.fs:206-270).  Returns false for pairs this backend does not handle so the frontend can try the other side

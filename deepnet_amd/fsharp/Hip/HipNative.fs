@@ -17,6 +17,7 @@ type internal Status =
     | IndexOutOfRange = 5
     | NotInitialized = 6
     | SingularMatrix = 7
+    | NoConvergence = 8
 
 /// DnhDType — the element types the reference marshals to kernels (Cuda/NativeTensor.fs:22-34).
 type internal DType =
@@ -70,6 +71,10 @@ module internal Native =
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_true_indices (DnhTensor& t, DnhTensor& src, nativeint stream)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_dot (DnhTensor& t, DnhTensor& a, DnhTensor& b, nativeint stream)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_batched_invert (DnhTensor& t, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_batched_svd (DnhTensor& s, DnhTensor& u, DnhTensor& v, DnhTensor& src, nativeint stream)
+    // the same entry point with u = v = NULL: singular values only
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl, EntryPoint="dnh_batched_svd")>] extern int dnh_batched_svd_values (DnhTensor& s, nativeint u, nativeint v, DnhTensor& src, nativeint stream)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_symmetric_eig (int part, DnhTensor& eigVals, DnhTensor& eigVecs, DnhTensor& src, nativeint stream)
 
     /// Maps a status to the exception type the reference's backends raise for the same condition.
     let check (status: int) =
@@ -83,4 +88,5 @@ module internal Native =
             | Status.OutOfMemory -> raise (OutOfMemoryException msg)
             | Status.IndexOutOfRange -> raise (IndexOutOfRangeException msg)
             | Status.SingularMatrix -> raise (Tensor.SingularMatrixException msg)
+            | Status.NoConvergence -> failwith msg      // "SVD did not converge" (Host/HostBackend.fs:598)
             | _ -> failwithf "HIP tensor backend error %d: %s" status msg

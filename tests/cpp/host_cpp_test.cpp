@@ -278,6 +278,34 @@ static void doc_examples() {
         expect_throws<tn::SingularMatrixException>("doc.invert.singular", [] { tn::Tensor<double>::invert(tn::Tensor<double>::ofHost({1, 0, 0, 1, 2, 0, 1, 0, 0}, {3, 3})); });
         expect_throws<tn::NotSupportedException>("doc.invert.int", [] { tn::Tensor<int32_t>::invert(tn::Tensor<int32_t>::ofHost({1, 0, 0, 1}, {2, 2})); });
     }
+    // SVD and symmetric eigendecomposition through the C++ frontend: defining properties on small matrices
+    {
+        using TD = tn::Tensor<double>;
+        const std::vector<double> a{4, 0, 3, -5, 1, 2};                      // 3 x 2
+        auto r = TD::SVD(TD::ofHost(a, {3, 2}));
+        auto U = download(r.U), S = download(r.S), V = download(r.V);
+        bool ok = S.size() == 2 && S[0] >= S[1] && S[1] >= 0 && U.size() == 9 && V.size() == 4;
+        for (int i = 0; i < 3 && ok; i++)
+            for (int j = 0; j < 2; j++) {
+                double rec = 0;
+                for (int k = 0; k < 2; k++) rec += U[i * 3 + k] * S[k] * V[j * 2 + k];
+                ok = ok && std::fabs(rec - a[i * 2 + j]) <= 1e-12;
+            }
+        for (int p = 0; p < 3 && ok; p++)
+            for (int q = 0; q < 3; q++) {
+                double d = 0;
+                for (int i = 0; i < 3; i++) d += U[i * 3 + p] * U[i * 3 + q];
+                ok = ok && std::fabs(d - (p == q ? 1.0 : 0.0)) <= 1e-12;
+            }
+        report("parity.svd.3x2", ok);
+        auto s2 = download(TD::SVDWithoutUV(TD::ofHost(a, {3, 2})));
+        report("parity.svd.valuesOnly", s2.size() == 2 && std::fabs(s2[0] - S[0]) <= 1e-12 && std::fabs(s2[1] - S[1]) <= 1e-12);
+        auto e = TD::symmetricEigenDecomposition(tn::MatrixPart::Lower, TD::ofHost({2, 99, 99, -1, 2, 99, 0, -1, 2}, {3, 3}));
+        auto w = download(e.vals);
+        const double r2 = std::sqrt(2.0);
+        report("parity.eig.tridiagonal", w.size() == 3 && std::fabs(w[0] - (2 - r2)) <= 1e-12 && std::fabs(w[1] - 2) <= 1e-12 && std::fabs(w[2] - (2 + r2)) <= 1e-12);
+        expect_throws<tn::NotSupportedException>("doc.svd.int", [] { tn::Tensor<int32_t>::SVD(tn::Tensor<int32_t>::ofHost({1, 0, 0, 1}, {2, 2})); });
+    }
     // counting / convert / reshape of a transposed view copies
     EXPECT("doc.counting", download(TI::counting(5)) == (std::vector<int64_t>{0, 1, 2, 3, 4}));
     EXPECT("doc.convert", download(TF::ofHost({1.7f, -1.7f, 3.0f}, {3}).convert<int32_t>()) == (std::vector<int32_t>{1, -1, 3}));
