@@ -17,6 +17,7 @@
 //     positive semidefinite (equal magnitudes of opposite sign would otherwise share a singular subspace); then the singular
 //     values are lambda + mu and W holds the eigenvectors.  Absolute error of the eigenvalues: a few eps * |A|, as syevd's.
 #include "common.h"
+#include "wave_argmax.h"
 
 #include <algorithm>
 #include <limits>
@@ -40,6 +41,30 @@ __device__ __forceinline__ void pair_of(int ce, int r, int k, int* a, int* b) {
         *a = (r + k) % m;
         *b = (r - k + m) % m;
     }
+}
+
+// Sums of three values over a wavefront, left in lane 63, through DPP lane moves (see wave_argmax.h): row shifts by 1, 2, 4, 8
+// add up each row of 16 lanes into its lane 15 (a lane without a source adds zero), two row broadcasts carry the row sums on.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_fetch_or_zero(double v) {
+    const long long b = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)(unsigned)(b & 0xFFFFFFFFLL), CTRL, ROW_MASK, 0xF, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, ROW_MASK, 0xF, false);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ void sum3_step(double& a, double& b, double& c) {
+    a += dpp_fetch_or_zero<CTRL, ROW_MASK>(a);
+    b += dpp_fetch_or_zero<CTRL, ROW_MASK>(b);
+    c += dpp_fetch_or_zero<CTRL, ROW_MASK>(c);
+}
+__device__ __forceinline__ void wave_sum3_to_lane63(double& a, double& b, double& c) {
+    sum3_step<0x111, 0xF>(a, b, c);   // row_shr:1
+    sum3_step<0x112, 0xF>(a, b, c);   // row_shr:2: lane i now holds the sum of lanes i-3 .. i of its row
+    sum3_step<0x114, 0xF>(a, b, c);   // row_shr:4
+    sum3_step<0x118, 0xF>(a, b, c);   // row_shr:8: lane 15 of a row holds the row's sum
+    sum3_step<0x142, 0xA>(a, b, c);   // row_bcast:15 into rows 1 and 3
+    sum3_step<0x143, 0xC>(a, b, c);   // row_bcast:31 into rows 2 and 3: lane 63 holds the wavefront's sum
 }
 
 __device__ __forceinline__ double block_sum(double v, double* red) {
@@ -75,13 +100,8 @@ __global__ __launch_bounds__(kPairThreads) void jacobi_round_kernel(T* __restric
         sg += u * v;
     }
     // the three sums share one pair of barriers
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        sa += __shfl_xor(sa, off, 64);
-        sb += __shfl_xor(sb, off, 64);
-        sg += __shfl_xor(sg, off, 64);
-    }
-    if ((threadIdx.x & 63) == 0) {
+    wave_sum3_to_lane63(sa, sb, sg);
+    if ((threadIdx.x & 63) == 63) {
         red3[0][threadIdx.x >> 6] = sa;
         red3[1][threadIdx.x >> 6] = sb;
         red3[2][threadIdx.x >> 6] = sg;
@@ -112,7 +132,86 @@ __global__ __launch_bounds__(kPairThreads) void jacobi_round_kernel(T* __restric
             wq[i] = (T)(sn * u + cs * v);
         }
     }
-    if (threadIdx.x == 0) atomicAdd(rotations, 1);
+    if (threadIdx.x == 0) *rotations = 1;   // a flag, not a count: every writer stores the same value, no atomic queue at one address
+}
+
+// The same round for columns of at most NPT * 256 elements: a thread keeps its elements of both column pairs (X and W) in
+// registers, so every global load of the round is issued before the reduction and the rotation only computes and stores (the
+// two-pass form above waits for a second round trip after the barrier; a round is latency-bound, not bandwidth-bound).
+template <class T, int NPT>
+__global__ __launch_bounds__(kPairThreads) void jacobi_round_reg_kernel(T* __restrict__ x, T* __restrict__ w, int rows, int c, int ce, int round,
+                                                                        int wrows, int64_t bsx, int64_t bsw, double tol, int* rotations) {
+    __shared__ double red3[3][kPairThreads / 64];
+    int a, b;
+    pair_of(ce, round, blockIdx.x, &a, &b);
+    if (a >= c || b >= c) return;
+    const int p = a < b ? a : b, q = a < b ? b : a;
+    T* xp = x + (int64_t)blockIdx.y * bsx + (int64_t)p * rows;
+    T* xq = x + (int64_t)blockIdx.y * bsx + (int64_t)q * rows;
+    T* wp = w ? w + (int64_t)blockIdx.y * bsw + (int64_t)p * wrows : nullptr;
+    T* wq = w ? w + (int64_t)blockIdx.y * bsw + (int64_t)q * wrows : nullptr;
+    T u[NPT], v[NPT], wu[NPT], wv[NPT];
+#pragma unroll
+    for (int k = 0; k < NPT; k++) {
+        const int i = threadIdx.x + k * kPairThreads;
+        u[k] = i < rows ? xp[i] : T(0);
+        v[k] = i < rows ? xq[i] : T(0);
+    }
+    if (w) {
+#pragma unroll
+        for (int k = 0; k < NPT; k++) {
+            const int i = threadIdx.x + k * kPairThreads;
+            wu[k] = i < wrows ? wp[i] : T(0);
+            wv[k] = i < wrows ? wq[i] : T(0);
+        }
+    }
+    double sa = 0, sb = 0, sg = 0;
+#pragma unroll
+    for (int k = 0; k < NPT; k++) {
+        const double du = (double)u[k], dv = (double)v[k];
+        sa += du * du;
+        sb += dv * dv;
+        sg += du * dv;
+    }
+    wave_sum3_to_lane63(sa, sb, sg);
+    if ((threadIdx.x & 63) == 63) {
+        red3[0][threadIdx.x >> 6] = sa;
+        red3[1][threadIdx.x >> 6] = sb;
+        red3[2][threadIdx.x >> 6] = sg;
+    }
+    __syncthreads();
+    double alpha = 0, beta = 0, gamma = 0;
+#pragma unroll
+    for (int i = 0; i < kPairThreads / 64; i++) {
+        alpha += red3[0][i];
+        beta += red3[1][i];
+        gamma += red3[2][i];
+    }
+    if (gamma == 0.0 || fabs(gamma) <= tol * sqrt(alpha * beta)) return;
+    const double zeta = (beta - alpha) / (2.0 * gamma);
+    const double t = (zeta >= 0.0 ? 1.0 : -1.0) / (fabs(zeta) + sqrt(1.0 + zeta * zeta));
+    const double cs = 1.0 / sqrt(1.0 + t * t), sn = cs * t;
+#pragma unroll
+    for (int k = 0; k < NPT; k++) {
+        const int i = threadIdx.x + k * kPairThreads;
+        if (i < rows) {
+            const double du = (double)u[k], dv = (double)v[k];
+            xp[i] = (T)(cs * du - sn * dv);
+            xq[i] = (T)(sn * du + cs * dv);
+        }
+    }
+    if (w) {
+#pragma unroll
+        for (int k = 0; k < NPT; k++) {
+            const int i = threadIdx.x + k * kPairThreads;
+            if (i < wrows) {
+                const double du = (double)wu[k], dv = (double)wv[k];
+                wp[i] = (T)(cs * du - sn * dv);
+                wq[i] = (T)(sn * du + cs * dv);
+            }
+        }
+    }
+    if (threadIdx.x == 0) *rotations = 1;   // a flag, not a count: every writer stores the same value, no atomic queue at one address
 }
 
 // identity matrices [batch][n][n]
@@ -253,14 +352,11 @@ __global__ __launch_bounds__(256) void symmetrize_kernel(T* __restrict__ x, cons
     const int lo = i < j ? i : j, hi = i < j ? j : i;
     x[(int64_t)i * n + j] = lower ? a[(int64_t)hi * n + lo] : a[(int64_t)lo * n + hi];
 }
-template <class T>
-__global__ __launch_bounds__(256) void frobenius_kernel(const T* __restrict__ x, double* __restrict__ fro, int64_t total) {
+// fro = sqrt(sum of the squared column norms)
+__global__ __launch_bounds__(256) void frobenius_kernel(const double* __restrict__ norm, double* __restrict__ fro, int c) {
     __shared__ double red[4];
     double s = 0;
-    for (int64_t i = threadIdx.x; i < total; i += 256) {
-        const double v = (double)x[i];
-        s += v * v;
-    }
+    for (int i = threadIdx.x; i < c; i += 256) s += norm[i] * norm[i];
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) s += __shfl_xor(s, off, 64);
     if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
@@ -283,9 +379,17 @@ int32_t jacobi_run(T* x, T* w, int64_t batch, int rows, int c, int wrows, int* c
     const double tol = sqrt((double)rows) * (double)std::numeric_limits<T>::epsilon();   // as LAPACK's Jacobi SVD (xGESVJ)
     for (int sweep = 0; sweep < kMaxSweeps; sweep++) {
         hipLaunchKernelGGL(clear_int_kernel, dim3(1), dim3(1), 0, stream, counter);
-        for (int r = 0; r < ce - 1; r++)
-            hipLaunchKernelGGL((jacobi_round_kernel<T>), dim3((unsigned)(ce / 2), (unsigned)batch), dim3(kPairThreads), 0, stream, x, w, rows, c, ce, r,
-                               wrows, (int64_t)c * rows, (int64_t)c * wrows, tol, counter);
+        const int longest = rows > wrows ? rows : wrows;
+        const dim3 grid((unsigned)(ce / 2), (unsigned)batch);
+#define DNH_ROUND(KERNEL) hipLaunchKernelGGL((KERNEL), grid, dim3(kPairThreads), 0, stream, x, w, rows, c, ce, r, wrows, (int64_t)c * rows, (int64_t)c * wrows, tol, counter)
+        for (int r = 0; r < ce - 1; r++) {
+            if (longest <= 1 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 1>));
+            else if (longest <= 4 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 4>));
+            else if (longest <= 8 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 8>));
+            else if (sizeof(T) == 8 && longest <= 16 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 16>));   // single precision: the two-pass form measured faster at 4000 rows
+            else DNH_ROUND((jacobi_round_kernel<T>));
+        }
+#undef DNH_ROUND
         DNH_LAUNCH_CHECK();
         int rotated = 0;
         DNH_HIP(hipMemcpyAsync(&rotated, counter, sizeof(int), hipMemcpyDeviceToHost, stream));
@@ -462,7 +566,8 @@ int32_t eig_impl(int32_t part, const DnhTensor* vals, const DnhTensor* vecs, con
         DnhTensor ad = dense_like(src, A);
         DNH_TRY(dnh_copy(&ad, src, stream));
         hipLaunchKernelGGL((symmetrize_kernel<T>), dim3(cdiv(n, 256), (unsigned)n), dim3(256), 0, stream, X, A, n, part == 1 ? 1 : 0);
-        hipLaunchKernelGGL((frobenius_kernel<T>), dim3(1), dim3(256), 0, stream, X, mu, (int64_t)n * n);
+        hipLaunchKernelGGL((column_norm_kernel<T>), dim3((unsigned)n, 1), dim3(kPairThreads), 0, stream, X, norm, n, n, (int64_t)n * n);
+        hipLaunchKernelGGL(frobenius_kernel, dim3(1), dim3(256), 0, stream, norm, mu, n);
         hipLaunchKernelGGL((shift_diagonal_kernel<T>), dim3(cdiv(n, 256)), dim3(256), 0, stream, X, mu, n);
         hipLaunchKernelGGL((identity_kernel<T>), dim3(cdiv((int64_t)n * n, 256)), dim3(256), 0, stream, W, n, (int64_t)n * n);
         DNH_LAUNCH_CHECK();
