@@ -12,7 +12,8 @@
 //
 //   SVD of A (M x N):  the side with fewer vectors plays W (it comes out complete); the taller side's vectors are the
 //     normalised columns of X for the singular values above max(M, N) * eps * sigma_max, and an orthonormal basis of their
-//     complement for the rest: the nonzero columns of I - U1 U1^T after the same rotations have made them orthogonal.
+//     complement for the rest: the Householder QR of the columns found so far, Q^T U1 = [D; 0], and Q applied to the unit
+//     vectors that remain.
 //   Symmetric eigendecomposition:  the chosen triangle is mirrored, the matrix shifted by mu = its Frobenius norm so that it is
 //     positive semidefinite (equal magnitudes of opposite sign would otherwise share a singular subspace); then the singular
 //     values are lambda + mu and W holds the eigenvectors.  Absolute error of the eigenvalues: a few eps * |A|, as syevd's.
@@ -311,35 +312,90 @@ __global__ __launch_bounds__(256) void numeric_rank_kernel(const double* __restr
     if (threadIdx.x == 0) rank[blockIdx.x] = red[0] + red[1] + red[2] + red[3];
 }
 
-// z[b] (n x n, column-major = row-major, it is symmetric) = I - U1 U1^T with U1 = the first rank[b] columns of the row-major u[b]
-template <class T>
-__global__ __launch_bounds__(256) void complement_projector_kernel(T* __restrict__ z, const T* __restrict__ u, const int* __restrict__ rank, int n) {
-    const int j = blockIdx.x * 256 + threadIdx.x;
-    const int i = blockIdx.y;
-    const int64_t b = blockIdx.z;
-    if (j >= n) return;
-    const T* ub = u + b * (int64_t)n * n;
-    const int r = rank[b];
-    double s = (i == j) ? 1.0 : 0.0;
-    for (int k = 0; k < r; k++) s -= (double)ub[(int64_t)i * n + k] * (double)ub[(int64_t)j * n + k];
-    z[b * (int64_t)n * n + (int64_t)i * n + j] = (T)s;
-}
+// ---- orthonormal completion of the taller side -----------------------------------------------------------------------------------
+// U1 = the first rank[b] columns of the row-major u[b] (n x n) is orthonormal.  Its Householder QR, Q^T U1 = [D; 0] with D = diag(+-1),
+// gives Q = H_0 H_1 ... H_{r-1} whose columns r .. n-1 span the complement: they are Q applied to the unit vectors e_r .. e_{n-1}.
+// h[b][k][i] keeps column k (contiguous); below its diagonal it ends up holding the Householder vector v_k (v_k[k] = 1 implied).
 
-// The complement basis: the columns of z (after the rotations) with norm > 1/2, normalised, become columns rank[b], rank[b]+1, ...
-// of the row-major u[b].  order lists z's columns by descending norm, so output column rank + k takes z column order[k].
+// h[b][k][i] = u[b][i][k] for k < rank[b]
 template <class T>
-__global__ __launch_bounds__(256) void fill_complement_kernel(T* __restrict__ u, const T* __restrict__ z, const int* __restrict__ order,
-                                                              const double* __restrict__ norm, const int* __restrict__ rank, int n) {
+__global__ __launch_bounds__(256) void gather_u1_kernel(T* __restrict__ h, const T* __restrict__ u, const int* __restrict__ rank, int n, int c) {
     const int i = blockIdx.x * 256 + threadIdx.x;
     const int k = blockIdx.y;
     const int64_t b = blockIdx.z;
-    if (i >= n) return;
-    const int col = rank[b] + k;
-    if (col >= n) return;
-    const int j = order[b * n + k];
-    const double nj = norm[b * n + j];
-    if (!(nj > 0.5)) return;
-    u[(b * n + i) * (int64_t)n + col] = (T)((double)z[b * (int64_t)n * n + (int64_t)j * n + i] / nj);
+    if (i >= n || k >= rank[b]) return;
+    h[(b * c + k) * (int64_t)n + i] = u[(b * n + i) * (int64_t)n + k];
+}
+
+// Householder vector of column k (rows k .. n-1), one workgroup per matrix: tau[b][k], the vector scaled so that v[k] = 1
+template <class T>
+__global__ __launch_bounds__(kPairThreads) void house_vector_kernel(T* __restrict__ h, double* __restrict__ tau, const int* __restrict__ rank, int n,
+                                                                    int c, int k) {
+    __shared__ double red[kPairThreads / 64];
+    const int64_t b = blockIdx.x;
+    if (k >= rank[b]) return;
+    T* col = h + (b * c + k) * (int64_t)n;
+    double s = 0;
+    for (int i = k + 1 + threadIdx.x; i < n; i += kPairThreads) {
+        const double v = (double)col[i];
+        s += v * v;
+    }
+    const double alpha = (double)col[k];   // read by everyone before the barriers of the sum; thread 0 overwrites it at the end
+    const double sigma = block_sum(s, red);
+    if (sigma == 0.0) {   // already a multiple of e_k: H_k = I
+        if (threadIdx.x == 0) tau[b * c + k] = 0.0;
+        return;
+    }
+    const double beta = -copysign(sqrt(alpha * alpha + sigma), alpha);
+    const double scale = 1.0 / (alpha - beta);
+    for (int i = k + 1 + threadIdx.x; i < n; i += kPairThreads) col[i] = (T)((double)col[i] * scale);
+    if (threadIdx.x == 0) {
+        tau[b * c + k] = (beta - alpha) / beta;
+        col[k] = (T)beta;
+    }
+}
+
+// y <- (I - tau v v^T) y for the columns y = first + blockIdx.x of `m` (column stride n, `mc` columns per matrix, `limit[b]` of them
+// in use, counted from the rank when from_rank is set), v = Householder vector k of h
+template <class T>
+__global__ __launch_bounds__(kPairThreads) void house_apply_kernel(T* __restrict__ m, const T* __restrict__ h, const double* __restrict__ tau,
+                                                                   const int* __restrict__ rank, int n, int c, int mc, int k, int first, int from_rank) {
+    __shared__ double red[kPairThreads / 64];
+    const int64_t b = blockIdx.y;
+    const int r = rank[b];
+    const int j = first + blockIdx.x;
+    if (k >= r || j >= (from_rank ? n - r : r)) return;
+    const double t = tau[b * c + k];
+    if (t == 0.0) return;
+    const T* v = h + (b * c + k) * (int64_t)n;
+    T* y = m + (b * mc + j) * (int64_t)n;
+    double s = threadIdx.x == 0 ? (double)y[k] : 0.0;
+    for (int i = k + 1 + threadIdx.x; i < n; i += kPairThreads) s += (double)v[i] * (double)y[i];
+    const double w = t * block_sum(s, red);
+    if (threadIdx.x == 0) y[k] = (T)((double)y[k] - w);
+    for (int i = k + 1 + threadIdx.x; i < n; i += kPairThreads) y[i] = (T)((double)y[i] - w * (double)v[i]);
+}
+
+// e[b][j] = unit vector e_{rank[b] + j} for j < n - rank[b]
+template <class T>
+__global__ __launch_bounds__(256) void complement_seed_kernel(T* __restrict__ e, const int* __restrict__ rank, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const int j = blockIdx.y;
+    const int64_t b = blockIdx.z;
+    const int r = rank[b];
+    if (i >= n || j >= n - r) return;
+    e[(b * n + j) * (int64_t)n + i] = (i == r + j) ? T(1) : T(0);
+}
+
+// u[b][i][rank[b] + j] = e[b][j][i]
+template <class T>
+__global__ __launch_bounds__(256) void complement_store_kernel(T* __restrict__ u, const T* __restrict__ e, const int* __restrict__ rank, int n) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    const int j = blockIdx.y;
+    const int64_t b = blockIdx.z;
+    const int r = rank[b];
+    if (i >= n || j >= n - r) return;
+    u[(b * n + i) * (int64_t)n + r + j] = e[(b * n + j) * (int64_t)n + i];
 }
 
 // symmetric work matrix from one triangle of the row-major a[b] (n x n), plus fro[b] = its Frobenius norm (second kernel adds it
@@ -455,18 +511,23 @@ int32_t svd_impl(const DnhTensor* s, const DnhTensor* u, const DnhTensor* v, con
     const size_t sz_w = want_uv ? align_up(sizeof(T) * (size_t)batch * Cn * Cn) : 0;
     const size_t sz_big = want_uv ? align_up(sizeof(T) * (size_t)batch * R * R) : 0;      // the tall side's vectors, row-major
     const size_t sz_small = want_uv ? align_up(sizeof(T) * (size_t)batch * Cn * Cn) : 0;   // the short side's vectors, row-major
-    const size_t sz_z = want_uv ? sz_big : 0;                                              // projector for the complement
+    const size_t sz_z = want_uv ? sz_big : 0;                                              // the complement's columns
+    const size_t sz_h = want_uv ? sz_x : 0;                                                // Householder vectors of the completion
+    const size_t sz_tau = want_uv ? align_up(sizeof(double) * (size_t)batch * Cn) : 0;
     const size_t sz_norm = align_up(sizeof(double) * (size_t)batch * R);
     const size_t sz_ord = align_up(sizeof(int) * (size_t)batch * R);
     const size_t sz_misc = align_up(sizeof(double) * (size_t)batch) + align_up(sizeof(int) * (size_t)batch) + 256;
     void* block = nullptr;
-    DNH_TRY(dnh_alloc_async(sz_x + sz_w + sz_big + sz_small + sz_z + sz_norm + sz_ord + sz_misc + align_up(sizeof(T) * (size_t)batch * K), stream, &block));
+    DNH_TRY(dnh_alloc_async(sz_x + sz_w + sz_big + sz_small + sz_z + sz_h + sz_tau + sz_norm + sz_ord + sz_misc + align_up(sizeof(T) * (size_t)batch * K), stream,
+                            &block));
     char* base = (char*)block;
     T* X = (T*)base;                       base += sz_x;
     T* W = want_uv ? (T*)base : nullptr;   base += sz_w;
     T* Big = (T*)base;                     base += sz_big;
     T* Small = (T*)base;                   base += sz_small;
     T* Z = (T*)base;                       base += sz_z;
+    T* Hh = (T*)base;                      base += sz_h;
+    double* tau = (double*)base;           base += sz_tau;
     double* norm = (double*)base;          base += sz_norm;
     int* order = (int*)base;               base += sz_ord;
     double* kmax = (double*)base;          base += align_up(sizeof(double) * (size_t)batch);
@@ -520,13 +581,20 @@ int32_t svd_impl(const DnhTensor* s, const DnhTensor* u, const DnhTensor* v, con
             for (int64_t b = 0; b < batch; b++) need_complement = need_complement || hr[(size_t)b] < R;
         }
         if (need_complement) {
-            hipLaunchKernelGGL((complement_projector_kernel<T>), dim3(cdiv(R, 256), (unsigned)R, (unsigned)batch), dim3(256), 0, stream, Z, Big, rank, R);
+            // Householder QR of the orthonormal columns found so far, then Q applied to the remaining unit vectors
+            hipLaunchKernelGGL((gather_u1_kernel<T>), dim3(cdiv(R, 256), (unsigned)Cn, (unsigned)batch), dim3(256), 0, stream, Hh, Big, rank, R, Cn);
+            for (int k = 0; k < Cn; k++) {
+                hipLaunchKernelGGL((house_vector_kernel<T>), dim3((unsigned)batch), dim3(kPairThreads), 0, stream, Hh, tau, rank, R, Cn, k);
+                if (k + 1 < Cn)
+                    hipLaunchKernelGGL((house_apply_kernel<T>), dim3((unsigned)(Cn - k - 1), (unsigned)batch), dim3(kPairThreads), 0, stream, Hh, Hh, tau, rank,
+                                       R, Cn, Cn, k, k + 1, 0);
+            }
             DNH_LAUNCH_CHECK();
-            DNH_TRY(jacobi_run<T>(Z, (T*)nullptr, batch, R, R, 0, counter, stream, "SVD (complement basis)"));
-            hipLaunchKernelGGL((column_norm_kernel<T>), dim3((unsigned)R, (unsigned)batch), dim3(kPairThreads), 0, stream, Z, norm, R, R, (int64_t)R * R);
-            hipLaunchKernelGGL(rank_kernel, dim3(cdiv(R, 256), (unsigned)batch), dim3(256), 0, stream, norm, order, R, 1);
-            hipLaunchKernelGGL((fill_complement_kernel<T>), dim3(cdiv(R, 256), (unsigned)R, (unsigned)batch), dim3(256), 0, stream, Big, Z, order, norm, rank,
-                               R);
+            hipLaunchKernelGGL((complement_seed_kernel<T>), dim3(cdiv(R, 256), (unsigned)R, (unsigned)batch), dim3(256), 0, stream, Z, rank, R);
+            for (int k = Cn - 1; k >= 0; k--)
+                hipLaunchKernelGGL((house_apply_kernel<T>), dim3((unsigned)R, (unsigned)batch), dim3(kPairThreads), 0, stream, Z, Hh, tau, rank, R, Cn, R, k, 0,
+                                   1);
+            hipLaunchKernelGGL((complement_store_kernel<T>), dim3(cdiv(R, 256), (unsigned)R, (unsigned)batch), dim3(256), 0, stream, Big, Z, rank, R);
             DNH_LAUNCH_CHECK();
         }
         {
