@@ -699,6 +699,92 @@ bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t strea
     return true;
 }
 
+// ---- integer types ------------------------------------------------------------------------------------------------------------
+// The reference's host backend computes dot for the types BLAS does not cover as multiply + sumAxis in the element type
+// (Host/HostBackend.fs:544-546), i.e. with wrapping arithmetic; its CUDA backend has no such path.  Wrapping is a ring
+// homomorphism, so products and sums are formed in the unsigned type of at least 32 bits and truncated once at the end:
+// bit-identical to wrapping at every step.  No matrix cores for 32/64-bit integers: a 64 x 64 tile per workgroup, a 4 x 4
+// block of outputs per thread, operands staged through LDS.
+template <class T>
+__global__ __launch_bounds__(256) void gemm_int_kernel(T* __restrict__ c, const T* __restrict__ a, const T* __restrict__ b, GemmArgs g) {
+    using U = typename std::conditional<sizeof(T) == 8, uint64_t, uint32_t>::type;
+    constexpr int TM = 64, TN = 64, TK = 16;
+    __shared__ U As[TK][TM + 4];
+    __shared__ U Bs[TK][TN + 4];
+    uint32_t bid = blockIdx.x;
+    const uint32_t tn = bid % g.tiles_n;
+    bid /= g.tiles_n;
+    const uint32_t tm = bid % g.tiles_m;
+    bid /= g.tiles_m;
+    int64_t oa = 0, ob = 0, oc = 0;
+    for (int d = g.nbatch - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
+        const uint32_t i = bid - q * g.bshape[d];
+        bid = q;
+        oa += (int64_t)i * g.bsa[d];
+        ob += (int64_t)i * g.bsb[d];
+        oc += (int64_t)i * g.bsc[d];
+    }
+    a += oa;
+    b += ob;
+    c += oc;
+    const int64_t m0 = (int64_t)tm * TM, n0 = (int64_t)tn * TN;
+    const int tid = threadIdx.x, tx = tid % 16, ty = tid / 16;
+    U acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = 0;
+    for (int64_t k0 = 0; k0 < g.K; k0 += TK) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int idx = tid + i * 256;
+            {
+                const int row = idx / TK, kk = idx % TK;
+                const int64_t m = m0 + row, k = k0 + kk;
+                As[kk][row] = (m < g.M && k < g.K) ? (U)a[m * g.sam + k * g.sak] : U(0);
+            }
+            {
+                const int kk = idx / TN, col = idx % TN;
+                const int64_t k = k0 + kk, n = n0 + col;
+                Bs[kk][col] = (k < g.K && n < g.N) ? (U)b[k * g.sbk + n * g.sbn] : U(0);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < TK; kk++) {
+            U av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; j++) bv[j] = Bs[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] += av[i] * bv[j];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int64_t m = m0 + ty * 4 + i, n = n0 + tx * 4 + j;
+            if (m < g.M && n < g.N) c[m * g.scm + n * g.scn] = (T)acc[i][j];
+        }
+}
+
+template <class T>
+int32_t launch_gemm_int(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hipStream_t stream) {
+    g.tiles_m = cdiv(g.M, 64);
+    g.tiles_n = cdiv(g.N, 64);
+    const int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
+    if (blocks > 0x7FFFFFFF) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: too many output tiles");
+    hipLaunchKernelGGL((gemm_int_kernel<T>), dim3((unsigned)blocks), dim3(256), 0, stream, c, a, b, g);
+    DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
+
 }  // namespace
 
 namespace dnh {
@@ -731,8 +817,7 @@ extern "C" int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTens
     DNH_TRY(check_tensor(a, "dnh_dot"));
     DNH_TRY(check_tensor(b, "dnh_dot"));
     if (t->dtype != a->dtype || t->dtype != b->dtype) return fail(DNH_ERR_INVALID_ARG, "dnh_dot: dtypes differ");
-    if (t->dtype != DNH_F32 && t->dtype != DNH_F64)
-        return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: only single and double have a device kernel; the frontend computes other types as multiply + sumAxis (Host/HostBackend.fs:544-546)");
+    if (t->dtype == DNH_BOOL) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: multiplication is not defined for bool");
     const int nt = t->ndims, na = a->ndims, nb = b->ndims;
     GemmArgs g;
     memset(&g, 0, sizeof(g));
@@ -771,6 +856,33 @@ extern "C" int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTens
     g.tiles_n = cdiv(g.N, BN);
     hipStream_t s = (hipStream_t)stream;
     int32_t st = DNH_OK;
+    if (!dtype_is_fp(t->dtype)) {
+        if (g.N == 1 && g.nbatch == 0 && g.K > 0) {
+            // vector forms: element-wise product into a temporary, then its fold along k: both at memory speed, whatever M and K are
+            const int es = dtype_size(t->dtype);
+            void* tmp = nullptr;
+            DNH_TRY(dnh_alloc_async((size_t)g.M * (size_t)g.K * es, s, &tmp));
+            DnhTensor pd, ad, bd;
+            memset(&pd, 0, sizeof(pd));
+            pd.base = tmp; pd.ndims = 2; pd.dtype = t->dtype;
+            pd.shape[0] = g.M; pd.shape[1] = g.K; pd.stride[0] = g.K; pd.stride[1] = 1;
+            ad = pd; ad.base = a->base; ad.offset = a->offset; ad.stride[0] = g.sam; ad.stride[1] = g.sak;
+            bd = pd; bd.base = b->base; bd.offset = b->offset; bd.stride[0] = 0; bd.stride[1] = g.sbk;
+            DnhTensor td = *t;
+            td.ndims = 1; td.shape[0] = g.M; td.stride[0] = g.scm;
+            st = dnh_binary(DNH_MULTIPLY, &pd, &ad, &bd, stream);
+            if (st == DNH_OK) st = dnh_reduce_last_axis(DNH_SUM, &td, &pd, stream);
+            (void)dnh_free_async(tmp, s);
+            return st;
+        }
+#define DNH_INT_DOT(DT, CT) case DT: return launch_gemm_int<CT>(g, (CT*)elem_ptr(t), (const CT*)elem_ptr(a), (const CT*)elem_ptr(b), batch, s);
+        switch (t->dtype) {
+            DNH_INT_DOT(DNH_U8, uint8_t) DNH_INT_DOT(DNH_I8, int8_t) DNH_INT_DOT(DNH_I32, int32_t) DNH_INT_DOT(DNH_U32, uint32_t)
+            DNH_INT_DOT(DNH_I64, int64_t) DNH_INT_DOT(DNH_U64, uint64_t)
+        }
+#undef DNH_INT_DOT
+        return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: unsupported element type");
+    }
     if (t->dtype == DNH_F32 && try_gemv<float>(g, (float*)elem_ptr(t), (const float*)elem_ptr(a), (const float*)elem_ptr(b), s, &st)) return st;
     if (t->dtype == DNH_F64 && try_gemv<double>(g, (double*)elem_ptr(t), (const double*)elem_ptr(a), (const double*)elem_ptr(b), s, &st)) return st;
     if (t->dtype == DNH_F32) return launch_gemm<float>(g, (float*)elem_ptr(t), (const float*)elem_ptr(a), (const float*)elem_ptr(b), batch, s);

@@ -235,7 +235,8 @@ int32_t dnh_true_indices(const DnhTensor* t_i64, const DnhTensor* src_bool, void
 /* ---------------------------------------------------------------------------------------------------
  * Dot: ITensorBackend VecVecDot / MatVecDot / MatMatDot / BatchedMatMatDot (TensorBackend.fs:137-140;
  * Host/HostBackend.fs:463-546).  The ranks of (t, a, b) select the variant exactly as Tensor.FillDot does
- * (Tensor.fs:2714-2730): (0,1,1) (1,2,1) (2,2,2) or (n,n,n) with n>2.  fp32 and fp64.
+ * (Tensor.fs:2714-2730): (0,1,1) (1,2,1) (2,2,2) or (n,n,n) with n>2.  fp32 and fp64 on the
+ * matrix cores; the integer types wrap like the host backend's multiply + sumAxis (HostBackend.fs:544-546); bool: status 2.
  * ------------------------------------------------------------------------------------------------- */
 int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream);
 

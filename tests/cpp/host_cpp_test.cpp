@@ -402,9 +402,9 @@ static void oracle_parity() {
         check_close("parity.f32.dot.batched.broadcast", ba.toDevice().dot(bb.toDevice()), o_dot(bab, bbb, {3, 2, 33, 17}), 0, 65 * 1.2e-7 * 65 * 4);
         HostT<float> v = randf({K});
         check_close("parity.f32.dot.matvec", a.toDevice().dot(v.toDevice()), o_dot(a, v, {M}), 0, K * 1.2e-7 * K * 4);
-        // like the reference's CUDA backend (BLAS for single and double only), integer dot is not a device operation
-        HostT<int32_t> ia = randi<int32_t>({37, 41}, -50, 50), ib = randi<int32_t>({41, 29}, -50, 50);
-        expect_throws<tn::NotSupportedException>("parity.i32.dot.notSupported", [&] { ia.toDevice().dot(ib.toDevice()); });
+        // integer dot wraps like the host backend's multiply + sumAxis (HostBackend.fs:544-546): bit-exact
+        HostT<int32_t> ia = randi<int32_t>({37, 41}, -2000000000, 2000000000), ib = randi<int32_t>({41, 29}, -2000000000, 2000000000);
+        check_exact("parity.i32.dot", ia.toDevice().dot(ib.toDevice()), o_dot(ia, ib, {37, 29}));
         HostT<double> da = HostT<double>({64, 48}), db = HostT<double>({48, 80});
         for (auto& x : *da.data) x = std::uniform_real_distribution<double>(-2, 2)(g_rng);
         for (auto& x : *db.data) x = std::uniform_real_distribution<double>(-2, 2)(g_rng);

@@ -149,10 +149,41 @@ def test_config5_block_small(H, G, rng):
     assert np.allclose(got.sum(axis=2), 1.0, atol=1e-5)
 
 
-def test_non_float_dot_not_supported(G):
-    a = G.ofNumpy(np.ones((4, 4), np.int32))
+def test_bool_dot_not_supported(G):
+    a = G.ofNumpy(np.ones((4, 4), np.bool_))
     with pytest.raises(NotImplementedError):
         a @ a
+
+
+@pytest.mark.parametrize("dt", [np.uint8, np.int8, np.int32, np.uint32, np.int64, np.uint64])
+def test_integer_dot_wraps_like_the_host_backend(H, G, rng, dt):
+    """The reference's host backend computes dot of the types BLAS does not cover as multiply + sumAxis in the element type
+    (Host/HostBackend.fs:544-546): wrapping arithmetic, so the result is bit-exact whatever the summation order."""
+    info = np.iinfo(dt)
+
+    def rnd(shape):
+        return rng.integers(info.min, info.max, size=shape, dtype=dt, endpoint=True)
+    for sa, sb in [((5, 3), (3, 3)), ((70, 130), (130, 65)), ((64, 300), (300, 64)), ((1, 1000), (1000, 1)), ((3, 2, 33, 40), (3, 2, 40, 17))]:
+        a, b = rnd(sa), rnd(sb)
+        ref, got = both(H, G, lambda a, b: a @ b, a, b)
+        assert ref.dtype == got.dtype == dt and np.array_equal(ref, got)
+        with np.errstate(over="ignore"):
+            assert np.array_equal(got, np.matmul(a, b))          # numpy's integer matmul wraps the same way
+    # transposed views, broadcast batch dimension, vector forms (strided vector), empty inner dimension
+    a, b = rnd((40, 33)), rnd((40, 17))
+    ref, got = both(H, G, lambda a, b: a.T @ b, a, b)
+    assert np.array_equal(ref, got)
+    a, b = rnd((4, 20, 30)), rnd((1, 30, 10))
+    ref, got = both(H, G, lambda a, b: a @ b, a, b)
+    assert np.array_equal(ref, got)
+    m, v = rnd((300, 5000)), rnd((10000,))
+    ref, got = both(H, G, lambda m, v: m @ v[0:10000][1:10000].reshape([9999])[0:5000], m, v)
+    assert np.array_equal(ref, got)
+    u, w = rnd((100000,)), rnd((100000,))
+    ref, got = both(H, G, lambda u, w: u @ w, u, w)
+    assert ref.shape == got.shape == () and np.array_equal(ref, got)
+    ref, got = both(H, G, lambda a, b: a @ b, np.zeros((5, 0), dt), np.zeros((0, 7), dt))
+    assert np.array_equal(got, np.zeros((5, 7), dt)) and np.array_equal(ref, got)
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
