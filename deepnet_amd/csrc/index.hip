@@ -56,6 +56,7 @@ __device__ __forceinline__ int64_t offset_of(const Lay& l, uint32_t i) {
 struct IndexArgs {
     Lay iter;                              // the iteration space: target (gather) or source (scatter)
     Lay other;                             // the indexed tensor: source (gather) or target (scatter)
+    int64_t other_shape[DNH_MAX_DIMS];     // its extents in full width: the indexed tensor may hold more than 2^32 elements
     const int64_t* idx[DNH_MAX_DIMS];      // per dimension of `other`; nullptr = identity
     int64_t idx_stride[DNH_MAX_DIMS][DNH_MAX_DIMS];
 };
@@ -72,7 +73,7 @@ __device__ __forceinline__ bool indexed_offset(const IndexArgs& a, const uint32_
         } else {
             j = pos[d];
         }
-        ok = ok && j >= 0 && j < (int64_t)a.other.shape[d];
+        ok = ok && j >= 0 && j < a.other_shape[d];
         o += j * a.other.stride[d];
     }
     *off = o;
@@ -125,6 +126,7 @@ int32_t make_index_args(IndexArgs* a, const DnhTensor* iter, const DnhTensor* ot
     memset(a, 0, sizeof(*a));
     a->iter = lay_of(iter);
     a->other = lay_of(other);
+    for (int d = 0; d < DNH_MAX_DIMS; d++) a->other_shape[d] = d < other->ndims ? other->shape[d] : 1;
     for (int d = 0; d < n_idx; d++) {
         if (idx[d]) {
             DNH_TRY(check_tensor(idx[d], what));
