@@ -258,6 +258,29 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6)):
             r = new([], dt)
             timed(6, f"VecVecDot 64Mi {nm}", 2 * (1 << 26) * sz, lambda i: [("dot", (D(r), D(u), D(v)))])
             del mats, u, v
+    if 7 in which:
+        # the step either side of every benchmark: host <-> device copies of 256 MiB (wall clock, synchronous calls)
+        import time
+        lib, check = T.lib, T.native.check
+        nbytes = 256 << 20
+        dev = new([nbytes], np.uint8)
+        dptr = dev.Storage.Pointer()
+        pinned = C.c_void_p()
+        check(lib.dnh_host_alloc(nbytes, C.byref(pinned)))
+        C.memset(pinned, 1, nbytes)
+        pageable = np.ones(nbytes, np.uint8)
+        for kind, hptr in (("pinned", pinned.value), ("pageable", pageable.ctypes.data)):
+            for name, call in (("H2D", lambda: lib.dnh_memcpy_h2d(dptr, hptr, nbytes, T.stream, 1)),
+                               ("D2H", lambda: lib.dnh_memcpy_d2h(hptr, dptr, nbytes, T.stream, 1))):
+                for _ in range(2):
+                    check(call())
+                t0 = time.perf_counter()
+                for _ in range(5):
+                    check(call())
+                ms = (time.perf_counter() - t0) / 5 * 1e3
+                log(f"[cfg7] {name} 256 MiB {kind:8s} host memory {ms:9.2f} ms  {nbytes / ms / 1e6:8.1f} GB/s")
+                results.append({"cfg": 7, "op": f"{name} {kind}", "ms": ms, "GBps": nbytes / ms / 1e6})
+        check(lib.dnh_host_free(pinned))
     return results
 
 
