@@ -215,6 +215,437 @@ __global__ __launch_bounds__(kPairThreads) void jacobi_round_reg_kernel(T* __res
     if (threadIdx.x == 0) *rotations = 1;   // a flag, not a count: every writer stores the same value, no atomic queue at one address
 }
 
+// ---- block rounds ---------------------------------------------------------------------------------------------------------
+// The same sweep on blocks of 16 columns: a workgroup takes a pair of blocks (32 columns), forms their 32 x 32 Gram matrix
+// G = B^T B in double precision on the matrix cores, diagonalises G by cyclic two-sided Jacobi rotations in LDS while
+// accumulating the rotations in Q (G <- J^T G J, Q <- Q J), and replaces the columns by B Q (and the same columns of W by
+// W Q), again on the matrix cores.  The entries of G are the very sums alpha, beta, gamma of the column-pair form, so the
+// rotation test is the same; one round touches the matrices once for 16 x 16 + 2 * 120 column pairs instead of one, which
+// divides the memory traffic of a sweep by 16.  A sweep in which no workgroup finds an entry of its G above the threshold
+// ends the iteration, as before.  There are only C / 32 pairs, too few workgroups for the two passes over the rows, so a round
+// is three launches: the partial Gram matrices of every (pair, piece of the rows); per pair the sum of the pieces and the
+// diagonalisation (Q to memory); Q applied to every (pair, piece of the rows of X and of W).
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+constexpr int kBlockCols = 16;
+#ifndef DNH_JACOBI_BLOCK_MIN_COLS
+#define DNH_JACOBI_BLOCK_MIN_COLS 64
+#endif
+constexpr int kBlockMinCols = DNH_JACOBI_BLOCK_MIN_COLS;   // below this the column-pair rounds are used
+
+// Four consecutive elements p[i .. i+3] of a column of `n` elements, raw: the caller converts (and zeroes what `ok4` excludes)
+// when it uses them, so that the loads of the next step stay in flight during the matrix instructions of the current one.
+template <class T>
+struct Raw4 {
+    T v[4];
+};
+template <class T>
+__device__ __forceinline__ Raw4<T> load4_raw(const T* __restrict__ p, int i, int n, bool ok, bool vec) {
+    Raw4<T> r;
+    if (vec && i + 4 <= n) {
+        typedef T V4 __attribute__((ext_vector_type(4), aligned(16)));
+        const V4 v = *reinterpret_cast<const V4*>(p + i);
+#pragma unroll
+        for (int j = 0; j < 4; j++) r.v[j] = v[j];
+    } else {
+#pragma unroll
+        for (int j = 0; j < 4; j++) r.v[j] = p[(ok && i + j < n) ? i + j : 0];
+    }
+    return r;
+}
+
+// Rows of M (`n` per column, columns of the two blocks at pcol / qcol) times Q: one wavefront per 16 rows.  Computed as
+// (Q^T M^T): operand lane l supplies Q[4s + l/16][16t + l%16] and M[row0 + l%16][column 4s + l/16]; accumulator register r
+// holds row l%16 of column 16t + 4r + l/16, so a store instruction writes 16 consecutive rows of four columns.
+template <class T, int NW>
+__device__ __forceinline__ void apply_block_rotation(T* __restrict__ m, int n, int begin, int end, int c, int pcol, int qcol, const double* __restrict__ Q, int wave,
+                                                     int lane) {
+    constexpr int STEP = NW * 16;
+    const int lc = lane & 15, lk = lane >> 4;
+    double qa[8][2];
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        qa[s][0] = Q[(4 * s + lk) * 32 + lc];
+        qa[s][1] = Q[(4 * s + lk) * 32 + 16 + lc];
+    }
+    int64_t off[8];
+    unsigned col_ok = 0;
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        const int col = (s < 4 ? pcol : qcol - 16) + 4 * s + lk;
+        if (col < c) col_ok |= 1u << s;
+        off[s] = col < c ? (int64_t)col * n : 0;
+    }
+    T cur[8], nxt[8];
+    int r0 = begin + wave * 16;
+    if (r0 < end) {
+        const int row = r0 + lc < n ? r0 + lc : 0;
+#pragma unroll
+        for (int s = 0; s < 8; s++) cur[s] = m[off[s] + row];
+    }
+    for (; r0 < end; r0 += STEP) {
+        const int rn = r0 + STEP;
+        if (rn < end) {
+            const int row = rn + lc < n ? rn + lc : 0;
+#pragma unroll
+            for (int s = 0; s < 8; s++) nxt[s] = m[off[s] + row];
+        }
+        const int row = r0 + lc;
+        const bool row_ok = row < n;
+        f64x4 acc0 = {0, 0, 0, 0}, acc1 = {0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const double xs = (row_ok && ((col_ok >> s) & 1u)) ? (double)cur[s] : 0.0;
+            acc0 = __builtin_amdgcn_mfma_f64_16x16x4f64(qa[s][0], xs, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f64_16x16x4f64(qa[s][1], xs, acc1, 0, 0, 0);
+        }
+        if (row_ok) {
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int cp = pcol + 4 * r + lk, cq = qcol + 4 * r + lk;
+                if (cp < c) m[(int64_t)cp * n + row] = (T)acc0[r];
+                if (cq < c) m[(int64_t)cq * n + row] = (T)acc1[r];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 8; s++) cur[s] = nxt[s];
+    }
+}
+
+// Partial Gram matrices: workgroup (pair, piece, matrix) covers rows [piece * chunk, (piece + 1) * chunk) (chunk a multiple of 16)
+// and writes G_pp, G_pq, G_qq (3 x 256 doubles) to partial[((matrix * pairs + pair) * pieces + piece) * 768].
+constexpr int kGramThreads = 256;
+template <class T>
+__global__ __launch_bounds__(kGramThreads) void jacobi_block_gram_kernel(const T* __restrict__ x, double* __restrict__ partial, int rows, int chunk, int c, int nbe,
+                                                                         int round, int64_t bsx) {
+    constexpr int NW = kGramThreads / 64;
+    __shared__ double part[NW][3][256];
+    int ba, bb;
+    pair_of(nbe, round, blockIdx.x, &ba, &bb);
+    const int nb = (c + kBlockCols - 1) / kBlockCols;
+    if (ba >= nb || bb >= nb) return;
+    const int pcol = (ba < bb ? ba : bb) * kBlockCols, qcol = (ba < bb ? bb : ba) * kBlockCols;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lc = lane & 15, lk = lane >> 4;
+    const T* xb = x + (int64_t)blockIdx.z * bsx;
+    const int begin = (int)blockIdx.y * chunk, end = begin + chunk < rows ? begin + chunk : rows;
+    // operand lane l supplies rows r0 + 4 (l/16) + j (j = 0..3 over four MFMAs) of column l%16 of each block
+    const bool okp = pcol + lc < c, okq = qcol + lc < c;
+    const T* xp = xb + (int64_t)(okp ? pcol + lc : 0) * rows;
+    const T* xq = xb + (int64_t)(okq ? qcol + lc : 0) * rows;
+    const bool vec = (rows & 3) == 0;
+    f64x4 gpp = {0, 0, 0, 0}, gpq = {0, 0, 0, 0}, gqq = {0, 0, 0, 0};
+    Raw4<T> ca, cb, na, nb4;
+    int r0 = begin + wave * 16;
+    if (r0 < end) {
+        ca = load4_raw(xp, r0 + 4 * lk, rows, okp, vec);
+        cb = load4_raw(xq, r0 + 4 * lk, rows, okq, vec);
+    }
+    for (; r0 < end; r0 += NW * 16) {
+        const int rn = r0 + NW * 16;
+        if (rn < end) {
+            na = load4_raw(xp, rn + 4 * lk, rows, okp, vec);
+            nb4 = load4_raw(xq, rn + 4 * lk, rows, okq, vec);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const bool in = r0 + 4 * lk + j < rows;
+            const double a = (in && okp) ? (double)ca.v[j] : 0.0;
+            const double b = (in && okq) ? (double)cb.v[j] : 0.0;
+            gpp = __builtin_amdgcn_mfma_f64_16x16x4f64(a, a, gpp, 0, 0, 0);
+            gpq = __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, gpq, 0, 0, 0);
+            gqq = __builtin_amdgcn_mfma_f64_16x16x4f64(b, b, gqq, 0, 0, 0);
+        }
+        ca = na;
+        cb = nb4;
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        part[wave][0][(4 * r + lk) * 16 + lc] = gpp[r];
+        part[wave][1][(4 * r + lk) * 16 + lc] = gpq[r];
+        part[wave][2][(4 * r + lk) * 16 + lc] = gqq[r];
+    }
+    __syncthreads();
+    double* out = partial + (((int64_t)blockIdx.z * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y) * 768;
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int s = 0; s < 3; s++) {
+        double v = 0;
+#pragma unroll
+        for (int k = 0; k < NW; k++) v += part[k][s][t];
+        out[s * 256 + t] = v;
+    }
+}
+
+// Single precision: the same two passes on v_mfma_f32_32x32x2_f32, whose accumulator is the whole 32 x 32 matrix.  Rounding
+// the sums of a piece to single precision perturbs gamma by about eps * |x_p| |x_q|, well below the rotation threshold
+// sqrt(rows) * eps * |x_p| |x_q|; the pieces are added in double precision.
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+__device__ __forceinline__ int block_pair_column(int k, int pcol, int qcol) { return k < 16 ? pcol + k : qcol + k - 16; }
+
+__global__ __launch_bounds__(kGramThreads) void jacobi_block_gram_f32_kernel(const float* __restrict__ x, double* __restrict__ partial, int rows, int chunk, int c,
+                                                                             int nbe, int round, int64_t bsx) {
+    constexpr int NW = kGramThreads / 64;
+    __shared__ float part[NW][3][256];
+    int ba, bb;
+    pair_of(nbe, round, blockIdx.x, &ba, &bb);
+    const int nb = (c + kBlockCols - 1) / kBlockCols;
+    if (ba >= nb || bb >= nb) return;
+    const int pcol = (ba < bb ? ba : bb) * kBlockCols, qcol = (ba < bb ? bb : ba) * kBlockCols;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lm = lane & 31, lk = lane >> 5;
+    const int begin = (int)blockIdx.y * chunk, end = begin + chunk < rows ? begin + chunk : rows;
+    // operand lane l supplies rows r0 + 8 h + 4 (l/32) + j (h = 0, 1; j = 0..3: eight MFMAs per 16 rows) of column l%32 of the pair
+    const int col = block_pair_column(lm, pcol, qcol);
+    const bool ok = col < c;
+    const float* xc = x + (int64_t)blockIdx.z * bsx + (int64_t)(ok ? col : 0) * rows;
+    const bool vec = (rows & 3) == 0;
+    f32x16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+    Raw4<float> c0, c1, n0, n1;
+    int r0 = begin + wave * 16;
+    if (r0 < end) {
+        c0 = load4_raw(xc, r0 + 4 * lk, rows, ok, vec);
+        c1 = load4_raw(xc, r0 + 8 + 4 * lk, rows, ok, vec);
+    }
+    for (; r0 < end; r0 += NW * 16) {
+        const int rn = r0 + NW * 16;
+        if (rn < end) {
+            n0 = load4_raw(xc, rn + 4 * lk, rows, ok, vec);
+            n1 = load4_raw(xc, rn + 8 + 4 * lk, rows, ok, vec);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float a = (ok && r0 + 4 * lk + j < rows) ? c0.v[j] : 0.0f;
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, a, acc, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float a = (ok && r0 + 8 + 4 * lk + j < rows) ? c1.v[j] : 0.0f;
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, a, acc, 0, 0, 0);
+        }
+        c0 = n0;
+        c1 = n1;
+    }
+    // accumulator register r of lane l holds G[8 (r/4) + 4 (l/32) + r%4][l%32]; the lower left block is the transpose of the upper right
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int row = 8 * (r >> 2) + 4 * lk + (r & 3);
+        if (row < 16) part[wave][lm < 16 ? 0 : 1][row * 16 + (lm & 15)] = acc[r];
+        else if (lm >= 16) part[wave][2][(row - 16) * 16 + lm - 16] = acc[r];
+    }
+    __syncthreads();
+    double* out = partial + (((int64_t)blockIdx.z * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y) * 768;
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int s = 0; s < 3; s++) {
+        double v = 0;
+#pragma unroll
+        for (int k = 0; k < NW; k++) v += (double)part[k][s][t];
+        out[s * 256 + t] = v;
+    }
+}
+
+// Rows [begin, end) of M times Q in single precision, 32 rows per wavefront step: operand lane l supplies Q[2s + l/32][l%32] and
+// M[row0 + l%32][column 2s + l/32]; accumulator register r holds row l%32 of column 8 (r/4) + 4 (l/32) + r%4: a store
+// instruction writes 32 consecutive rows (a whole 128-byte line) of two columns.
+template <int NW>
+__device__ __forceinline__ void apply_block_rotation_f32(float* __restrict__ m, int n, int begin, int end, int c, int pcol, int qcol, const double* __restrict__ Q,
+                                                         int wave, int lane) {
+    constexpr int STEP = NW * 32;
+    const int lm = lane & 31, lk = lane >> 5;
+    float qa[16];
+    int64_t off[16];
+    unsigned col_ok = 0;
+#pragma unroll
+    for (int s = 0; s < 16; s++) {
+        qa[s] = (float)Q[(2 * s + lk) * 32 + lm];
+        const int col = block_pair_column(2 * s + lk, pcol, qcol);
+        if (col < c) col_ok |= 1u << s;
+        off[s] = col < c ? (int64_t)col * n : 0;
+    }
+    float cur[16], nxt[16];
+    int r0 = begin + wave * 32;
+    if (r0 < end) {
+        const int row = r0 + lm < n ? r0 + lm : 0;
+#pragma unroll
+        for (int s = 0; s < 16; s++) cur[s] = m[off[s] + row];
+    }
+    for (; r0 < end; r0 += STEP) {
+        const int rn = r0 + STEP;
+        if (rn < end) {
+            const int row = rn + lm < n ? rn + lm : 0;
+#pragma unroll
+            for (int s = 0; s < 16; s++) nxt[s] = m[off[s] + row];
+        }
+        const int row = r0 + lm;
+        const bool row_ok = row < n;
+        f32x16 acc;
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+#pragma unroll
+        for (int s = 0; s < 16; s++) {
+            const float xs = (row_ok && ((col_ok >> s) & 1u)) ? cur[s] : 0.0f;
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[s], xs, acc, 0, 0, 0);
+        }
+        if (row_ok) {
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int col = block_pair_column(8 * (r >> 2) + 4 * lk + (r & 3), pcol, qcol);
+                if (col < c) m[(int64_t)col * n + row] = acc[r];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 16; s++) cur[s] = nxt[s];
+    }
+}
+
+// The second launch of a round, one workgroup per pair: G from the pieces, its diagonalisation; Q goes to qbuf[pair][32][32] and
+// flag[pair] says whether anything was rotated (the third launch skips the pair otherwise).  `full`: one cyclic sweep over all
+// 496 column pairs of the 32 (31 steps of 16 disjoint pairs); otherwise only the 256 pairs between the two blocks (16 steps): the
+// pairs inside a block were made orthogonal when the block last had its full round (one round of every sweep, a different one
+// each sweep so that the block that sits out changes) and are disturbed by the other rotations only to second order.
+constexpr int kSolveThreads = 256;
+template <class T>
+__global__ __launch_bounds__(kSolveThreads) void jacobi_block_solve_kernel(const double* __restrict__ partial, int pieces, double* __restrict__ qbuf,
+                                                                           int* __restrict__ flag, int c, int nbe, int round, int full, double tol,
+                                                                           int* rotations) {
+    __shared__ double G[32][33];
+    __shared__ double Q[32][33];
+    __shared__ double H[32][33];
+    __shared__ int above;
+    int ba, bb;
+    pair_of(nbe, round, blockIdx.x, &ba, &bb);
+    const int nb = (c + kBlockCols - 1) / kBlockCols;
+    if (ba >= nb || bb >= nb) return;
+    const int64_t pair_id = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
+    const double* part = partial + pair_id * pieces * 768;
+    if (threadIdx.x == 0) above = 0;
+    __syncthreads();
+    if (threadIdx.x < 256) {
+        const int t = threadIdx.x, i = t >> 4, j = t & 15;
+        double pp = 0, pq = 0, qq = 0;
+        for (int k = 0; k < pieces; k++) {
+            pp += part[k * 768 + t];
+            pq += part[k * 768 + 256 + t];
+            qq += part[k * 768 + 512 + t];
+        }
+        G[i][j] = pp;
+        G[i][16 + j] = pq;
+        G[16 + j][i] = pq;
+        G[16 + i][16 + j] = qq;
+    }
+    for (int e = threadIdx.x; e < 1024; e += kSolveThreads) Q[e >> 5][e & 31] = (e >> 5) == (e & 31) ? 1.0 : 0.0;
+    __syncthreads();
+    // anything to rotate at all?
+    for (int e = threadIdx.x; e < 1024; e += kSolveThreads) {
+        const int i = e >> 5, j = e & 31;
+        if (i < j) {
+            const double g = G[i][j];
+            if (g != 0.0 && fabs(g) > tol * sqrt(G[i][i] * G[j][j])) above = 1;
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) flag[pair_id] = above;
+    if (!above) return;   // uniform
+    if (threadIdx.x == 0) *rotations = 1;
+
+    // Two tasks per thread and step: pair k of the step and the indices i, i + 16.  Every thread derives its pair's rotation
+    // itself from the three entries of G (same inputs, same instructions: the same bits in every thread), rotates columns p, q
+    // of rows i, i + 16 of G into H and of Q in place, and after the barrier rows p, q of columns i, i + 16 of H back into G.
+    static_assert(kSolveThreads == 256, "two (pair, index) tasks per thread");
+    {
+        const int k = threadIdx.x & 15, i = threadIdx.x >> 4;
+        const double tol2 = tol * tol;
+        const int steps = full ? 31 : 16;
+        for (int r = 0; r < steps; r++) {
+            int p, q;
+            if (full) {
+                // pair k of round r among 32 players (pair_of without its divisions: r < 31, k < 16)
+                int a = k == 0 ? 31 : r + k, b = k == 0 ? r : r - k;
+                if (k != 0 && a >= 31) a -= 31;
+                if (b < 0) b += 31;
+                p = a < b ? a : b;
+                q = a < b ? b : a;
+            } else {
+                p = k;
+                q = 16 + ((k + r) & 15);
+            }
+            const double alpha = G[p][p], beta = G[q][q], gamma = G[p][q];
+            double cs = 1.0, sn = 0.0;
+            if (gamma * gamma > tol2 * alpha * beta) {
+                // tan of the rotation angle to single precision on operands scaled into [-1, 1] (an angle that is off by 1e-7 of
+                // itself leaves 1e-7 of gamma behind, far below what the next visit removes anyway); cos and sin from it in
+                // double precision, so that the rotation is orthogonal to working accuracy: 1 / sqrt(1 + t^2) by two Newton steps.
+                const double d = beta - alpha, g2 = 2.0 * gamma;
+                const double big = fabs(d) > fabs(g2) ? fabs(d) : fabs(g2);
+                const int e = __builtin_amdgcn_frexp_exp(big);
+                const float df = (float)ldexp(d, -e), gf = (float)ldexp(g2, -e);
+                const float hf = __builtin_sqrtf(df * df + gf * gf);
+                const float tf = gf * __builtin_amdgcn_rcpf(df >= 0.0f ? df + hf : df - hf);
+                double t = (double)tf;
+                if (tf == 0.0f) {   // |gamma| below single precision's range next to |beta - alpha|: the same formula in double precision
+                    const double zeta = d / g2;
+                    t = (zeta >= 0.0 ? 1.0 : -1.0) / (fabs(zeta) + sqrt(1.0 + zeta * zeta));
+                }
+                const double x = 1.0 + t * t;
+                double y = (double)__builtin_amdgcn_rsqf((float)x);
+                y = y * (1.5 - 0.5 * x * y * y);
+                y = y * (1.5 - 0.5 * x * y * y);
+                cs = y;
+                sn = y * t;
+            }
+#pragma unroll
+            for (int ii = i; ii < 32; ii += 16) {
+                const double u = G[ii][p], v = G[ii][q];
+                H[ii][p] = cs * u - sn * v;
+                H[ii][q] = sn * u + cs * v;
+                if (sn != 0.0) {
+                    const double qu = Q[ii][p], qv = Q[ii][q];
+                    Q[ii][p] = cs * qu - sn * qv;
+                    Q[ii][q] = sn * qu + cs * qv;
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int ii = i; ii < 32; ii += 16) {
+                const double u = H[p][ii], v = H[q][ii];
+                G[p][ii] = cs * u - sn * v;
+                G[q][ii] = sn * u + cs * v;
+            }
+            __syncthreads();
+        }
+    }
+    for (int e = threadIdx.x; e < 1024; e += kSolveThreads) qbuf[pair_id * 1024 + e] = Q[e >> 5][e & 31];
+}
+
+// The third launch: workgroup (pair, piece, matrix) applies its pair's Q to its piece of the rows of X (pieces 0 .. xpieces - 1) or
+// of W (the pieces after those).
+constexpr int kApplyThreads = 256;
+template <class T>
+__global__ __launch_bounds__(kApplyThreads) void jacobi_block_apply_kernel(T* __restrict__ x, T* __restrict__ w, const double* __restrict__ qbuf,
+                                                                           const int* __restrict__ flag, int rows, int chunk, int xpieces, int wrows, int wchunk,
+                                                                           int c, int nbe, int round, int64_t bsx, int64_t bsw) {
+    int ba, bb;
+    pair_of(nbe, round, blockIdx.x, &ba, &bb);
+    const int nb = (c + kBlockCols - 1) / kBlockCols;
+    if (ba >= nb || bb >= nb) return;
+    const int64_t pair_id = (int64_t)blockIdx.z * gridDim.x + blockIdx.x;
+    if (!flag[pair_id]) return;
+    const int pcol = (ba < bb ? ba : bb) * kBlockCols, qcol = (ba < bb ? bb : ba) * kBlockCols;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const double* Q = qbuf + pair_id * 1024;
+    if ((int)blockIdx.y < xpieces) {
+        const int begin = (int)blockIdx.y * chunk, end = begin + chunk < rows ? begin + chunk : rows;
+        if constexpr (sizeof(T) == 4) apply_block_rotation_f32<kApplyThreads / 64>(x + (int64_t)blockIdx.z * bsx, rows, begin, end, c, pcol, qcol, Q, wave, lane);
+        else apply_block_rotation<T, kApplyThreads / 64>(x + (int64_t)blockIdx.z * bsx, rows, begin, end, c, pcol, qcol, Q, wave, lane);
+    } else {
+        const int begin = ((int)blockIdx.y - xpieces) * wchunk, end = begin + wchunk < wrows ? begin + wchunk : wrows;
+        if constexpr (sizeof(T) == 4) apply_block_rotation_f32<kApplyThreads / 64>(w + (int64_t)blockIdx.z * bsw, wrows, begin, end, c, pcol, qcol, Q, wave, lane);
+        else apply_block_rotation<T, kApplyThreads / 64>(w + (int64_t)blockIdx.z * bsw, wrows, begin, end, c, pcol, qcol, Q, wave, lane);
+    }
+}
+
 // identity matrices [batch][n][n]
 template <class T>
 __global__ __launch_bounds__(256) void identity_kernel(T* w, int n, int64_t total) {
@@ -427,17 +858,63 @@ __global__ __launch_bounds__(256) void shift_diagonal_kernel(T* __restrict__ x, 
 
 __global__ void clear_int_kernel(int* p) { *p = 0; }
 
+size_t align_up(size_t b) { return (b + 255) / 256 * 256; }
+
 // Sweeps until a sweep rotates nothing.  x: [batch][c][rows], w: [batch][c][wrows] or null.
 template <class T>
 int32_t jacobi_run(T* x, T* w, int64_t batch, int rows, int c, int wrows, int* counter, hipStream_t stream, const char* what) {
     if (c < 2 || batch == 0 || rows == 0) return DNH_OK;
     const int ce = c + (c & 1);
     const double tol = sqrt((double)rows) * (double)std::numeric_limits<T>::epsilon();   // as LAPACK's Jacobi SVD (xGESVJ)
+    // block rounds: three launches per round.  Rows are cut into pieces (multiples of 32 rows, at least 128) so that the Gram and
+    // the apply launches bring about four workgroups per CU.
+    const bool blocked = c >= kBlockMinCols && batch <= 65535;
+    const int nb = (c + kBlockCols - 1) / kBlockCols, nbe = nb + (nb & 1), pairs = nbe / 2;
+    int xpieces = 1, chunk = rows, wpieces = 0, wchunk = 32;
+    double *partial = nullptr, *qbuf = nullptr;
+    int* flag = nullptr;
+    void* block_ws = nullptr;
+    if (blocked) {
+        const int64_t want = std::max<int64_t>(1, (int64_t)4 * device_cus() / ((int64_t)pairs * batch));
+        xpieces = (int)std::max<int64_t>(1, std::min<int64_t>(want, rows / 128));
+        chunk = (int)cdiv(cdiv(rows, xpieces), 32) * 32;
+        xpieces = (int)cdiv(rows, chunk);
+        if (w && wrows > 0) {
+            wpieces = (int)std::max<int64_t>(1, std::min<int64_t>(want, wrows / 128));
+            wchunk = (int)cdiv(cdiv(wrows, wpieces), 32) * 32;
+            wpieces = (int)cdiv(wrows, wchunk);
+        }
+        const size_t sz_part = align_up(sizeof(double) * 768 * (size_t)xpieces * pairs * batch);
+        const size_t sz_q = align_up(sizeof(double) * 1024 * (size_t)pairs * batch);
+        DNH_TRY(dnh_alloc_async(sz_part + sz_q + sizeof(int) * (size_t)pairs * batch, stream, &block_ws));
+        partial = (double*)block_ws;
+        qbuf = (double*)((char*)block_ws + sz_part);
+        flag = (int*)((char*)block_ws + sz_part + sz_q);
+    }
+    struct Release {
+        void* p;
+        hipStream_t s;
+        ~Release() { if (p) (void)dnh_free_async(p, s); }
+    } release{block_ws, stream};
     for (int sweep = 0; sweep < kMaxSweeps; sweep++) {
         hipLaunchKernelGGL(clear_int_kernel, dim3(1), dim3(1), 0, stream, counter);
         const int longest = rows > wrows ? rows : wrows;
         const dim3 grid((unsigned)(ce / 2), (unsigned)batch);
 #define DNH_ROUND(KERNEL) hipLaunchKernelGGL((KERNEL), grid, dim3(kPairThreads), 0, stream, x, w, rows, c, ce, r, wrows, (int64_t)c * rows, (int64_t)c * wrows, tol, counter)
+        if (blocked) {
+            for (int r = 0; r < nbe - 1; r++) {
+                if constexpr (sizeof(T) == 4)
+                    hipLaunchKernelGGL(jacobi_block_gram_f32_kernel, dim3((unsigned)pairs, (unsigned)xpieces, (unsigned)batch), dim3(kGramThreads), 0, stream, x,
+                                       partial, rows, chunk, c, nbe, r, (int64_t)c * rows);
+                else
+                    hipLaunchKernelGGL((jacobi_block_gram_kernel<T>), dim3((unsigned)pairs, (unsigned)xpieces, (unsigned)batch), dim3(kGramThreads), 0, stream, x,
+                                       partial, rows, chunk, c, nbe, r, (int64_t)c * rows);
+                hipLaunchKernelGGL((jacobi_block_solve_kernel<T>), dim3((unsigned)pairs, (unsigned)batch), dim3(kSolveThreads), 0, stream, partial, xpieces, qbuf,
+                                   flag, c, nbe, r, (r == sweep % (nbe - 1)) ? 1 : 0, tol, counter);
+                hipLaunchKernelGGL((jacobi_block_apply_kernel<T>), dim3((unsigned)pairs, (unsigned)(xpieces + wpieces), (unsigned)batch), dim3(kApplyThreads), 0,
+                                   stream, x, w, qbuf, flag, rows, chunk, xpieces, wrows, wchunk, c, nbe, r, (int64_t)c * rows, (int64_t)c * wrows);
+            }
+        } else
         for (int r = 0; r < ce - 1; r++) {
             if (longest <= 1 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 1>));
             else if (longest <= 4 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 4>));
@@ -455,7 +932,6 @@ int32_t jacobi_run(T* x, T* w, int64_t batch, int rows, int c, int wrows, int* c
     return fail(DNH_ERR_NO_CONVERGENCE, "%s did not converge in %d sweeps", what, kMaxSweeps);
 }
 
-size_t align_up(size_t b) { return (b + 255) / 256 * 256; }
 
 // Fills a dense row-major descriptor of `t`'s shape over `base`.
 DnhTensor dense_like(const DnhTensor* t, void* base) {
