@@ -695,15 +695,56 @@ __global__ __launch_bounds__(256) void max_key_kernel(const double* __restrict__
     if (threadIdx.x == 0) kmax[blockIdx.x] = fmax(fmax(red[0], red[1]), fmax(red[2], red[3]));
 }
 
+// Scaling by a power of two (exact): every matrix is brought to a largest magnitude in [0.5, 1) before the sweeps, so that the
+// squares summed in the Gram entries neither overflow nor vanish whatever the magnitude of the input (single precision sums
+// them on the matrix cores in single precision); the values are scaled back when they are written.
+__global__ __launch_bounds__(64) void clear_scale_kernel(unsigned long long* maxbits, int count) {
+    const int i = blockIdx.x * 64 + threadIdx.x;
+    if (i < count) maxbits[i] = 0ull;
+}
+template <class T>
+__global__ __launch_bounds__(256) void max_abs_kernel(const T* __restrict__ x, unsigned long long* __restrict__ maxbits, int64_t per_matrix) {
+    __shared__ double red[4];
+    const T* xb = x + (int64_t)blockIdx.y * per_matrix;
+    double m = 0.0;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < per_matrix; i += (int64_t)gridDim.x * 256) {
+        const double v = fabs((double)xb[i]);
+        m = v > m ? v : m;   // NaN never enters
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const double other = __shfl_xor(m, o);
+        m = other > m ? other : m;
+    }
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int k = 1; k < 4; k++) m = red[k] > m ? red[k] : m;
+        atomicMax(maxbits + blockIdx.y, (unsigned long long)__double_as_longlong(m));   // non-negative doubles order like their bits
+    }
+}
+__device__ __forceinline__ int scale_exponent(unsigned long long bits) {
+    const double m = __longlong_as_double((long long)bits);
+    return (m > 0.0 && m <= 1.7976931348623157e308) ? __builtin_amdgcn_frexp_exp(m) : 0;
+}
+template <class T>
+__global__ __launch_bounds__(256) void scale_down_kernel(T* __restrict__ x, const unsigned long long* __restrict__ maxbits, int* __restrict__ exps,
+                                                         int64_t per_matrix) {
+    const int e = scale_exponent(maxbits[blockIdx.y]);
+    if (blockIdx.x == 0 && threadIdx.x == 0) exps[blockIdx.y] = e;
+    if (e == 0) return;
+    T* xb = x + (int64_t)blockIdx.y * per_matrix;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < per_matrix; i += (int64_t)gridDim.x * 256) xb[i] = (T)ldexp((double)xb[i], -e);
+}
+
 // out[b][k] = (T)(key[b][order[b][k]] + shift[b] * sign) for k < count
 template <class T>
 __global__ __launch_bounds__(256) void pick_values_kernel(T* __restrict__ out, const double* __restrict__ key, const int* __restrict__ order,
-                                                          const double* __restrict__ shift, double sign, int c, int count) {
+                                                          const double* __restrict__ shift, double sign, const int* __restrict__ exps, int c, int count) {
     const int k = blockIdx.x * 256 + threadIdx.x;
     if (k >= count) return;
     const int64_t b = blockIdx.y;
     const double v = key[b * c + order[b * c + k]] + (shift ? sign * shift[b] : 0.0);
-    out[b * count + k] = (T)v;
+    out[b * count + k] = (T)ldexp(v, exps[b]);
 }
 
 // Row-major output matrix [b][n][n] whose column k is column order[k] of the column-major work matrix src ([b][c][n]),
@@ -860,6 +901,15 @@ __global__ void clear_int_kernel(int* p) { *p = 0; }
 
 size_t align_up(size_t b) { return (b + 255) / 256 * 256; }
 
+// Scales every matrix of x ([batch][per_matrix]) to a largest magnitude in [0.5, 1); exps[b] receives the exponent taken out.
+template <class T>
+void prescale(T* x, int64_t batch, int64_t per_matrix, unsigned long long* maxbits, int* exps, hipStream_t stream) {
+    const unsigned blocks = (unsigned)std::max<int64_t>(1, std::min<int64_t>(cdiv(per_matrix, 256 * 8), 1024));
+    hipLaunchKernelGGL(clear_scale_kernel, dim3(cdiv(batch, 64)), dim3(64), 0, stream, maxbits, (int)batch);
+    hipLaunchKernelGGL((max_abs_kernel<T>), dim3(blocks, (unsigned)batch), dim3(256), 0, stream, x, maxbits, per_matrix);
+    hipLaunchKernelGGL((scale_down_kernel<T>), dim3(blocks, (unsigned)batch), dim3(256), 0, stream, x, maxbits, exps, per_matrix);
+}
+
 // Sweeps until a sweep rotates nothing.  x: [batch][c][rows], w: [batch][c][wrows] or null.
 template <class T>
 int32_t jacobi_run(T* x, T* w, int64_t batch, int rows, int c, int wrows, int* counter, hipStream_t stream, const char* what) {
@@ -992,7 +1042,8 @@ int32_t svd_impl(const DnhTensor* s, const DnhTensor* u, const DnhTensor* v, con
     const size_t sz_tau = want_uv ? align_up(sizeof(double) * (size_t)batch * Cn) : 0;
     const size_t sz_norm = align_up(sizeof(double) * (size_t)batch * R);
     const size_t sz_ord = align_up(sizeof(int) * (size_t)batch * R);
-    const size_t sz_misc = align_up(sizeof(double) * (size_t)batch) + align_up(sizeof(int) * (size_t)batch) + 256;
+    const size_t sz_misc = align_up(sizeof(double) * (size_t)batch) + align_up(sizeof(int) * (size_t)batch) + 256 + align_up(sizeof(unsigned long long) * (size_t)batch) +
+                           align_up(sizeof(int) * (size_t)batch);
     void* block = nullptr;
     DNH_TRY(dnh_alloc_async(sz_x + sz_w + sz_big + sz_small + sz_z + sz_h + sz_tau + sz_norm + sz_ord + sz_misc + align_up(sizeof(T) * (size_t)batch * K), stream,
                             &block));
@@ -1009,6 +1060,8 @@ int32_t svd_impl(const DnhTensor* s, const DnhTensor* u, const DnhTensor* v, con
     double* kmax = (double*)base;          base += align_up(sizeof(double) * (size_t)batch);
     int* rank = (int*)base;                base += align_up(sizeof(int) * (size_t)batch);
     int* counter = (int*)base;             base += 256;
+    unsigned long long* maxbits = (unsigned long long*)base;   base += align_up(sizeof(unsigned long long) * (size_t)batch);
+    int* exps = (int*)base;                base += align_up(sizeof(int) * (size_t)batch);
     T* Sv = (T*)base;
 
     auto body = [&]() -> int32_t {
@@ -1023,6 +1076,7 @@ int32_t svd_impl(const DnhTensor* s, const DnhTensor* u, const DnhTensor* v, con
             else      { xd.stride[nd - 2] = R; xd.stride[nd - 1] = 1; }   // A[i][j] -> X[i][j], R = N: column i of X = row i of A
         }
         DNH_TRY(dnh_copy(&xd, src, stream));
+        prescale<T>(X, batch, (int64_t)Cn * R, maxbits, exps, stream);
         if (want_uv) {
             const int64_t total = batch * Cn * Cn;
             hipLaunchKernelGGL((identity_kernel<T>), dim3(cdiv(total, 256)), dim3(256), 0, stream, W, Cn, total);
@@ -1031,7 +1085,7 @@ int32_t svd_impl(const DnhTensor* s, const DnhTensor* u, const DnhTensor* v, con
         hipLaunchKernelGGL((column_norm_kernel<T>), dim3((unsigned)Cn, (unsigned)batch), dim3(kPairThreads), 0, stream, X, norm, R, Cn, (int64_t)Cn * R);
         hipLaunchKernelGGL(rank_kernel, dim3(cdiv(Cn, 256), (unsigned)batch), dim3(256), 0, stream, norm, order, Cn, 1);
         hipLaunchKernelGGL((pick_values_kernel<T>), dim3(cdiv(K, 256), (unsigned)batch), dim3(256), 0, stream, Sv, norm, order, (const double*)nullptr, 0.0,
-                           Cn, K);
+                           exps, Cn, K);
         DNH_LAUNCH_CHECK();
         {
             DnhTensor sd = dense_like(s, Sv);
@@ -1095,7 +1149,7 @@ int32_t eig_impl(int32_t part, const DnhTensor* vals, const DnhTensor* vecs, con
     const size_t sz_norm = align_up(sizeof(double) * (size_t)n);
     const size_t sz_ord = align_up(sizeof(int) * (size_t)n);
     void* block = nullptr;
-    DNH_TRY(dnh_alloc_async(4 * sz_m + sz_norm + sz_ord + 512 + align_up(sizeof(T) * (size_t)n), stream, &block));
+    DNH_TRY(dnh_alloc_async(4 * sz_m + sz_norm + sz_ord + 1024 + align_up(sizeof(T) * (size_t)n), stream, &block));
     char* base = (char*)block;
     T* A = (T*)base;               base += sz_m;   // dense copy of src
     T* X = (T*)base;               base += sz_m;   // mirrored triangle + mu I (symmetric: its rows are its columns)
@@ -1105,11 +1159,14 @@ int32_t eig_impl(int32_t part, const DnhTensor* vals, const DnhTensor* vecs, con
     int* order = (int*)base;       base += sz_ord;
     double* mu = (double*)base;    base += 256;
     int* counter = (int*)base;     base += 256;
+    unsigned long long* maxbits = (unsigned long long*)base;   base += 256;
+    int* exps = (int*)base;        base += 256;
     T* Vals = (T*)base;
     auto body = [&]() -> int32_t {
         DnhTensor ad = dense_like(src, A);
         DNH_TRY(dnh_copy(&ad, src, stream));
         hipLaunchKernelGGL((symmetrize_kernel<T>), dim3(cdiv(n, 256), (unsigned)n), dim3(256), 0, stream, X, A, n, part == 1 ? 1 : 0);
+        prescale<T>(X, 1, (int64_t)n * n, maxbits, exps, stream);
         hipLaunchKernelGGL((column_norm_kernel<T>), dim3((unsigned)n, 1), dim3(kPairThreads), 0, stream, X, norm, n, n, (int64_t)n * n);
         hipLaunchKernelGGL(frobenius_kernel, dim3(1), dim3(256), 0, stream, norm, mu, n);
         hipLaunchKernelGGL((shift_diagonal_kernel<T>), dim3(cdiv(n, 256)), dim3(256), 0, stream, X, mu, n);
@@ -1119,7 +1176,7 @@ int32_t eig_impl(int32_t part, const DnhTensor* vals, const DnhTensor* vecs, con
         // the column norms are lambda + mu >= 0; ascending eigenvalues, eigenvector k = column order[k] of W
         hipLaunchKernelGGL((column_norm_kernel<T>), dim3((unsigned)n, 1), dim3(kPairThreads), 0, stream, X, norm, n, n, (int64_t)n * n);
         hipLaunchKernelGGL(rank_kernel, dim3(cdiv(n, 256), 1), dim3(256), 0, stream, norm, order, n, 0);
-        hipLaunchKernelGGL((pick_values_kernel<T>), dim3(cdiv(n, 256), 1), dim3(256), 0, stream, Vals, norm, order, (const double*)mu, -1.0, n, n);
+        hipLaunchKernelGGL((pick_values_kernel<T>), dim3(cdiv(n, 256), 1), dim3(256), 0, stream, Vals, norm, order, (const double*)mu, -1.0, exps, n, n);
         hipLaunchKernelGGL((scatter_columns_kernel<T>), dim3(cdiv(n, 256), (unsigned)n, 1), dim3(256), 0, stream, Out, W, order, (const double*)nullptr,
                            (const double*)nullptr, 0.0, n, n, (int64_t)n * n);
         DNH_LAUNCH_CHECK();

@@ -130,3 +130,39 @@ def test_decompositions_need_floating_point_and_matrices(G):
         T.symmetricEigenDecomposition("Upper", G.ofNumpy(np.ones((2, 3), np.float32)))
     with pytest.raises(ValueError):
         T.pseudoInvert(G.ofNumpy(np.ones((5, 3), np.float32)))     # the reference's pseudoInvert only takes square matrices
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", [(3, 96, 80), (1030, 200), (200, 1030), (2, 257, 129)])
+def test_svd_block_rounds(H, G, rng, dt, shape):
+    """64 columns and more take the block rounds: batches, several pieces of the rows, a last block of fewer than 16 columns, an odd
+    number of blocks, row counts that are not multiples of 4."""
+    a = rng.standard_normal(shape).astype(dt)
+    (ur, sr, vr), (u, s, v) = both(H, G, lambda x: type(x).SVD(x), a)
+    check_svd(a, u, s, v, sr)
+    ref, got = both(H, G, lambda x: type(x).SVDWithoutUV(x), a)
+    assert np.abs(got.astype(np.float64) - ref).max() <= tol_of(dt, max(shape[-2:])) * np.abs(ref).max()
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_svd_block_rounds_rank_deficient_and_graded(H, G, rng, dt):
+    low = (rng.standard_normal((300, 40)) @ rng.standard_normal((40, 100))).astype(dt)          # rank 40 of 100
+    graded = (rng.standard_normal((150, 90)) * np.logspace(0, -5 if dt == np.float32 else -12, 90)).astype(dt)
+    for a in (low, graded, np.zeros((70, 70), dt), np.eye(80, dtype=dt)):
+        (ur, sr, vr), (u, s, v) = both(H, G, lambda x: type(x).SVD(x), a)
+        check_svd(a, u, s, v, sr)
+
+
+@pytest.mark.parametrize("dt,scale", [(np.float32, 1e-25), (np.float32, 1e25), (np.float64, 1e-170), (np.float64, 1e170)])
+@pytest.mark.parametrize("n", [6, 80])
+def test_extreme_magnitudes(H, G, rng, dt, scale, n):
+    """Entries whose squares leave the element type's range: the work matrix is scaled by a power of two first."""
+    a = (rng.standard_normal((n + 3, n)) * scale).astype(dt)
+    (ur, sr, vr), (u, s, v) = both(H, G, lambda x: type(x).SVD(x), a)
+    assert np.all(np.isfinite(s)) and s[0] > 0
+    check_svd(a, u, s, v, sr)
+    b = rng.standard_normal((n, n))
+    sym = ((b + b.T) / 2 * scale).astype(dt)
+    (wr, vr2), (w, v2) = both(H, G, lambda x: type(x).symmetricEigenDecomposition("Upper", x), sym)
+    assert np.all(np.isfinite(w)) and np.abs(w).max() > 0
+    check_eig(sym, w, v2, wr)
