@@ -11,7 +11,7 @@
 // number as with the eigenvalues of A^T A).
 //
 //   SVD of A (M x N):  the side with fewer vectors plays W (it comes out complete); the taller side's vectors are the
-//     normalised columns of X for the singular values above max(M, N) * eps * sigma_max, and an orthonormal basis of their
+//     normalised columns of X for the singular values above 4 eps * sigma_max, and an orthonormal basis of their
 //     complement for the rest: the Householder QR of the columns found so far, Q^T U1 = [D; 0], and Q applied to the unit
 //     vectors that remain.
 //   Symmetric eigendecomposition:  the chosen triangle is mirrored, the matrix shifted by mu = its Frobenius norm so that it is
@@ -1092,7 +1092,9 @@ int32_t svd_impl(const DnhTensor* s, const DnhTensor* u, const DnhTensor* v, con
             DNH_TRY(dnh_copy(s, &sd, stream));
         }
         if (!want_uv) return DNH_OK;
-        const double rel = (double)R * (double)std::numeric_limits<T>::epsilon();
+        // A column of X is normalised into a vector when its norm is above 4 eps sigma_max: the sweeps end on a test relative to the
+        // norms, so even short columns are orthogonal to the others to sqrt(R) eps; below that a column is rounding residue.
+        const double rel = 4.0 * (double)std::numeric_limits<T>::epsilon();
         hipLaunchKernelGGL(max_key_kernel, dim3((unsigned)batch), dim3(256), 0, stream, norm, kmax, Cn);
         hipLaunchKernelGGL(numeric_rank_kernel, dim3((unsigned)batch), dim3(256), 0, stream, norm, kmax, rel, Cn, rank);
         // short side: W's columns in the order of the singular values (always complete)
