@@ -227,10 +227,7 @@ __global__ __launch_bounds__(kPairThreads) void jacobi_round_reg_kernel(T* __res
 // diagonalisation (Q to memory); Q applied to every (pair, piece of the rows of X and of W).
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 constexpr int kBlockCols = 16;
-#ifndef DNH_JACOBI_BLOCK_MIN_COLS
-#define DNH_JACOBI_BLOCK_MIN_COLS 64
-#endif
-constexpr int kBlockMinCols = DNH_JACOBI_BLOCK_MIN_COLS;   // below this the column-pair rounds are used
+constexpr int kBlockMinCols = 64;   // below this the column-pair rounds are used
 
 // Four consecutive elements p[i .. i+3] of a column of `n` elements, raw: the caller converts (and zeroes what `ok4` excludes)
 // when it uses them, so that the loads of the next step stay in flight during the matrix instructions of the current one.
@@ -367,6 +364,7 @@ __global__ __launch_bounds__(kGramThreads) void jacobi_block_gram_kernel(const T
     __syncthreads();
     double* out = partial + (((int64_t)blockIdx.z * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y) * 768;
     const int t = threadIdx.x;
+    if (t < 256)
 #pragma unroll
     for (int s = 0; s < 3; s++) {
         double v = 0;
@@ -437,6 +435,7 @@ __global__ __launch_bounds__(kGramThreads) void jacobi_block_gram_f32_kernel(con
     __syncthreads();
     double* out = partial + (((int64_t)blockIdx.z * gridDim.x + blockIdx.x) * gridDim.y + blockIdx.y) * 768;
     const int t = threadIdx.x;
+    if (t < 256)
 #pragma unroll
     for (int s = 0; s < 3; s++) {
         double v = 0;
