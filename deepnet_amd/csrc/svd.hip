@@ -7,8 +7,8 @@
 // applied to the columns of W, which starts as the identity.  The C / 2 pairs of a round of the round-robin schedule are
 // disjoint, so a round is one launch with one workgroup per pair and matrix; C - 1 rounds visit every pair once (a sweep).
 // When a sweep rotates nothing, X = A W has orthogonal columns: their norms are the singular values, the normalised
-// columns the left vectors, W the right vectors.  Relative accuracy is that of the rotations (no squaring of the condition
-// number as with the eigenvalues of A^T A).
+// columns the left vectors, W the right vectors.  With 64 columns or more the sweeps run on blocks of 16 columns (see "block
+// rounds" below): the same rotations, found from the 32 x 32 Gram matrix of a pair of blocks and applied as one 32 x 32 factor.
 //
 //   SVD of A (M x N):  the side with fewer vectors plays W (it comes out complete); the taller side's vectors are the
 //     normalised columns of X for the singular values above 4 eps * sigma_max, and an orthonormal basis of their
