@@ -2,13 +2,11 @@
 // 145).  The reference's host backend calls LAPACK gesdd / syevd (Tensor/Tensor/Host/HostBackend.fs:579-628); its CUDA backend
 // does not implement either (Tensor/Tensor/Cuda/CudaBackend.fs:486-492).
 //
-// Both run on one-sided Jacobi (Hestenes) rotations, which need nothing but column pairs: for the columns x_p, x_q of a work
-// matrix X (R rows, C <= R columns, every column contiguous) a plane rotation makes them orthogonal, and the same rotation is
-// applied to the columns of W, which starts as the identity.  The C / 2 pairs of a round of the round-robin schedule are
-// disjoint, so a round is one launch with one workgroup per pair and matrix; C - 1 rounds visit every pair once (a sweep).
-// When a sweep rotates nothing, X = A W has orthogonal columns: their norms are the singular values, the normalised
-// columns the left vectors, W the right vectors.  With 64 columns or more the sweeps run on blocks of 16 columns (see "block
-// rounds" below): the same rotations, found from the 32 x 32 Gram matrix of a pair of blocks and applied as one 32 x 32 factor.
+// Both run on one-sided Jacobi (Hestenes) rotations: for two columns x_p, x_q of a work matrix X (R rows, C <= R columns, every
+// column contiguous) a plane rotation makes them orthogonal, and the same rotation is applied to the columns of W, which starts
+// as the identity.  When a sweep over all pairs rotates nothing, X = A W has orthogonal columns: their norms are the singular
+// values, the normalised columns the left vectors, W the right vectors.  The sweeps run on blocks of 16 columns (see "block
+// rounds" below): the rotations of a pair of blocks are found from its 32 x 32 Gram matrix and applied as one 32 x 32 factor.
 //
 //   SVD of A (M x N):  the side with fewer vectors plays W (it comes out complete); the taller side's vectors are the
 //     normalised columns of X for the singular values above 4 eps * sigma_max, and an orthonormal basis of their
@@ -44,30 +42,7 @@ __device__ __forceinline__ void pair_of(int ce, int r, int k, int* a, int* b) {
     }
 }
 
-// Sums of three values over a wavefront, left in lane 63, through DPP lane moves (see wave_argmax.h): row shifts by 1, 2, 4, 8
-// add up each row of 16 lanes into its lane 15 (a lane without a source adds zero), two row broadcasts carry the row sums on.
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ double dpp_fetch_or_zero(double v) {
-    const long long b = __double_as_longlong(v);
-    const int lo = __builtin_amdgcn_update_dpp(0, (int)(unsigned)(b & 0xFFFFFFFFLL), CTRL, ROW_MASK, 0xF, false);
-    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), CTRL, ROW_MASK, 0xF, false);
-    return __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
-}
-template <int CTRL, int ROW_MASK>
-__device__ __forceinline__ void sum3_step(double& a, double& b, double& c) {
-    a += dpp_fetch_or_zero<CTRL, ROW_MASK>(a);
-    b += dpp_fetch_or_zero<CTRL, ROW_MASK>(b);
-    c += dpp_fetch_or_zero<CTRL, ROW_MASK>(c);
-}
-__device__ __forceinline__ void wave_sum3_to_lane63(double& a, double& b, double& c) {
-    sum3_step<0x111, 0xF>(a, b, c);   // row_shr:1
-    sum3_step<0x112, 0xF>(a, b, c);   // row_shr:2: lane i now holds the sum of lanes i-3 .. i of its row
-    sum3_step<0x114, 0xF>(a, b, c);   // row_shr:4
-    sum3_step<0x118, 0xF>(a, b, c);   // row_shr:8: lane 15 of a row holds the row's sum
-    sum3_step<0x142, 0xA>(a, b, c);   // row_bcast:15 into rows 1 and 3
-    sum3_step<0x143, 0xC>(a, b, c);   // row_bcast:31 into rows 2 and 3: lane 63 holds the wavefront's sum
-}
-
+// Sum of one value per thread over the workgroup (kPairThreads threads).
 __device__ __forceinline__ double block_sum(double v, double* red) {
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
@@ -81,153 +56,18 @@ __device__ __forceinline__ double block_sum(double v, double* red) {
     return s;
 }
 
-// One round: workgroup (k, matrix) orthogonalises columns p, q of X and applies the rotation to the same columns of W.
-// X is [batch][c][r] (column j of a matrix = r contiguous values), W is [batch][c][cw_rows] or null.
-template <class T>
-__global__ __launch_bounds__(kPairThreads) void jacobi_round_kernel(T* __restrict__ x, T* __restrict__ w, int rows, int c, int ce, int round,
-                                                                    int wrows, int64_t bsx, int64_t bsw, double tol, int* rotations) {
-    __shared__ double red3[3][kPairThreads / 64];
-    int a, b;
-    pair_of(ce, round, blockIdx.x, &a, &b);
-    if (a >= c || b >= c) return;
-    const int p = a < b ? a : b, q = a < b ? b : a;
-    T* xp = x + (int64_t)blockIdx.y * bsx + (int64_t)p * rows;
-    T* xq = x + (int64_t)blockIdx.y * bsx + (int64_t)q * rows;
-    double sa = 0, sb = 0, sg = 0;
-    for (int i = threadIdx.x; i < rows; i += kPairThreads) {
-        const double u = (double)xp[i], v = (double)xq[i];
-        sa += u * u;
-        sb += v * v;
-        sg += u * v;
-    }
-    // the three sums share one pair of barriers
-    wave_sum3_to_lane63(sa, sb, sg);
-    if ((threadIdx.x & 63) == 63) {
-        red3[0][threadIdx.x >> 6] = sa;
-        red3[1][threadIdx.x >> 6] = sb;
-        red3[2][threadIdx.x >> 6] = sg;
-    }
-    __syncthreads();
-    double alpha = 0, beta = 0, gamma = 0;
-#pragma unroll
-    for (int i = 0; i < kPairThreads / 64; i++) {
-        alpha += red3[0][i];
-        beta += red3[1][i];
-        gamma += red3[2][i];
-    }
-    if (gamma == 0.0 || fabs(gamma) <= tol * sqrt(alpha * beta)) return;   // uniform: every thread holds the same sums
-    const double zeta = (beta - alpha) / (2.0 * gamma);
-    const double t = (zeta >= 0.0 ? 1.0 : -1.0) / (fabs(zeta) + sqrt(1.0 + zeta * zeta));
-    const double cs = 1.0 / sqrt(1.0 + t * t), sn = cs * t;
-    for (int i = threadIdx.x; i < rows; i += kPairThreads) {
-        const double u = (double)xp[i], v = (double)xq[i];
-        xp[i] = (T)(cs * u - sn * v);
-        xq[i] = (T)(sn * u + cs * v);
-    }
-    if (w) {
-        T* wp = w + (int64_t)blockIdx.y * bsw + (int64_t)p * wrows;
-        T* wq = w + (int64_t)blockIdx.y * bsw + (int64_t)q * wrows;
-        for (int i = threadIdx.x; i < wrows; i += kPairThreads) {
-            const double u = (double)wp[i], v = (double)wq[i];
-            wp[i] = (T)(cs * u - sn * v);
-            wq[i] = (T)(sn * u + cs * v);
-        }
-    }
-    if (threadIdx.x == 0) *rotations = 1;   // a flag, not a count: every writer stores the same value, no atomic queue at one address
-}
-
-// The same round for columns of at most NPT * 256 elements: a thread keeps its elements of both column pairs (X and W) in
-// registers, so every global load of the round is issued before the reduction and the rotation only computes and stores (the
-// two-pass form above waits for a second round trip after the barrier; a round is latency-bound, not bandwidth-bound).
-template <class T, int NPT>
-__global__ __launch_bounds__(kPairThreads) void jacobi_round_reg_kernel(T* __restrict__ x, T* __restrict__ w, int rows, int c, int ce, int round,
-                                                                        int wrows, int64_t bsx, int64_t bsw, double tol, int* rotations) {
-    __shared__ double red3[3][kPairThreads / 64];
-    int a, b;
-    pair_of(ce, round, blockIdx.x, &a, &b);
-    if (a >= c || b >= c) return;
-    const int p = a < b ? a : b, q = a < b ? b : a;
-    T* xp = x + (int64_t)blockIdx.y * bsx + (int64_t)p * rows;
-    T* xq = x + (int64_t)blockIdx.y * bsx + (int64_t)q * rows;
-    T* wp = w ? w + (int64_t)blockIdx.y * bsw + (int64_t)p * wrows : nullptr;
-    T* wq = w ? w + (int64_t)blockIdx.y * bsw + (int64_t)q * wrows : nullptr;
-    T u[NPT], v[NPT], wu[NPT], wv[NPT];
-#pragma unroll
-    for (int k = 0; k < NPT; k++) {
-        const int i = threadIdx.x + k * kPairThreads;
-        u[k] = i < rows ? xp[i] : T(0);
-        v[k] = i < rows ? xq[i] : T(0);
-    }
-    if (w) {
-#pragma unroll
-        for (int k = 0; k < NPT; k++) {
-            const int i = threadIdx.x + k * kPairThreads;
-            wu[k] = i < wrows ? wp[i] : T(0);
-            wv[k] = i < wrows ? wq[i] : T(0);
-        }
-    }
-    double sa = 0, sb = 0, sg = 0;
-#pragma unroll
-    for (int k = 0; k < NPT; k++) {
-        const double du = (double)u[k], dv = (double)v[k];
-        sa += du * du;
-        sb += dv * dv;
-        sg += du * dv;
-    }
-    wave_sum3_to_lane63(sa, sb, sg);
-    if ((threadIdx.x & 63) == 63) {
-        red3[0][threadIdx.x >> 6] = sa;
-        red3[1][threadIdx.x >> 6] = sb;
-        red3[2][threadIdx.x >> 6] = sg;
-    }
-    __syncthreads();
-    double alpha = 0, beta = 0, gamma = 0;
-#pragma unroll
-    for (int i = 0; i < kPairThreads / 64; i++) {
-        alpha += red3[0][i];
-        beta += red3[1][i];
-        gamma += red3[2][i];
-    }
-    if (gamma == 0.0 || fabs(gamma) <= tol * sqrt(alpha * beta)) return;
-    const double zeta = (beta - alpha) / (2.0 * gamma);
-    const double t = (zeta >= 0.0 ? 1.0 : -1.0) / (fabs(zeta) + sqrt(1.0 + zeta * zeta));
-    const double cs = 1.0 / sqrt(1.0 + t * t), sn = cs * t;
-#pragma unroll
-    for (int k = 0; k < NPT; k++) {
-        const int i = threadIdx.x + k * kPairThreads;
-        if (i < rows) {
-            const double du = (double)u[k], dv = (double)v[k];
-            xp[i] = (T)(cs * du - sn * dv);
-            xq[i] = (T)(sn * du + cs * dv);
-        }
-    }
-    if (w) {
-#pragma unroll
-        for (int k = 0; k < NPT; k++) {
-            const int i = threadIdx.x + k * kPairThreads;
-            if (i < wrows) {
-                const double du = (double)wu[k], dv = (double)wv[k];
-                wp[i] = (T)(cs * du - sn * dv);
-                wq[i] = (T)(sn * du + cs * dv);
-            }
-        }
-    }
-    if (threadIdx.x == 0) *rotations = 1;   // a flag, not a count: every writer stores the same value, no atomic queue at one address
-}
-
 // ---- block rounds ---------------------------------------------------------------------------------------------------------
-// The same sweep on blocks of 16 columns: a workgroup takes a pair of blocks (32 columns), forms their 32 x 32 Gram matrix
-// G = B^T B in double precision on the matrix cores, diagonalises G by cyclic two-sided Jacobi rotations in LDS while
-// accumulating the rotations in Q (G <- J^T G J, Q <- Q J), and replaces the columns by B Q (and the same columns of W by
-// W Q), again on the matrix cores.  The entries of G are the very sums alpha, beta, gamma of the column-pair form, so the
-// rotation test is the same; one round touches the matrices once for 16 x 16 + 2 * 120 column pairs instead of one, which
-// divides the memory traffic of a sweep by 16.  A sweep in which no workgroup finds an entry of its G above the threshold
-// ends the iteration, as before.  There are only C / 32 pairs, too few workgroups for the two passes over the rows, so a round
+// Blocks of 16 columns are paired by the round-robin schedule (blocks / 2 disjoint pairs per round, blocks - 1 rounds per sweep).
+// For a pair of blocks (32 columns B) the 32 x 32 Gram matrix G = B^T B is formed on the matrix cores, G is diagonalised by
+// cyclic two-sided Jacobi rotations in LDS while the rotations accumulate in Q (G <- J^T G J, Q <- Q J), and the columns are
+// replaced by B Q (the same columns of W by W Q), again on the matrix cores.  The entries of G are the sums
+// alpha = |x_p|^2, beta = |x_q|^2, gamma = x_p . x_q that define the rotation of columns p, q (a pair is rotated when
+// |gamma| > tol sqrt(alpha beta), tol = sqrt(rows) eps as in LAPACK's xGESVJ); one round moves the matrices once for
+// 16 x 16 + 2 * 120 column pairs.  A sweep in which no workgroup finds an entry of its G above the threshold ends the iteration.  There are only C / 32 pairs, too few workgroups for the two passes over the rows, so a round
 // is three launches: the partial Gram matrices of every (pair, piece of the rows); per pair the sum of the pieces and the
 // diagonalisation (Q to memory); Q applied to every (pair, piece of the rows of X and of W).
 typedef double f64x4 __attribute__((ext_vector_type(4)));
 constexpr int kBlockCols = 16;
-constexpr int kBlockMinCols = 64;   // below this the column-pair rounds are used
 
 // Four consecutive elements p[i .. i+3] of a column of `n` elements, raw: the caller converts (and zeroes what `ok4` excludes)
 // when it uses them, so that the loads of the next step stay in flight during the matrix instructions of the current one.
@@ -319,7 +159,7 @@ __global__ __launch_bounds__(kGramThreads) void jacobi_block_gram_kernel(const T
     int ba, bb;
     pair_of(nbe, round, blockIdx.x, &ba, &bb);
     const int nb = (c + kBlockCols - 1) / kBlockCols;
-    if (ba >= nb || bb >= nb) return;
+    if (ba >= nb && bb >= nb) return;   // a block paired with the bye still rotates its own columns (the other 16 read as zero)
     const int pcol = (ba < bb ? ba : bb) * kBlockCols, qcol = (ba < bb ? bb : ba) * kBlockCols;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lc = lane & 15, lk = lane >> 4;
@@ -387,7 +227,7 @@ __global__ __launch_bounds__(kGramThreads) void jacobi_block_gram_f32_kernel(con
     int ba, bb;
     pair_of(nbe, round, blockIdx.x, &ba, &bb);
     const int nb = (c + kBlockCols - 1) / kBlockCols;
-    if (ba >= nb || bb >= nb) return;
+    if (ba >= nb && bb >= nb) return;   // a block paired with the bye still rotates its own columns (the other 16 read as zero)
     const int pcol = (ba < bb ? ba : bb) * kBlockCols, qcol = (ba < bb ? bb : ba) * kBlockCols;
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int lm = lane & 31, lk = lane >> 5;
@@ -516,7 +356,7 @@ __global__ __launch_bounds__(kSolveThreads) void jacobi_block_solve_kernel(const
     int ba, bb;
     pair_of(nbe, round, blockIdx.x, &ba, &bb);
     const int nb = (c + kBlockCols - 1) / kBlockCols;
-    if (ba >= nb || bb >= nb) return;
+    if (ba >= nb && bb >= nb) return;   // a block paired with the bye still rotates its own columns (the other 16 read as zero)
     const int64_t pair_id = (int64_t)blockIdx.y * gridDim.x + blockIdx.x;
     const double* part = partial + pair_id * pieces * 768;
     if (threadIdx.x == 0) above = 0;
@@ -628,7 +468,7 @@ __global__ __launch_bounds__(kApplyThreads) void jacobi_block_apply_kernel(T* __
     int ba, bb;
     pair_of(nbe, round, blockIdx.x, &ba, &bb);
     const int nb = (c + kBlockCols - 1) / kBlockCols;
-    if (ba >= nb || bb >= nb) return;
+    if (ba >= nb && bb >= nb) return;   // a block paired with the bye still rotates its own columns (the other 16 read as zero)
     const int64_t pair_id = (int64_t)blockIdx.z * gridDim.x + blockIdx.x;
     if (!flag[pair_id]) return;
     const int pcol = (ba < bb ? ba : bb) * kBlockCols, qcol = (ba < bb ? bb : ba) * kBlockCols;
@@ -913,65 +753,54 @@ void prescale(T* x, int64_t batch, int64_t per_matrix, unsigned long long* maxbi
 template <class T>
 int32_t jacobi_run(T* x, T* w, int64_t batch, int rows, int c, int wrows, int* counter, hipStream_t stream, const char* what) {
     if (c < 2 || batch == 0 || rows == 0) return DNH_OK;
-    const int ce = c + (c & 1);
+    constexpr int64_t kMaxGridZ = 65535;
+    if (batch > kMaxGridZ) {
+        for (int64_t b0 = 0; b0 < batch; b0 += kMaxGridZ) {
+            const int64_t nbatch = std::min<int64_t>(kMaxGridZ, batch - b0);
+            DNH_TRY(jacobi_run<T>(x + b0 * c * rows, w ? w + b0 * c * wrows : nullptr, nbatch, rows, c, wrows, counter, stream, what));
+        }
+        return DNH_OK;
+    }
     const double tol = sqrt((double)rows) * (double)std::numeric_limits<T>::epsilon();   // as LAPACK's Jacobi SVD (xGESVJ)
-    // block rounds: three launches per round.  Rows are cut into pieces (multiples of 32 rows, at least 128) so that the Gram and
-    // the apply launches bring about four workgroups per CU.
-    const bool blocked = c >= kBlockMinCols && batch <= 65535;
+    // Three launches per round.  Rows are cut into pieces (multiples of 32 rows, at least 128) so that the Gram and the apply
+    // launches bring about four workgroups per CU.
     const int nb = (c + kBlockCols - 1) / kBlockCols, nbe = nb + (nb & 1), pairs = nbe / 2;
     int xpieces = 1, chunk = rows, wpieces = 0, wchunk = 32;
-    double *partial = nullptr, *qbuf = nullptr;
-    int* flag = nullptr;
-    void* block_ws = nullptr;
-    if (blocked) {
-        const int64_t want = std::max<int64_t>(1, (int64_t)4 * device_cus() / ((int64_t)pairs * batch));
-        xpieces = (int)std::max<int64_t>(1, std::min<int64_t>(want, rows / 128));
-        chunk = (int)cdiv(cdiv(rows, xpieces), 32) * 32;
-        xpieces = (int)cdiv(rows, chunk);
-        if (w && wrows > 0) {
-            wpieces = (int)std::max<int64_t>(1, std::min<int64_t>(want, wrows / 128));
-            wchunk = (int)cdiv(cdiv(wrows, wpieces), 32) * 32;
-            wpieces = (int)cdiv(wrows, wchunk);
-        }
-        const size_t sz_part = align_up(sizeof(double) * 768 * (size_t)xpieces * pairs * batch);
-        const size_t sz_q = align_up(sizeof(double) * 1024 * (size_t)pairs * batch);
-        DNH_TRY(dnh_alloc_async(sz_part + sz_q + sizeof(int) * (size_t)pairs * batch, stream, &block_ws));
-        partial = (double*)block_ws;
-        qbuf = (double*)((char*)block_ws + sz_part);
-        flag = (int*)((char*)block_ws + sz_part + sz_q);
+    const int64_t want = std::max<int64_t>(1, (int64_t)4 * device_cus() / ((int64_t)pairs * batch));
+    xpieces = (int)std::max<int64_t>(1, std::min<int64_t>(want, rows / 128));
+    chunk = (int)cdiv(cdiv(rows, xpieces), 32) * 32;
+    xpieces = (int)cdiv(rows, chunk);
+    if (w && wrows > 0) {
+        wpieces = (int)std::max<int64_t>(1, std::min<int64_t>(want, wrows / 128));
+        wchunk = (int)cdiv(cdiv(wrows, wpieces), 32) * 32;
+        wpieces = (int)cdiv(wrows, wchunk);
     }
+    const size_t sz_part = align_up(sizeof(double) * 768 * (size_t)xpieces * pairs * batch);
+    const size_t sz_q = align_up(sizeof(double) * 1024 * (size_t)pairs * batch);
+    void* block_ws = nullptr;
+    DNH_TRY(dnh_alloc_async(sz_part + sz_q + sizeof(int) * (size_t)pairs * batch, stream, &block_ws));
+    double* partial = (double*)block_ws;
+    double* qbuf = (double*)((char*)block_ws + sz_part);
+    int* flag = (int*)((char*)block_ws + sz_part + sz_q);
     struct Release {
         void* p;
         hipStream_t s;
-        ~Release() { if (p) (void)dnh_free_async(p, s); }
+        ~Release() { (void)dnh_free_async(p, s); }
     } release{block_ws, stream};
     for (int sweep = 0; sweep < kMaxSweeps; sweep++) {
         hipLaunchKernelGGL(clear_int_kernel, dim3(1), dim3(1), 0, stream, counter);
-        const int longest = rows > wrows ? rows : wrows;
-        const dim3 grid((unsigned)(ce / 2), (unsigned)batch);
-#define DNH_ROUND(KERNEL) hipLaunchKernelGGL((KERNEL), grid, dim3(kPairThreads), 0, stream, x, w, rows, c, ce, r, wrows, (int64_t)c * rows, (int64_t)c * wrows, tol, counter)
-        if (blocked) {
-            for (int r = 0; r < nbe - 1; r++) {
-                if constexpr (sizeof(T) == 4)
-                    hipLaunchKernelGGL(jacobi_block_gram_f32_kernel, dim3((unsigned)pairs, (unsigned)xpieces, (unsigned)batch), dim3(kGramThreads), 0, stream, x,
-                                       partial, rows, chunk, c, nbe, r, (int64_t)c * rows);
-                else
-                    hipLaunchKernelGGL((jacobi_block_gram_kernel<T>), dim3((unsigned)pairs, (unsigned)xpieces, (unsigned)batch), dim3(kGramThreads), 0, stream, x,
-                                       partial, rows, chunk, c, nbe, r, (int64_t)c * rows);
-                hipLaunchKernelGGL((jacobi_block_solve_kernel<T>), dim3((unsigned)pairs, (unsigned)batch), dim3(kSolveThreads), 0, stream, partial, xpieces, qbuf,
-                                   flag, c, nbe, r, (r == sweep % (nbe - 1)) ? 1 : 0, tol, counter);
-                hipLaunchKernelGGL((jacobi_block_apply_kernel<T>), dim3((unsigned)pairs, (unsigned)(xpieces + wpieces), (unsigned)batch), dim3(kApplyThreads), 0,
-                                   stream, x, w, qbuf, flag, rows, chunk, xpieces, wrows, wchunk, c, nbe, r, (int64_t)c * rows, (int64_t)c * wrows);
-            }
-        } else
-        for (int r = 0; r < ce - 1; r++) {
-            if (longest <= 1 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 1>));
-            else if (longest <= 4 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 4>));
-            else if (longest <= 8 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 8>));
-            else if (sizeof(T) == 8 && longest <= 16 * kPairThreads) DNH_ROUND((jacobi_round_reg_kernel<T, 16>));   // single precision: the two-pass form measured faster at 4000 rows
-            else DNH_ROUND((jacobi_round_kernel<T>));
+        for (int r = 0; r < nbe - 1; r++) {
+            if constexpr (sizeof(T) == 4)
+                hipLaunchKernelGGL(jacobi_block_gram_f32_kernel, dim3((unsigned)pairs, (unsigned)xpieces, (unsigned)batch), dim3(kGramThreads), 0, stream, x, partial,
+                                   rows, chunk, c, nbe, r, (int64_t)c * rows);
+            else
+                hipLaunchKernelGGL((jacobi_block_gram_kernel<T>), dim3((unsigned)pairs, (unsigned)xpieces, (unsigned)batch), dim3(kGramThreads), 0, stream, x, partial,
+                                   rows, chunk, c, nbe, r, (int64_t)c * rows);
+            hipLaunchKernelGGL((jacobi_block_solve_kernel<T>), dim3((unsigned)pairs, (unsigned)batch), dim3(kSolveThreads), 0, stream, partial, xpieces, qbuf, flag, c,
+                               nbe, r, (r == sweep % (nbe - 1)) ? 1 : 0, tol, counter);
+            hipLaunchKernelGGL((jacobi_block_apply_kernel<T>), dim3((unsigned)pairs, (unsigned)(xpieces + wpieces), (unsigned)batch), dim3(kApplyThreads), 0, stream, x,
+                               w, qbuf, flag, rows, chunk, xpieces, wrows, wchunk, c, nbe, r, (int64_t)c * rows, (int64_t)c * wrows);
         }
-#undef DNH_ROUND
         DNH_LAUNCH_CHECK();
         int rotated = 0;
         DNH_HIP(hipMemcpyAsync(&rotated, counter, sizeof(int), hipMemcpyDeviceToHost, stream));
