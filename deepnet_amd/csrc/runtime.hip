@@ -6,6 +6,9 @@
 #include <atomic>
 #include <map>
 #include <mutex>
+#include <thread>
+#include <vector>
+#include <cstring>
 #include <unordered_map>
 
 namespace dnh {
@@ -15,6 +18,8 @@ std::mutex g_mu;
 std::atomic<uint64_t> g_epoch{1};   // bumped when the device is chosen
 bool g_init = false;
 int g_device = 0;
+std::mutex g_pinned_mu;
+std::map<uintptr_t, size_t> g_pinned;   // blocks handed out by dnh_host_alloc
 int g_cus = 256;
 std::map<hipStream_t, int32_t*> g_error_flags;   // one index-error word per stream, so concurrent streams do not see each other's errors
 
@@ -311,12 +316,20 @@ int32_t dnh_host_alloc(size_t bytes, void** out) {
     DNH_TRY(ensure_init());
     *out = nullptr;
     DNH_HIP(hipHostMalloc(out, bytes ? bytes : 1, hipHostMallocDefault));
+    {
+        std::lock_guard<std::mutex> lock(g_pinned_mu);
+        g_pinned[(uintptr_t)*out] = bytes ? bytes : 1;
+    }
     return DNH_OK;
 }
 
 int32_t dnh_host_free(void* ptr) {
     if (!ptr) return DNH_OK;
     DNH_TRY(ensure_init());
+    {
+        std::lock_guard<std::mutex> lock(g_pinned_mu);
+        g_pinned.erase((uintptr_t)ptr);
+    }
     DNH_HIP(hipHostFree(ptr));
     return DNH_OK;
 }
@@ -328,10 +341,106 @@ int32_t dnh_memset(void* dst, int32_t byte_value, size_t bytes, void* stream) {
     return DNH_OK;
 }
 
+// ---- large copies between pageable host memory and the device ------------------------------------------------------------------
+// The reference registers host arrays with the driver to copy at the full link rate (Tensor/Tensor/Cuda/CudaRegMem.fs); memory
+// that already exists cannot be registered here, and a plain copy from pageable memory runs at a third to a half of the pinned
+// rate.  Synchronous copies of 16 MiB and more are therefore staged by the library: a few host threads, each with two pinned
+// 4 MiB chunks and a stream of its own, move their share of the chunks (host copy of one chunk while the other is on the link).
+namespace {
+constexpr size_t kStageChunk = (size_t)4 << 20;
+constexpr size_t kStageMin = (size_t)16 << 20;
+constexpr int kStageThreads = 6;
+
+struct Stager {
+    std::mutex mu;   // one staged copy at a time
+    bool ready = false;
+    void* pinned[kStageThreads][2] = {};
+    hipStream_t stream[kStageThreads] = {};
+    hipEvent_t done[kStageThreads][2] = {};
+};
+Stager g_stager;
+
+bool is_pinned(const void* p, size_t bytes) {
+    std::lock_guard<std::mutex> lock(g_pinned_mu);
+    auto it = g_pinned.upper_bound((uintptr_t)p);
+    if (it == g_pinned.begin()) return false;
+    --it;
+    return (uintptr_t)p + bytes <= it->first + it->second;
+}
+
+int32_t stager_init_locked() {
+    if (g_stager.ready) return DNH_OK;
+    for (int t = 0; t < kStageThreads; t++) {
+        DNH_HIP(hipStreamCreateWithFlags(&g_stager.stream[t], hipStreamNonBlocking));
+        for (int k = 0; k < 2; k++) {
+            DNH_HIP(hipHostMalloc(&g_stager.pinned[t][k], kStageChunk, hipHostMallocDefault));
+            DNH_HIP(hipEventCreateWithFlags(&g_stager.done[t][k], hipEventDisableTiming));
+        }
+    }
+    g_stager.ready = true;
+    return DNH_OK;
+}
+
+// Worker t moves chunks t, t + kStageThreads, ...; returns the first HIP error it met.
+hipError_t stage_worker(int t, bool to_device, char* dev, char* host, size_t bytes) {
+    hipError_t e = hipSetDevice(g_device);
+    if (e != hipSuccess) return e;
+    const size_t chunks = (bytes + kStageChunk - 1) / kStageChunk;
+    hipStream_t s = g_stager.stream[t];
+    int slot = 0;
+    size_t prev_off = 0, prev_len = 0;
+    int prev_slot = -1;
+    for (size_t i = (size_t)t; i < chunks; i += kStageThreads, slot ^= 1) {
+        const size_t off = i * kStageChunk, len = bytes - off < kStageChunk ? bytes - off : kStageChunk;
+        void* pin = g_stager.pinned[t][slot];
+        if (to_device) {
+            if ((e = hipEventSynchronize(g_stager.done[t][slot])) != hipSuccess) return e;   // the chunk's previous transfer has left it
+            memcpy(pin, host + off, len);
+            if ((e = hipMemcpyAsync(dev + off, pin, len, hipMemcpyHostToDevice, s)) != hipSuccess) return e;
+            if ((e = hipEventRecord(g_stager.done[t][slot], s)) != hipSuccess) return e;
+        } else {
+            if ((e = hipMemcpyAsync(pin, dev + off, len, hipMemcpyDeviceToHost, s)) != hipSuccess) return e;
+            if ((e = hipEventRecord(g_stager.done[t][slot], s)) != hipSuccess) return e;
+            if (prev_slot >= 0) {
+                if ((e = hipEventSynchronize(g_stager.done[t][prev_slot])) != hipSuccess) return e;
+                memcpy(host + prev_off, g_stager.pinned[t][prev_slot], prev_len);
+            }
+            prev_off = off;
+            prev_len = len;
+            prev_slot = slot;
+        }
+    }
+    if (!to_device && prev_slot >= 0) {
+        if ((e = hipEventSynchronize(g_stager.done[t][prev_slot])) != hipSuccess) return e;
+        memcpy(host + prev_off, g_stager.pinned[t][prev_slot], prev_len);
+    }
+    return hipStreamSynchronize(s);
+}
+
+int32_t staged_copy(bool to_device, void* dev, void* host, size_t bytes, hipStream_t stream) {
+    std::lock_guard<std::mutex> lock(g_stager.mu);
+    DNH_TRY(stager_init_locked());
+    DNH_HIP(hipStreamSynchronize(stream));   // everything queued before the copy has finished with the device buffer
+    hipError_t errs[kStageThreads];
+    std::vector<std::thread> workers;
+    for (int t = 1; t < kStageThreads; t++)
+        workers.emplace_back([&, t] { errs[t] = stage_worker(t, to_device, (char*)dev, (char*)host, bytes); });
+    errs[0] = stage_worker(0, to_device, (char*)dev, (char*)host, bytes);
+    for (auto& w : workers) w.join();
+    for (int t = 0; t < kStageThreads; t++) DNH_HIP(errs[t]);
+    return DNH_OK;
+}
+}  // namespace
+
 static int32_t copy_impl(void* dst, const void* src, size_t bytes, void* stream, int32_t sync, hipMemcpyKind kind) {
     DNH_TRY(ensure_init());
     if (bytes == 0) return DNH_OK;
     if (!dst || !src) return fail(DNH_ERR_INVALID_ARG, "memcpy: null pointer");
+    if (sync && bytes >= kStageMin && kind != hipMemcpyDeviceToDevice) {
+        const bool to_device = kind == hipMemcpyHostToDevice;
+        void* host = to_device ? const_cast<void*>(src) : dst;
+        if (!is_pinned(host, bytes)) return staged_copy(to_device, to_device ? dst : const_cast<void*>(src), host, bytes, (hipStream_t)stream);
+    }
     DNH_HIP(hipMemcpyAsync(dst, src, bytes, kind, (hipStream_t)stream));
     if (sync) DNH_HIP(hipStreamSynchronize((hipStream_t)stream));
     return DNH_OK;

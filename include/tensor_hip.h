@@ -166,6 +166,8 @@ int32_t dnh_pool_stats(DnhPoolStats* stats);
 int32_t dnh_host_alloc(size_t bytes, void** out);     /* pinned host memory for transfers                      */
 int32_t dnh_host_free(void* ptr);
 int32_t dnh_memset(void* dst, int32_t byte_value, size_t bytes, void* stream);
+/* sync != 0: the call returns when the bytes have arrived.  Synchronous copies of 16 MiB and more between the device and host
+ * memory that did not come from dnh_host_alloc are staged through pinned chunks on several host threads (callers take turns). */
 int32_t dnh_memcpy_h2d(void* dst, const void* src, size_t bytes, void* stream, int32_t sync);
 int32_t dnh_memcpy_d2h(void* dst, const void* src, size_t bytes, void* stream, int32_t sync);
 int32_t dnh_memcpy_d2d(void* dst, const void* src, size_t bytes, void* stream, int32_t sync);
