@@ -166,3 +166,13 @@ def test_extreme_magnitudes(H, G, rng, dt, scale, n):
     (wr, vr2), (w, v2) = both(H, G, lambda x: type(x).symmetricEigenDecomposition("Upper", x), sym)
     assert np.all(np.isfinite(w)) and np.abs(w).max() > 0
     check_eig(sym, w, v2, wr)
+
+
+def test_svd_more_matrices_than_one_launch_takes(H, G, rng):
+    """70000 matrices: the sweeps run on slices of at most 65535 matrices."""
+    a = rng.standard_normal((70000, 3, 2)).astype(np.float32)
+    u, s, v = (G.toNumpy(t) for t in type(G.ofNumpy(a)).SVD(G.ofNumpy(a)))
+    ref = np.linalg.svd(a.astype(np.float64), compute_uv=False)
+    assert np.abs(s - ref).max() <= 1e-5 * ref.max()
+    recon = (u[..., :, :2] * s[..., None, :]) @ np.swapaxes(v, -1, -2)
+    assert np.abs(recon - a).max() <= 1e-5 * ref.max()
