@@ -1,6 +1,8 @@
 """Differential test over seeded random shapes and views: the same frontend call sequence on the oracle device and on the GPU,
 integer element types so every comparison is bit-exact.  Views are built from permutations, slices, reversed axes, inserted and
 broadcast axes; extents include 1 and ragged sizes around the vector widths and tile edges of the kernels."""
+import os
+
 import numpy as np
 import pytest
 
@@ -8,6 +10,8 @@ from deepnet_amd.tensor import Tensor
 from util import assert_exact
 
 pytestmark = pytest.mark.gpu
+
+MORE = int(os.environ.get("DNH_FUZZ_SEEDS_FACTOR", "1"))   # more seeds for an occasional longer run
 
 EXTENTS = [1, 2, 3, 4, 5, 7, 8, 15, 16, 17, 31, 33, 63, 64, 65, 127, 130, 257]
 
@@ -48,7 +52,7 @@ def make_operands(rng, H, G, dtype, max_elems=200_000):
     return a
 
 
-@pytest.mark.parametrize("seed", range(40))
+@pytest.mark.parametrize("seed", range(40 * MORE))
 def test_random_views_elementwise_and_folds(H, G, seed):
     rng = np.random.default_rng(1000 + seed)
     for case in range(25):
@@ -97,7 +101,7 @@ def test_random_views_elementwise_and_folds(H, G, seed):
                 raise AssertionError(f"seed {seed} case {case} result {k} dtype {np.dtype(dtype)} shape {a_np.shape}: {e}") from None
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(12 * MORE))
 def test_random_gather_scatter(H, G, seed):
     rng = np.random.default_rng(2000 + seed)
     for case in range(15):
@@ -126,7 +130,7 @@ def test_random_gather_scatter(H, G, seed):
             assert_exact(ref, got)
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(16 * MORE))
 def test_random_views_float(H, G, seed):
     """fp32 / fp64: exactly rounded operations, comparisons, max/min and arg folds are bit-exact; sums within (n + 64) u S."""
     rng = np.random.default_rng(3000 + seed)
