@@ -429,6 +429,169 @@ __global__ __launch_bounds__(64 * SG) void gemm_split_finish_kernel(T* __restric
     }
 }
 
+// ---- single precision on the bf16 matrix instructions ----------------------------------------------------------------------
+// v_mfma_f32_32x32x16_bf16 runs 16 times the rate of v_mfma_f32_32x32x2_f32.  A float is the exact sum of three bf16 numbers
+// (its 24 significant bits cut into 8 + 8 + 8 by truncation: hi = the upper 16 bits of a, mid = those of a - hi, lo = those of
+// a - hi - mid, every difference exact), so a.b = sum of nine bf16 products, each exact in the instruction's fp32 accumulator.
+// The six largest are kept: hi.hi, hi.mid, mid.hi, hi.lo, lo.hi, mid.mid; the three dropped (mid.lo, lo.mid, lo.lo) are below
+// 2^-21 |a||b|, usually 2^-25, i.e. a few units of the rounding of one fp32 product, against a contract of K of them.  Six bf16
+// instructions of K = 16 replace eight fp32 instructions of K = 2 per 32 x 32 x 16 block: 2.7 times fewer matrix-pipe cycles.
+// Two deviations from fp32 arithmetic, both outside finite normal inputs: an infinite element gives NaN in its row / column of
+// the product (inf - inf in its mid part; IEEE gives +-inf unless it meets a zero), and elements below 2^-126 (denormal) lose
+// precision, since their parts are bf16 denormals.  NaN stays NaN.  DNH_DOT_BF16X3=0 in the environment keeps every product on
+// the fp32 instructions.
+// Row-major, 16-byte aligned operands with K a multiple of 16 and no K split; everything else takes gemm_kernel.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+constexpr int kX3BK = 16;
+constexpr int kX3Row = 24;   // bf16 per LDS row: 16 of data + 8 of padding (48 bytes: 16-byte reads of 16 consecutive rows hit all banks once)
+
+// Splits eight floats into their hi / mid / lo bf16 parts, packed as 8 x bf16 = 16 bytes each.
+__device__ __forceinline__ void split3_bf16(const float (&v)[8], u32x4& hi, u32x4& mid, u32x4& lo) {
+    uint32_t h[8], m[8], l[8];   // the part sits in the upper 16 bits of each word
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        h[e] = __float_as_uint(v[e]);
+        const float r1 = v[e] - __uint_as_float(h[e] & 0xFFFF0000u);
+        m[e] = __float_as_uint(r1);
+        const float r2 = r1 - __uint_as_float(m[e] & 0xFFFF0000u);
+        l[e] = __float_as_uint(r2);
+    }
+    // one byte permute packs the upper halves of two words: result = {x1[31:16], x0[31:16]}
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        hi[e] = __builtin_amdgcn_perm(h[2 * e + 1], h[2 * e], 0x07060302u);
+        mid[e] = __builtin_amdgcn_perm(m[2 * e + 1], m[2 * e], 0x07060302u);
+        lo[e] = __builtin_amdgcn_perm(l[2 * e + 1], l[2 * e], 0x07060302u);
+    }
+}
+
+__global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restrict__ c, const float* __restrict__ a, const float* __restrict__ b, GemmArgs g) {
+    __shared__ __align__(16) __bf16 As[2][3][BM][kX3Row];
+    __shared__ __align__(16) __bf16 Bs[2][3][BN][kX3Row];
+
+    uint32_t bid = blockIdx.x;
+    if (g.xcd_chunk) bid = (bid % 8u) * g.xcd_chunk + bid / 8u;
+    const uint32_t tn = bid % g.tiles_n;
+    bid /= g.tiles_n;
+    const uint32_t tm = bid % g.tiles_m;
+    bid /= g.tiles_m;
+    int64_t oa = 0, ob = 0, oc = 0;
+    for (int d = g.nbatch - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
+        const uint32_t i = bid - q * g.bshape[d];
+        bid = q;
+        oa += (int64_t)i * g.bsa[d];
+        ob += (int64_t)i * g.bsb[d];
+        oc += (int64_t)i * g.bsc[d];
+    }
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    a += oa;
+    b += ob;
+    c += oc;
+    const int tid = threadIdx.x;
+
+    // staging: A rows are k-contiguous (two 16-byte loads = 8 floats of one row); B rows are n-contiguous, and the instruction
+    // wants 8 consecutive k of one column, so a thread takes one column and 8 rows (lanes = consecutive columns: 256-byte rows)
+    const int a_row = tid >> 1, a_kh = tid & 1;
+    const int b_col = tid & 127, b_kh = tid >> 7;
+    const bool a_ok = m0 + a_row < g.M, b_ok = n0 + b_col < g.N;
+    const float* ap = a + (a_ok ? (m0 + a_row) * g.sam : 0) + a_kh * 8;
+    const float* bp = b + (int64_t)(b_kh * 8) * g.sbk + (b_ok ? n0 + b_col : 0);
+    float ra[8], rb[8];
+    auto load_tiles = [&](int64_t k0) {
+        const Pack<float, 4> v0 = load_pack<float, 4>(ap + k0), v1 = load_pack<float, 4>(ap + k0 + 4);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            ra[e] = v0.v[e];
+            ra[4 + e] = v1.v[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) rb[e] = bp[(k0 + e) * g.sbk];
+    };
+    auto store_tiles = [&](int buf) {
+        u32x4 hi, mid, lo;
+        if (!a_ok) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) ra[e] = 0.0f;
+        }
+        split3_bf16(ra, hi, mid, lo);
+        *reinterpret_cast<u32x4*>(&As[buf][0][a_row][a_kh * 8]) = hi;
+        *reinterpret_cast<u32x4*>(&As[buf][1][a_row][a_kh * 8]) = mid;
+        *reinterpret_cast<u32x4*>(&As[buf][2][a_row][a_kh * 8]) = lo;
+        if (!b_ok) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) rb[e] = 0.0f;
+        }
+        split3_bf16(rb, hi, mid, lo);
+        *reinterpret_cast<u32x4*>(&Bs[buf][0][b_col][b_kh * 8]) = hi;
+        *reinterpret_cast<u32x4*>(&Bs[buf][1][b_col][b_kh * 8]) = mid;
+        *reinterpret_cast<u32x4*>(&Bs[buf][2][b_col][b_kh * 8]) = lo;
+    };
+
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int lm = lane & 31, lk = lane >> 5;
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    load_tiles(0);
+    store_tiles(0);
+    __syncthreads();
+    int cur = 0;
+    for (int64_t k0 = 0; k0 < g.K; k0 += kX3BK) {
+        const bool more = k0 + kX3BK < g.K;
+        if (more) load_tiles(k0 + kX3BK);
+        bf16x8 av[2][3], bv[2][3];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int s = 0; s < 3; s++) {
+                av[i][s] = *reinterpret_cast<const bf16x8*>(&As[cur][s][wm + i * 32 + lm][lk * 8]);
+                bv[i][s] = *reinterpret_cast<const bf16x8*>(&Bs[cur][s][wn + i * 32 + lm][lk * 8]);
+            }
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                // smallest products first
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][1], bv[j][1], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][0], bv[j][2], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][2], bv[j][0], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][0], bv[j][1], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][1], bv[j][0], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][0], bv[j][0], acc[i][j], 0, 0, 0);
+            }
+        if (more) {
+            store_tiles(cur ^ 1);
+            __syncthreads();
+            cur ^= 1;
+        }
+    }
+    // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile
+    const bool full_mn = m0 + BM <= g.M && n0 + BN <= g.N;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
+                const int64_t n = n0 + wn + j * 32 + lm;
+                if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
+            }
+}
+
+bool use_bf16x3() {
+    static const bool on = [] { const char* e = getenv("DNH_DOT_BF16X3"); return !e || e[0] != '0'; }();
+    return on;
+}
+
 template <class T>
 int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hipStream_t stream) {
     int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
@@ -476,7 +639,12 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
     } else if (g.accumulate) {
         if (fast) DNH_GEMM(true, true, false); else DNH_GEMM(false, true, false);
     } else {
-        if (fast) DNH_GEMM(true, false, false); else DNH_GEMM(false, false, false);
+        bool x3 = false;
+        if constexpr (sizeof(T) == 4) x3 = fast && (g.K % kX3BK) == 0 && use_bf16x3();
+        if (x3) {
+            if constexpr (sizeof(T) == 4) hipLaunchKernelGGL(gemm_bf16x3_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+        } else if (fast) DNH_GEMM(true, false, false);
+        else DNH_GEMM(false, false, false);
     }
 #undef DNH_GEMM
     DNH_LAUNCH_CHECK();
