@@ -440,7 +440,7 @@ __global__ __launch_bounds__(64 * SG) void gemm_split_finish_kernel(T* __restric
 // the product (inf - inf in its mid part; IEEE gives +-inf unless it meets a zero), and elements below 2^-126 (denormal) lose
 // precision, since their parts are bf16 denormals.  NaN stays NaN.  DNH_DOT_BF16X3=0 in the environment keeps every product on
 // the fp32 instructions.
-// Row-major, 16-byte aligned operands with K a multiple of 16 and no K split; everything else takes gemm_kernel.
+// Row-major, 16-byte aligned operands (K splits included); accumulating and strided products take gemm_kernel.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kX3BK = 16;
@@ -466,6 +466,7 @@ __device__ __forceinline__ void split3_bf16(const float (&v)[8], u32x4& hi, u32x
     }
 }
 
+template <bool SPLIT, bool TAIL>
 __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restrict__ c, const float* __restrict__ a, const float* __restrict__ b, GemmArgs g) {
     __shared__ __align__(16) __bf16 As[2][3][BM][kX3Row];
     __shared__ __align__(16) __bf16 Bs[2][3][BN][kX3Row];
@@ -477,6 +478,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
     const uint32_t tm = bid % g.tiles_m;
     bid /= g.tiles_m;
     int64_t oa = 0, ob = 0, oc = 0;
+    uint32_t chunk_id = 0;
     for (int d = g.nbatch - 1; d >= 0; d--) {
         const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
         const uint32_t i = bid - q * g.bshape[d];
@@ -484,7 +486,10 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
         oa += (int64_t)i * g.bsa[d];
         ob += (int64_t)i * g.bsb[d];
         oc += (int64_t)i * g.bsc[d];
+        if (SPLIT && d == g.nbatch - 1) chunk_id = i;
     }
+    // this block's extent along k: the whole of K, or one chunk of it (SPLIT: the innermost batch dimension counts the chunks)
+    const int64_t K = SPLIT ? min(g.kchunk, g.K - (int64_t)chunk_id * g.kchunk) : g.K;
     const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
     a += oa;
     b += ob;
@@ -496,18 +501,31 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
     const int a_row = tid >> 1, a_kh = tid & 1;
     const int b_col = tid & 127, b_kh = tid >> 7;
     const bool a_ok = m0 + a_row < g.M, b_ok = n0 + b_col < g.N;
-    const float* ap = a + (a_ok ? (m0 + a_row) * g.sam : 0) + a_kh * 8;
-    const float* bp = b + (int64_t)(b_kh * 8) * g.sbk + (b_ok ? n0 + b_col : 0);
+    const float* arow = a + (a_ok ? (m0 + a_row) * g.sam : 0);
+    const float* bcol = b + (b_ok ? n0 + b_col : 0);
+    const float* ap = arow + a_kh * 8;
+    const float* bp = bcol + (int64_t)(b_kh * 8) * g.sbk;
     float ra[8], rb[8];
     auto load_tiles = [&](int64_t k0) {
-        const Pack<float, 4> v0 = load_pack<float, 4>(ap + k0), v1 = load_pack<float, 4>(ap + k0 + 4);
+        if (!TAIL || k0 + kX3BK <= K) {
+            const Pack<float, 4> v0 = load_pack<float, 4>(ap + k0), v1 = load_pack<float, 4>(ap + k0 + 4);
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            ra[e] = v0.v[e];
-            ra[4 + e] = v1.v[e];
+            for (int e = 0; e < 4; e++) {
+                ra[e] = v0.v[e];
+                ra[4 + e] = v1.v[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e++) rb[e] = bp[(k0 + e) * g.sbk];
+        } else {
+            // TAIL (K is not a multiple of 16): the last, partial K step takes element loads from addresses clamped into the row / column, zeros beyond K
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int64_t ka = k0 + a_kh * 8 + e, kb = k0 + b_kh * 8 + e;
+                const float va = arow[ka < K ? ka : K - 1], vb = bcol[(kb < K ? kb : K - 1) * g.sbk];
+                ra[e] = ka < K ? va : 0.0f;
+                rb[e] = kb < K ? vb : 0.0f;
+            }
         }
-#pragma unroll
-        for (int e = 0; e < 8; e++) rb[e] = bp[(k0 + e) * g.sbk];
     };
     auto store_tiles = [&](int buf) {
         u32x4 hi, mid, lo;
@@ -544,8 +562,8 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
     store_tiles(0);
     __syncthreads();
     int cur = 0;
-    for (int64_t k0 = 0; k0 < g.K; k0 += kX3BK) {
-        const bool more = k0 + kX3BK < g.K;
+    for (int64_t k0 = 0; k0 < K; k0 += kX3BK) {
+        const bool more = k0 + kX3BK < K;
         if (more) load_tiles(k0 + kX3BK);
         bf16x8 av[2][3], bv[2][3];
 #pragma unroll
@@ -634,15 +652,24 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
     }
     g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
 #define DNH_GEMM(FASTF, ACCF, SPLITF) hipLaunchKernelGGL((gemm_kernel<T, FASTF, ACCF, SPLITF>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g)
+    bool x3 = false;
+    if constexpr (sizeof(T) == 4) x3 = fast && !g.accumulate && use_bf16x3();
     if (splits > 1) {
-        if (fast) DNH_GEMM(true, false, true); else DNH_GEMM(false, false, true);
+        if (x3) {
+            if constexpr (sizeof(T) == 4) {
+                if (g.K % kX3BK) hipLaunchKernelGGL((gemm_bf16x3_kernel<true, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+                else hipLaunchKernelGGL((gemm_bf16x3_kernel<true, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+            }
+        } else if (fast) DNH_GEMM(true, false, true);
+        else DNH_GEMM(false, false, true);
     } else if (g.accumulate) {
         if (fast) DNH_GEMM(true, true, false); else DNH_GEMM(false, true, false);
     } else {
-        bool x3 = false;
-        if constexpr (sizeof(T) == 4) x3 = fast && (g.K % kX3BK) == 0 && use_bf16x3();
         if (x3) {
-            if constexpr (sizeof(T) == 4) hipLaunchKernelGGL(gemm_bf16x3_kernel, dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+            if constexpr (sizeof(T) == 4) {
+                if (g.K % kX3BK) hipLaunchKernelGGL((gemm_bf16x3_kernel<false, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+                else hipLaunchKernelGGL((gemm_bf16x3_kernel<false, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
+            }
         } else if (fast) DNH_GEMM(true, false, false);
         else DNH_GEMM(false, false, false);
     }
