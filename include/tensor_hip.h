@@ -238,7 +238,8 @@ int32_t dnh_true_indices(const DnhTensor* t_i64, const DnhTensor* src_bool, void
  * Dot: ITensorBackend VecVecDot / MatVecDot / MatMatDot / BatchedMatMatDot (TensorBackend.fs:137-140;
  * Host/HostBackend.fs:463-546).  The ranks of (t, a, b) select the variant exactly as Tensor.FillDot does
  * (Tensor.fs:2714-2730): (0,1,1) (1,2,1) (2,2,2) or (n,n,n) with n>2.  fp32 and fp64 on the
- * matrix cores; the integer types wrap like the host backend's multiply + sumAxis (HostBackend.fs:544-546); bool: status 2.
+ * matrix cores (row-major single-precision operands: bf16 instructions on floats cut into three bf16 parts, same error bound;
+ * an infinite element then gives NaN, DNH_DOT_BF16X3=0 in the environment selects the fp32 instructions); the integer types wrap like the host backend's multiply + sumAxis (HostBackend.fs:544-546); bool: status 2.
  * ------------------------------------------------------------------------------------------------- */
 int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream);
 
