@@ -35,6 +35,7 @@ struct GemmArgs {
     uint32_t xcd_chunk;                           // total tiles / 8 when divisible, else 0 (identity order)
     uint32_t accumulate;                          // 1: c += a.b (used by the blocked matrix inversion), 0: c = a.b
     int64_t kchunk;                               // > 0: the innermost batch dimension walks K in chunks of this many (split K)
+    uint32_t xcd_2d;                              // 1: one matrix whose tiles are dealt to the 8 XCDs as a 2 x 4 grid of regions
 };
 
 template <class T, bool FAST, bool ACC, bool SPLIT>
@@ -471,12 +472,22 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
     __shared__ __align__(16) __bf16 As[2][3][BM][kX3Row];
     __shared__ __align__(16) __bf16 Bs[2][3][BN][kX3Row];
 
-    uint32_t bid = blockIdx.x;
-    if (g.xcd_chunk) bid = (bid % 8u) * g.xcd_chunk + bid / 8u;
-    const uint32_t tn = bid % g.tiles_n;
-    bid /= g.tiles_n;
-    const uint32_t tm = bid % g.tiles_m;
-    bid /= g.tiles_m;
+    uint32_t bid = blockIdx.x, tm, tn;
+    if (g.xcd_2d) {
+        // one matrix: XCD x (workgroup ids are dealt round-robin) takes region (x / 4, x % 4) of a 2 x 4 grid of regions, row-major inside,
+        // so that the workgroups running together on an XCD share few A and B panels (a region of 16 x 8 tiles: 8 + 8 panels for 64
+        // workgroups instead of 2 + 32 with whole tile rows)
+        const uint32_t xcd = bid % 8u, local = bid / 8u, regw = g.tiles_n / 4u, regh = g.tiles_m / 2u;
+        tm = (xcd / 4u) * regh + local / regw;
+        tn = (xcd % 4u) * regw + local % regw;
+        bid = 0;
+    } else {
+        if (g.xcd_chunk) bid = (bid % 8u) * g.xcd_chunk + bid / 8u;
+        tn = bid % g.tiles_n;
+        bid /= g.tiles_n;
+        tm = bid % g.tiles_m;
+        bid /= g.tiles_m;
+    }
     int64_t oa = 0, ob = 0, oc = 0;
     uint32_t chunk_id = 0;
     for (int d = g.nbatch - 1; d >= 0; d--) {
@@ -654,6 +665,7 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
 #define DNH_GEMM(FASTF, ACCF, SPLITF) hipLaunchKernelGGL((gemm_kernel<T, FASTF, ACCF, SPLITF>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g)
     bool x3 = false;
     if constexpr (sizeof(T) == 4) x3 = fast && !g.accumulate && use_bf16x3();
+    g.xcd_2d = (x3 && g.nbatch == 0 && (g.tiles_m % 2u) == 0 && (g.tiles_n % 4u) == 0 && blocks >= 64) ? 1u : 0u;
     if (splits > 1) {
         if (x3) {
             if constexpr (sizeof(T) == 4) {
