@@ -441,7 +441,8 @@ __global__ __launch_bounds__(64 * SG) void gemm_split_finish_kernel(T* __restric
 // the product (inf - inf in its mid part; IEEE gives +-inf unless it meets a zero), and elements below 2^-126 (denormal) lose
 // precision, since their parts are bf16 denormals.  NaN stays NaN.  DNH_DOT_BF16X3=0 in the environment keeps every product on
 // the fp32 instructions.
-// Row-major, 16-byte aligned operands (K splits included); accumulating and strided products take gemm_kernel.
+// Every operand that is contiguous along one of its two dimensions (row-major or transposed; 16-byte aligned rows when k is the
+// contiguous one), K splits included; accumulating products and operands strided in both dimensions take gemm_kernel.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kX3BK = 16;
@@ -467,7 +468,71 @@ __device__ __forceinline__ void split3_bf16(const float (&v)[8], u32x4& hi, u32x
     }
 }
 
-template <bool SPLIT, bool TAIL>
+// Staging of one operand tile (128 rows x 16 k; "row" is m for A and n for B) from memory into the three bf16 tiles in LDS.
+//   KC: k is the contiguous direction.  Four lanes cover the 16 k of a row with one 16-byte load each (a wavefront reads 16 rows of
+//       64 contiguous bytes); a thread takes the same 4 k of rows r and r + 64 and writes 8 bytes per part and row.
+//   otherwise the rows are contiguous (row-major B, transposed A): a thread takes one row and 8 consecutive k with element loads
+//       (the lanes of a wavefront read 256 consecutive bytes) and writes 16 bytes per part.
+template <bool KC>
+struct X3Stage {
+    int row, kofs;      // first row and first k of this thread inside the tile
+    bool ok0, ok1;      // row (and for KC row + 64) inside the matrix
+    const float *p0, *p1;   // element (row, k = 0) of those rows; row 0 of the matrix when outside
+    int64_t ks;
+    __device__ __forceinline__ void init(const float* base, int64_t row0, int64_t limit, int64_t rs, int64_t kstride, int tid) {
+        row = KC ? tid >> 2 : tid & 127;
+        kofs = KC ? (tid & 3) * 4 : (tid >> 7) * 8;
+        ok0 = row0 + row < limit;
+        ok1 = KC && row0 + row + 64 < limit;
+        p0 = base + (ok0 ? (row0 + row) * rs : 0);
+        p1 = base + (ok1 ? (row0 + row + 64) * rs : 0);
+        ks = KC ? 1 : kstride;
+    }
+    template <bool TAIL>
+    __device__ __forceinline__ void load(int64_t k0, int64_t K, float (&r)[8]) const {
+        if (!TAIL || k0 + kX3BK <= K) {
+            if constexpr (KC) {
+                const Pack<float, 4> v0 = load_pack<float, 4>(p0 + k0 + kofs), v1 = load_pack<float, 4>(p1 + k0 + kofs);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    r[e] = v0.v[e];
+                    r[4 + e] = v1.v[e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) r[e] = p0[(k0 + kofs + e) * ks];
+            }
+        } else {
+            // TAIL (K is not a multiple of 16): the last, partial K step takes element loads from addresses clamped into the row, zeros beyond K
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int64_t k = k0 + kofs + (KC ? (e & 3) : e);
+                const float* p = (KC && e >= 4) ? p1 : p0;
+                const float v = p[(k < K ? k : K - 1) * ks];
+                r[e] = k < K ? v : 0.0f;
+            }
+        }
+    }
+    // cuts the staged elements into their parts and writes them to tile[part][row][k]
+    __device__ __forceinline__ void store(float (&r)[8], __bf16 (*tile)[BM][kX3Row]) const {
+#pragma unroll
+        for (int e = 0; e < 8; e++) r[e] = ((KC && e >= 4) ? ok1 : ok0) ? r[e] : 0.0f;
+        u32x4 part[3];
+        split3_bf16(r, part[0], part[1], part[2]);
+#pragma unroll
+        for (int s = 0; s < 3; s++) {
+            if constexpr (KC) {
+                typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+                *reinterpret_cast<u32x2*>(&tile[s][row][kofs]) = u32x2{part[s][0], part[s][1]};
+                *reinterpret_cast<u32x2*>(&tile[s][row + 64][kofs]) = u32x2{part[s][2], part[s][3]};
+            } else {
+                *reinterpret_cast<u32x4*>(&tile[s][row][kofs]) = part[s];
+            }
+        }
+    }
+};
+
+template <bool SPLIT, bool TAIL, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restrict__ c, const float* __restrict__ a, const float* __restrict__ b, GemmArgs g) {
     __shared__ __align__(16) __bf16 As[2][3][BM][kX3Row];
     __shared__ __align__(16) __bf16 Bs[2][3][BN][kX3Row];
@@ -507,55 +572,18 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
     c += oc;
     const int tid = threadIdx.x;
 
-    // staging: A rows are k-contiguous (two 16-byte loads = 8 floats of one row); B rows are n-contiguous, and the instruction
-    // wants 8 consecutive k of one column, so a thread takes one column and 8 rows (lanes = consecutive columns: 256-byte rows)
-    const int a_row = tid >> 1, a_kh = tid & 1;
-    const int b_col = tid & 127, b_kh = tid >> 7;
-    const bool a_ok = m0 + a_row < g.M, b_ok = n0 + b_col < g.N;
-    const float* arow = a + (a_ok ? (m0 + a_row) * g.sam : 0);
-    const float* bcol = b + (b_ok ? n0 + b_col : 0);
-    const float* ap = arow + a_kh * 8;
-    const float* bp = bcol + (int64_t)(b_kh * 8) * g.sbk;
+    X3Stage<A_KC> sa;
+    X3Stage<B_KC> sb;
+    sa.init(a, m0, g.M, g.sam, g.sak, tid);
+    sb.init(b, n0, g.N, g.sbn, g.sbk, tid);
     float ra[8], rb[8];
     auto load_tiles = [&](int64_t k0) {
-        if (!TAIL || k0 + kX3BK <= K) {
-            const Pack<float, 4> v0 = load_pack<float, 4>(ap + k0), v1 = load_pack<float, 4>(ap + k0 + 4);
-#pragma unroll
-            for (int e = 0; e < 4; e++) {
-                ra[e] = v0.v[e];
-                ra[4 + e] = v1.v[e];
-            }
-#pragma unroll
-            for (int e = 0; e < 8; e++) rb[e] = bp[(k0 + e) * g.sbk];
-        } else {
-            // TAIL (K is not a multiple of 16): the last, partial K step takes element loads from addresses clamped into the row / column, zeros beyond K
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const int64_t ka = k0 + a_kh * 8 + e, kb = k0 + b_kh * 8 + e;
-                const float va = arow[ka < K ? ka : K - 1], vb = bcol[(kb < K ? kb : K - 1) * g.sbk];
-                ra[e] = ka < K ? va : 0.0f;
-                rb[e] = kb < K ? vb : 0.0f;
-            }
-        }
+        sa.template load<TAIL>(k0, K, ra);
+        sb.template load<TAIL>(k0, K, rb);
     };
     auto store_tiles = [&](int buf) {
-        u32x4 hi, mid, lo;
-        if (!a_ok) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) ra[e] = 0.0f;
-        }
-        split3_bf16(ra, hi, mid, lo);
-        *reinterpret_cast<u32x4*>(&As[buf][0][a_row][a_kh * 8]) = hi;
-        *reinterpret_cast<u32x4*>(&As[buf][1][a_row][a_kh * 8]) = mid;
-        *reinterpret_cast<u32x4*>(&As[buf][2][a_row][a_kh * 8]) = lo;
-        if (!b_ok) {
-#pragma unroll
-            for (int e = 0; e < 8; e++) rb[e] = 0.0f;
-        }
-        split3_bf16(rb, hi, mid, lo);
-        *reinterpret_cast<u32x4*>(&Bs[buf][0][b_col][b_kh * 8]) = hi;
-        *reinterpret_cast<u32x4*>(&Bs[buf][1][b_col][b_kh * 8]) = mid;
-        *reinterpret_cast<u32x4*>(&Bs[buf][2][b_col][b_kh * 8]) = lo;
+        sa.store(ra, As[buf]);
+        sb.store(rb, Bs[buf]);
     };
 
     const int wave = tid >> 6, lane = tid & 63;
@@ -662,30 +690,41 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         }
     }
     g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
+#define DNH_X3_LAUNCH(SP, TL, AK, BK_) hipLaunchKernelGGL((gemm_bf16x3_kernel<SP, TL, AK, BK_>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g)
+#define DNH_X3_AB(SP, TL) do { if (a_kc) { if (b_kc) DNH_X3_LAUNCH(SP, TL, true, true); else DNH_X3_LAUNCH(SP, TL, true, false); } \
+                               else { if (b_kc) DNH_X3_LAUNCH(SP, TL, false, true); else DNH_X3_LAUNCH(SP, TL, false, false); } } while (0)
+#define DNH_X3(SP) do { if (g.K % kX3BK) DNH_X3_AB(SP, true); else DNH_X3_AB(SP, false); } while (0)
 #define DNH_GEMM(FASTF, ACCF, SPLITF) hipLaunchKernelGGL((gemm_kernel<T, FASTF, ACCF, SPLITF>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g)
     bool x3 = false;
-    if constexpr (sizeof(T) == 4) x3 = fast && !g.accumulate && use_bf16x3();
+    bool a_kc = false, b_kc = false;
+    if constexpr (sizeof(T) == 4) {
+        // each operand either k-contiguous with 16-byte aligned rows, or contiguous along its other dimension
+        a_kc = g.sak == 1 && (g.sam % 4) == 0 && aligned_to(a, 16);
+        b_kc = g.sbk == 1 && (g.sbn % 4) == 0 && aligned_to(b, 16);
+        for (int d = 0; d < orig.nbatch; d++) {
+            a_kc = a_kc && (orig.bsa[d] % 4) == 0;
+            b_kc = b_kc && (orig.bsb[d] % 4) == 0;
+        }
+        x3 = g.K > 0 && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_bf16x3();
+    }
     g.xcd_2d = (x3 && g.nbatch == 0 && (g.tiles_m % 2u) == 0 && (g.tiles_n % 4u) == 0 && blocks >= 64) ? 1u : 0u;
     if (splits > 1) {
         if (x3) {
-            if constexpr (sizeof(T) == 4) {
-                if (g.K % kX3BK) hipLaunchKernelGGL((gemm_bf16x3_kernel<true, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
-                else hipLaunchKernelGGL((gemm_bf16x3_kernel<true, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
-            }
+            if constexpr (sizeof(T) == 4) DNH_X3(true);
         } else if (fast) DNH_GEMM(true, false, true);
         else DNH_GEMM(false, false, true);
     } else if (g.accumulate) {
         if (fast) DNH_GEMM(true, true, false); else DNH_GEMM(false, true, false);
     } else {
         if (x3) {
-            if constexpr (sizeof(T) == 4) {
-                if (g.K % kX3BK) hipLaunchKernelGGL((gemm_bf16x3_kernel<false, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
-                else hipLaunchKernelGGL((gemm_bf16x3_kernel<false, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g);
-            }
+            if constexpr (sizeof(T) == 4) DNH_X3(false);
         } else if (fast) DNH_GEMM(true, false, false);
         else DNH_GEMM(false, false, false);
     }
 #undef DNH_GEMM
+#undef DNH_X3
+#undef DNH_X3_AB
+#undef DNH_X3_LAUNCH
     DNH_LAUNCH_CHECK();
     if (splits > 1) {
         constexpr int FV = 16 / (int)sizeof(T);

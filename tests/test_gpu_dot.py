@@ -252,3 +252,18 @@ def test_single_precision_on_bf16_parts_special_values(G):
     a[3, 5] = np.inf
     got = G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b))
     assert not np.any(np.isfinite(got[3])) and np.all(np.delete(got, 3, axis=0) == 16)
+
+
+@pytest.mark.parametrize("ta,tb", [(True, False), (False, True), (True, True)])
+@pytest.mark.parametrize("m,k,n", [(200, 64, 300), (257, 100, 130), (1100, 40, 1500)])
+def test_single_precision_on_bf16_parts_transposed_views(H, G, rng, ta, tb, m, k, n):
+    """Operands that are transposed views of row-major matrices take the same kernel with the other staging."""
+    a = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
+    b = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)
+    f = lambda x, y: (x.T if ta else x) @ (y.T if tb else y)
+    ref, got = both(H, G, f, a, b)
+    an, bn = (a.T if ta else a), (b.T if tb else b)
+    check_dot(ref, got, an, bn)
+    exact = an.astype(np.float64) @ bn.astype(np.float64)
+    S = np.abs(an).astype(np.float64) @ np.abs(bn).astype(np.float64)
+    assert np.all(np.abs(got - exact) <= 16 * 2.0 ** -24 * S)
