@@ -532,7 +532,7 @@ struct X3Stage {
     }
 };
 
-template <bool SPLIT, bool TAIL, bool A_KC, bool B_KC, bool ROWS_FAST>
+template <bool SPLIT, bool TAIL, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restrict__ c, const float* __restrict__ a, const float* __restrict__ b, GemmArgs g) {
     __shared__ __align__(16) __bf16 As[2][3][BM][kX3Row];
     __shared__ __align__(16) __bf16 Bs[2][3][BN][kX3Row];
@@ -632,45 +632,16 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
     }
     // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile
     const bool full_mn = m0 + BM <= g.M && n0 + BN <= g.N;
-    if constexpr (!ROWS_FAST) {
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+    for (int i = 0; i < 2; i++)
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+        for (int j = 0; j < 2; j++)
 #pragma unroll
-                for (int r = 0; r < 16; r++) {
-                    const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
-                    const int64_t n = n0 + wn + j * 32 + lm;
-                    if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
-                }
-    } else {
-        // The target's contiguous direction is this kernel's row index (a row-major product computed as B^T A^T, see the launch):
-        // the lanes of an accumulator run along the columns, so the wavefront's 64 x 64 block goes through LDS (the operand tiles
-        // are done with), written as [column][row] with four consecutive rows per 16-byte store, read back one column at a time
-        // with the lanes along the rows: 256 contiguous bytes per store instruction.
-        constexpr int TS = 68;   // floats per column of the staging block: 64 + 4, 16-byte aligned and conflict-free
-        static_assert(sizeof(As) >= 2 * 64 * TS * sizeof(float) && sizeof(Bs) >= 2 * 64 * TS * sizeof(float), "staging blocks of two wavefronts each");
-        __syncthreads();         // every wavefront has read its last operands
-        float* stage = reinterpret_cast<float*>(wave < 2 ? (void*)As : (void*)Bs) + (wave & 1) * 64 * TS;
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int q = 0; q < 4; q++) {
-                    Pack<float, 4> v;
-#pragma unroll
-                    for (int e = 0; e < 4; e++) v.v[e] = acc[i][j][4 * q + e];
-                    store_pack<float, 4>(stage + (j * 32 + lm) * TS + i * 32 + q * 8 + lk * 4, v);
-                }
-        // the block is private to the wavefront: its own LDS accesses are ordered, no barrier
-        const int64_t m = m0 + wm + lane;
-        for (int col = 0; col < 64; col++) {
-            const int64_t n = n0 + wn + col;
-            const float v = stage[col * TS + lane];
-            if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = v;
-        }
-    }
+            for (int r = 0; r < 16; r++) {
+                const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
+                const int64_t n = n0 + wn + j * 32 + lm;
+                if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
+            }
 }
 
 bool use_bf16x3() {
@@ -719,8 +690,7 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         }
     }
     g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
-#define DNH_X3_LAUNCH(SP, TL, AK, BK_) do { if (rows_fast) hipLaunchKernelGGL((gemm_bf16x3_kernel<SP, TL, AK, BK_, true>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g); \
-                                             else hipLaunchKernelGGL((gemm_bf16x3_kernel<SP, TL, AK, BK_, false>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g); } while (0)
+#define DNH_X3_LAUNCH(SP, TL, AK, BK_) hipLaunchKernelGGL((gemm_bf16x3_kernel<SP, TL, AK, BK_>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g)
 #define DNH_X3_AB(SP, TL) do { if (a_kc) { if (b_kc) DNH_X3_LAUNCH(SP, TL, true, true); else DNH_X3_LAUNCH(SP, TL, true, false); } \
                                else { if (b_kc) DNH_X3_LAUNCH(SP, TL, false, true); else DNH_X3_LAUNCH(SP, TL, false, false); } } while (0)
 #define DNH_X3(SP) do { if (g.K % kX3BK) DNH_X3_AB(SP, true); else DNH_X3_AB(SP, false); } while (0)
@@ -736,21 +706,6 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
             b_kc = b_kc && (orig.bsb[d] % 4) == 0;
         }
         x3 = g.K > 0 && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_bf16x3();
-    }
-    // A row-major product (A fetched in 64-byte pieces, B in 256-byte rows) runs faster with the roles exchanged, C^T = B^T A^T
-    // (measured at 4096^3: 149 against 190 TFLOP/s); the kernel then writes through its rows-contiguous epilogue.
-    bool rows_fast = false;
-    if (x3 && a_kc && !b_kc && g.scn == 1) {
-        std::swap(a, b);
-        std::swap(g.M, g.N);
-        std::swap(g.sam, g.sbn);
-        std::swap(g.sak, g.sbk);
-        std::swap(g.scm, g.scn);
-        std::swap(g.tiles_m, g.tiles_n);
-        for (int d = 0; d < g.nbatch; d++) std::swap(g.bsa[d], g.bsb[d]);
-        a_kc = false;
-        b_kc = true;
-        rows_fast = true;
     }
     g.xcd_2d = (x3 && g.nbatch == 0 && (g.tiles_m % 2u) == 0 && (g.tiles_n % 4u) == 0 && blocks >= 64) ? 1u : 0u;
     if (splits > 1) {
