@@ -26,7 +26,7 @@ class Timer:
         entry, args = call
         self.native.check(getattr(self.lib, "dnh_" + entry)(*args, self.stream))
 
-    def time(self, sets, reps=20, warm=3):
+    def time(self, sets, reps=20, warm=10):
         """sets: list of call lists (one list of (entry, args) per buffer set).  Returns average ms per pass over one set."""
         lib, check = self.lib, self.native.check
         for i in range(warm):
