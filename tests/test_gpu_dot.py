@@ -267,3 +267,30 @@ def test_single_precision_on_bf16_parts_transposed_views(H, G, rng, ta, tb, m, k
     exact = an.astype(np.float64) @ bn.astype(np.float64)
     S = np.abs(an).astype(np.float64) @ np.abs(bn).astype(np.float64)
     assert np.all(np.abs(got - exact) <= 16 * 2.0 ** -24 * S)
+
+
+def test_fp32_instruction_kernel_behind_the_switch():
+    """DNH_DOT_BF16X3=0 sends single-precision products to the fp32 matrix instructions (the switch is read once per process, so
+    this runs in a child process): same contract, and infinities follow IEEE arithmetic there."""
+    import os
+    import subprocess
+    import sys
+    code = r'''
+import numpy as np
+from deepnet_amd import hip as G
+rng = np.random.default_rng(3)
+for (m, k, n) in ((200, 64, 300), (384, 16, 256), (130, 70, 50), (1024, 1024, 1024)):
+    a = rng.standard_normal((m, k)).astype(np.float32); b = rng.standard_normal((k, n)).astype(np.float32)
+    got = G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b)).astype(np.float64)
+    exact = a.astype(np.float64) @ b.astype(np.float64)
+    S = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
+    assert np.all(np.abs(got - exact) <= (2 * k + 64) * 2.0 ** -24 * S), (m, k, n)
+a = np.ones((128, 16), np.float32); b = np.ones((16, 128), np.float32); a[3, 5] = np.inf
+got = G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b))
+assert np.all(np.isposinf(got[3])) and np.all(np.delete(got, 3, axis=0) == 16)
+print("ok")
+'''
+    env = dict(os.environ, DNH_DOT_BF16X3="0")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
