@@ -143,6 +143,12 @@ LAPACK_OP_SIGNATURES = {
     "symmetric_eig": [C.c_int32, _T, _T, _T],  # part (0 upper, 1 lower), eigvals, eigvecs, src
 }
 
+# entry points with no counterpart in the reference's interface (hence none in the oracle)
+DEVICE_ONLY_OP_SIGNATURES = {
+    "reduce_last_axis_noalloc": [C.c_int32, _T, _T],   # dnh_reduce_last_axis with its partial results in a static device array
+}
+STATIC_SCRATCH_BYTES = 8 << 20
+
 # every symbol include/tensor_hip.h declares
 EXPORTED_SYMBOLS = [
     "dnh_init", "dnh_device_info", "dnh_last_error", "dnh_async_error",
@@ -151,4 +157,4 @@ EXPORTED_SYMBOLS = [
     "dnh_memcpy_h2d", "dnh_memcpy_d2h", "dnh_memcpy_d2d",
     "dnh_stream_create", "dnh_stream_destroy", "dnh_stream_sync", "dnh_device_sync",
     "dnh_event_create", "dnh_event_destroy", "dnh_event_record", "dnh_event_sync", "dnh_event_elapsed_ms",
-] + ["dnh_" + k for k in OP_SIGNATURES] + ["dnh_" + k for k in LAPACK_OP_SIGNATURES]
+] + ["dnh_" + k for k in OP_SIGNATURES] + ["dnh_" + k for k in LAPACK_OP_SIGNATURES] + ["dnh_" + k for k in DEVICE_ONLY_OP_SIGNATURES]

@@ -6,6 +6,8 @@
 #include "reduce_kernels.h"
 #include "ops.h"
 
+#include <mutex>
+
 using namespace dnh;
 
 namespace {
@@ -92,16 +94,16 @@ template <class X> struct RFind {
 };
 
 template <template <class> class RT>
-int32_t run_numeric(const DnhTensor* t, const DnhTensor* s, hipStream_t st, const char* what) {
+int32_t run_numeric(const DnhTensor* t, const DnhTensor* s, hipStream_t st, const char* what, const PartialStore& ps) {
     switch (s->dtype) {
-        case DNH_U8: return launch_reduce(RT<uint8_t>{}, t, s, st, what);
-        case DNH_I8: return launch_reduce(RT<int8_t>{}, t, s, st, what);
-        case DNH_I32: return launch_reduce(RT<int32_t>{}, t, s, st, what);
-        case DNH_U32: return launch_reduce(RT<uint32_t>{}, t, s, st, what);
-        case DNH_I64: return launch_reduce(RT<int64_t>{}, t, s, st, what);
-        case DNH_U64: return launch_reduce(RT<uint64_t>{}, t, s, st, what);
-        case DNH_F32: return launch_reduce(RT<float>{}, t, s, st, what);
-        case DNH_F64: return launch_reduce(RT<double>{}, t, s, st, what);
+        case DNH_U8: return launch_reduce(RT<uint8_t>{}, t, s, st, what, ps);
+        case DNH_I8: return launch_reduce(RT<int8_t>{}, t, s, st, what, ps);
+        case DNH_I32: return launch_reduce(RT<int32_t>{}, t, s, st, what, ps);
+        case DNH_U32: return launch_reduce(RT<uint32_t>{}, t, s, st, what, ps);
+        case DNH_I64: return launch_reduce(RT<int64_t>{}, t, s, st, what, ps);
+        case DNH_U64: return launch_reduce(RT<uint64_t>{}, t, s, st, what, ps);
+        case DNH_F32: return launch_reduce(RT<float>{}, t, s, st, what, ps);
+        case DNH_F64: return launch_reduce(RT<double>{}, t, s, st, what, ps);
     }
     return fail(DNH_ERR_NOT_SUPPORTED, "%s is not defined for %s", what, dtype_name(s->dtype));
 }
@@ -123,27 +125,68 @@ int32_t run_arg(const DnhTensor* t, const DnhTensor* s, hipStream_t st, const ch
 
 }  // namespace
 
-extern "C" int32_t dnh_reduce_last_axis(int32_t op, const DnhTensor* t, const DnhTensor* src, void* stream) {
-    DNH_TRY(ensure_init());
-    DNH_TRY(check_tensor(t, "dnh_reduce_last_axis"));
-    DNH_TRY(check_tensor(src, "dnh_reduce_last_axis"));
-    hipStream_t st = (hipStream_t)stream;
+// The folds of dnh_reduce_last_axis; `ps` says where the partial results of a two-pass fold are kept.
+static int32_t reduce_impl(const char* entry, int32_t op, const DnhTensor* t, const DnhTensor* src, hipStream_t st, const PartialStore& ps) {
+    DNH_TRY(check_tensor(t, entry));
+    DNH_TRY(check_tensor(src, entry));
     if (op == DNH_ALL || op == DNH_ANY) {
         if (src->dtype != DNH_BOOL || t->dtype != DNH_BOOL) return fail(DNH_ERR_INVALID_ARG, "All/Any need bool source and target");
-        return op == DNH_ALL ? launch_reduce(RAll{}, t, src, st, "AllLastAxis") : launch_reduce(RAny{}, t, src, st, "AnyLastAxis");
+        return op == DNH_ALL ? launch_reduce(RAll{}, t, src, st, "AllLastAxis", ps) : launch_reduce(RAny{}, t, src, st, "AnyLastAxis", ps);
     }
     if (op == DNH_COUNT_TRUE) {
         if (src->dtype != DNH_BOOL || t->dtype != DNH_I64) return fail(DNH_ERR_INVALID_ARG, "CountTrue needs a bool source and an int64 target");
-        return launch_reduce(RCountTrue{}, t, src, st, "CountTrueLastAxis");
+        return launch_reduce(RCountTrue{}, t, src, st, "CountTrueLastAxis", ps);
     }
-    if (t->dtype != src->dtype) return fail(DNH_ERR_INVALID_ARG, "dnh_reduce_last_axis: target is %s but source is %s", dtype_name(t->dtype), dtype_name(src->dtype));
+    if (t->dtype != src->dtype) return fail(DNH_ERR_INVALID_ARG, "%s: target is %s but source is %s", entry, dtype_name(t->dtype), dtype_name(src->dtype));
     switch (op) {
-        case DNH_SUM: return run_numeric<RSum>(t, src, st, "SumLastAxis");
-        case DNH_PRODUCT: return run_numeric<RProd>(t, src, st, "ProductLastAxis");
-        case DNH_MIN: return run_numeric<RMin>(t, src, st, "MinLastAxis");
-        case DNH_MAX: return run_numeric<RMax>(t, src, st, "MaxLastAxis");
+        case DNH_SUM: return run_numeric<RSum>(t, src, st, "SumLastAxis", ps);
+        case DNH_PRODUCT: return run_numeric<RProd>(t, src, st, "ProductLastAxis", ps);
+        case DNH_MIN: return run_numeric<RMin>(t, src, st, "MinLastAxis", ps);
+        case DNH_MAX: return run_numeric<RMax>(t, src, st, "MaxLastAxis", ps);
     }
-    return fail(DNH_ERR_INVALID_ARG, "dnh_reduce_last_axis: unknown op %d", op);
+    return fail(DNH_ERR_INVALID_ARG, "%s: unknown op %d", entry, op);
+}
+
+extern "C" int32_t dnh_reduce_last_axis(int32_t op, const DnhTensor* t, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    return reduce_impl("dnh_reduce_last_axis", op, t, src, (hipStream_t)stream, PartialStore());
+}
+
+// ---- the fold entry point that allocates nothing ---------------------------------------------------------------------------------
+// Partial results of two-pass folds live in a file-scope device array instead of the stream's workspace.  Every GPU the library runs
+// on holds its own copy of the array, at its own address, until the process ends.  In host code the array's name is only a handle for
+// hipGetSymbolAddress: the device address is looked up once per device and that pointer is what the kernels receive.
+static __device__ __align__(256) unsigned char scratch[DNH_STATIC_SCRATCH_BYTES];
+
+namespace {
+constexpr int kMaxScratchDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxScratchDevices] = {};
+
+// Device address of `scratch` on the calling thread's current device (looked up on the first call per device).
+int32_t static_scratch(void** out) {
+    int dev = -1;
+    DNH_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxScratchDevices) return fail(DNH_ERR_NOT_SUPPORTED, "static scratch: device %d outside 0..%d", dev, kMaxScratchDevices - 1);
+    std::lock_guard<std::mutex> lock(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        DNH_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        if (!p) return fail(DNH_ERR_HIP, "static scratch: hipGetSymbolAddress returned a null address");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return DNH_OK;
+}
+}  // namespace
+
+extern "C" int32_t dnh_reduce_last_axis_noalloc(int32_t op, const DnhTensor* t, const DnhTensor* src, void* stream) {
+    DNH_TRY(ensure_init());
+    PartialStore ps;
+    DNH_TRY(static_scratch(&ps.fixed));
+    ps.fixed_bytes = DNH_STATIC_SCRATCH_BYTES;
+    // Partials are written by the first pass before the second reads them, so nothing in the array has to start at zero.
+    return reduce_impl("dnh_reduce_last_axis_noalloc", op, t, src, (hipStream_t)stream, ps);
 }
 
 extern "C" int32_t dnh_arg_reduce_last_axis(int32_t op, const DnhTensor* t, const DnhTensor* src, void* stream) {

@@ -261,8 +261,25 @@ int32_t launch_finish(const R& r, typename R::State* partial, typename R::Out* o
     return DNH_OK;
 }
 
+// Where the State partials of a two-pass fold go: the stream's grow-on-demand workspace, or a buffer of fixed size the caller
+// names (the entry point that may not allocate), which refuses what does not fit.
+struct PartialStore {
+    void* fixed = nullptr;
+    size_t fixed_bytes = 0;
+};
+
+inline int32_t partial_buffer(const PartialStore& ps, hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease, const char* what) {
+    if (!ps.fixed) return workspace(stream, bytes, out, lease);
+    if (bytes > ps.fixed_bytes)
+        return fail(DNH_ERR_NOT_SUPPORTED, "%s: this fold needs %zu bytes of partial results, the static scratch array holds %zu", what, bytes,
+                    ps.fixed_bytes);
+    *out = ps.fixed;
+    return DNH_OK;
+}
+
 template <class R>
-int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStream_t stream, const char* what) {
+int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStream_t stream, const char* what,
+                      const PartialStore& ps = PartialStore()) {
     using In = typename R::In;
     using Out = typename R::Out;
     using State = typename R::State;
@@ -339,7 +356,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         }
         State* partial = nullptr;
         WorkspaceLease lease;
-        if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial, lease));
+        if (splits > 1) DNH_TRY(partial_buffer(ps, stream, sizeof(State) * (size_t)nout * splits, (void**)&partial, lease, what));
         const dim3 grid((unsigned)row_blocks, splits);
 #define DNH_ROWS(V, TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, V, TPR, false>), grid, dim3(kBlock), 0, stream, r, (const void*)src, out, partial, o, nout, n, sr, chunk, splits)
         if (vec) {
@@ -403,7 +420,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         if (total_blocks <= 0x7FFFFFFF) {
             State* partial = nullptr;
             WorkspaceLease lease;
-            if (splits > 1) DNH_TRY(workspace(stream, sizeof(State) * (size_t)nout * splits, (void**)&partial, lease));
+            if (splits > 1) DNH_TRY(partial_buffer(ps, stream, sizeof(State) * (size_t)nout * splits, (void**)&partial, lease, what));
             const dim3 grid((unsigned)total_blocks);
             const uint32_t xcd_chunk = (total_blocks % 8 == 0 && total_blocks >= 64) ? (uint32_t)(total_blocks / 8) : 0u;
 #define DNH_COLS(V, W) hipLaunchKernelGGL((reduce_cols_kernel<R, V, W>), grid, dim3(kBlock), 0, stream, r, src, out, partial, oo, col_tiles, (uint32_t)base_blocks, xcd_chunk, nc, tc_stride, n, sr, chunk, splits)

@@ -58,7 +58,7 @@ def load() -> C.CDLL:
         "dnh_event_sync": [vp],
         "dnh_event_elapsed_ms": [vp, vp, C.POINTER(C.c_float)],
     }
-    for name, args in list(abi.OP_SIGNATURES.items()) + list(abi.LAPACK_OP_SIGNATURES.items()):
+    for name, args in list(abi.OP_SIGNATURES.items()) + list(abi.LAPACK_OP_SIGNATURES.items()) + list(abi.DEVICE_ONLY_OP_SIGNATURES.items()):
         sigs["dnh_" + name] = list(args) + [vp]  # every op takes the stream last
     for name, args in sigs.items():
         fn = getattr(lib, name)

@@ -211,6 +211,16 @@ int32_t dnh_if_then_else(const DnhTensor* t, const DnhTensor* cond_bool, const D
  * strides of `src` are arbitrary and select the kernel strategy.
  * ------------------------------------------------------------------------------------------------- */
 int32_t dnh_reduce_last_axis(int32_t op, const DnhTensor* t, const DnhTensor* src, void* stream);
+/* The folds of dnh_reduce_last_axis for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid it).  No counterpart in the reference.  Same arguments, same kernels and bit-identical results;
+ * the partial results of two-pass folds are kept in an array of DNH_STATIC_SCRATCH_BYTES that is part of the library's device
+ * image, so the call never allocates or frees.  A fold whose partials do not fit returns DNH_ERR_NOT_SUPPORTED: folds with a state
+ * as wide as their elements need at most about 4 MiB whatever the shape; only CountTrue down the columns of a bool matrix (an
+ * int64 per column and chunk of 512 rows, for up to 1024 chunks x column tiles) can need more.  Every call on one GPU shares that
+ * GPU's array and leaves its partials there: calls that overlap on one GPU, on any streams, race; issue them on one stream or
+ * order them yourself. */
+#define DNH_STATIC_SCRATCH_BYTES (8u << 20)
+int32_t dnh_reduce_last_axis_noalloc(int32_t op, const DnhTensor* t, const DnhTensor* src, void* stream);
 int32_t dnh_arg_reduce_last_axis(int32_t op, const DnhTensor* t_i64, const DnhTensor* src, void* stream);
 /* ITensorBackend.FindLastAxis (TensorBackend.fs:135; Host/ScalarOps.fs:656-665): first index equal to *value, else DNH_NOT_FOUND. */
 int32_t dnh_find_last_axis(const void* value, const DnhTensor* t_i64, const DnhTensor* src, void* stream);
