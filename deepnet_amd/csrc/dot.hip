@@ -437,10 +437,13 @@ __global__ __launch_bounds__(64 * SG) void gemm_split_finish_kernel(T* __restric
 // The six largest are kept: hi.hi, hi.mid, mid.hi, hi.lo, lo.hi, mid.mid; the three dropped (mid.lo, lo.mid, lo.lo) are below
 // 2^-21 |a||b|, usually 2^-25, i.e. a few units of the rounding of one fp32 product, against a contract of K of them.  Six bf16
 // instructions of K = 16 replace eight fp32 instructions of K = 2 per 32 x 32 x 16 block: 2.7 times fewer matrix-pipe cycles.
-// Two deviations from fp32 arithmetic, both outside finite normal inputs: an infinite element gives NaN in its row / column of
-// the product (inf - inf in its mid part; IEEE gives +-inf unless it meets a zero), and elements below 2^-126 (denormal) lose
-// precision, since their parts are bf16 denormals.  NaN stays NaN.  DNH_DOT_BF16X3=0 in the environment keeps every product on
-// the fp32 instructions.
+// The cut is exact only for finite elements whose parts are representable: an infinite element would give inf - inf = NaN in its
+// mid part, and below 2^-109 the lo part (lowest bit 2^(e-23)) falls under the smallest bf16 denormal, 2^-133.  Every staged element
+// is therefore classified (one multiply by 2^-17 and one class test: infinite, or denormal after the scaling); a workgroup that has
+// met such an element in its rows of A or columns of B recomputes its tile with the fp32 matrix instruction (fp32_tile_fallback:
+// IEEE products and sums, inf x finite = inf, inf x 0 = NaN, as the reference's sgemm).  NaN needs no fallback: one part of a NaN is
+// a NaN.  Products with K < 16 (no whole K step; worst case 8 u per product from the three dropped terms against 1 u of one
+// rounded fp32 product) stay on the fp32 instructions.  DNH_DOT_BF16X3=0 in the environment keeps every product there.
 // Every operand that is contiguous along one of its two dimensions (row-major or transposed; 16-byte aligned rows when k is the
 // contiguous one), K splits included; accumulating products and operands strided in both dimensions take gemm_kernel.
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -479,6 +482,7 @@ struct X3Stage {
     bool ok0, ok1;      // row (and for KC row + 64) inside the matrix
     const float *p0, *p1;   // element (row, k = 0) of those rows; row 0 of the matrix when outside
     int64_t ks;
+    bool bad;           // an element staged so far is infinite or too small to cut into bf16 parts
     __device__ __forceinline__ void init(const float* base, int64_t row0, int64_t limit, int64_t rs, int64_t kstride, int tid) {
         row = KC ? tid >> 2 : tid & 127;
         kofs = KC ? (tid & 3) * 4 : (tid >> 7) * 8;
@@ -487,6 +491,7 @@ struct X3Stage {
         p0 = base + (ok0 ? (row0 + row) * rs : 0);
         p1 = base + (ok1 ? (row0 + row + 64) * rs : 0);
         ks = KC ? 1 : kstride;
+        bad = false;
     }
     template <bool TAIL>
     __device__ __forceinline__ void load(int64_t k0, int64_t K, float (&r)[8]) const {
@@ -514,9 +519,13 @@ struct X3Stage {
         }
     }
     // cuts the staged elements into their parts and writes them to tile[part][row][k]
-    __device__ __forceinline__ void store(float (&r)[8], __bf16 (*tile)[BM][kX3Row]) const {
+    __device__ __forceinline__ void store(float (&r)[8], __bf16 (*tile)[BM][kX3Row]) {
 #pragma unroll
         for (int e = 0; e < 8; e++) r[e] = ((KC && e >= 4) ? ok1 : ok0) ? r[e] : 0.0f;
+        // +-inf stays infinite under the scaling; |x| < 2^-109 (x != 0) becomes denormal; zero stays zero
+        constexpr int kClassInfOrDenormal = (1 << 2) | (1 << 4) | (1 << 7) | (1 << 9);
+#pragma unroll
+        for (int e = 0; e < 8; e++) bad |= __builtin_amdgcn_classf(r[e] * 0x1p-17f, kClassInfOrDenormal);
         u32x4 part[3];
         split3_bf16(r, part[0], part[1], part[2]);
 #pragma unroll
@@ -531,6 +540,59 @@ struct X3Stage {
         }
     }
 };
+
+// One 128 x 128 tile of c = a . b over k in [0, K) on v_mfma_f32_32x32x2_f32, operands fetched element by element through their
+// strides: the slow, IEEE-faithful path of a workgroup of gemm_bf16x3_kernel whose operands hold infinite or very small elements.
+// A32 / B32: [16][BM + PAD] floats of LDS each; every thread of the block calls it.
+__device__ __forceinline__ void fp32_tile_fallback(float* c, const float* a, const float* b, const GemmArgs& g, int64_t m0, int64_t n0, int64_t K,
+                                                float (*A32)[BM + PAD], float (*B32)[BN + PAD]) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64, lk = lane >> 5, lm = lane & 31;
+    f32x16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+    for (int64_t k0 = 0; k0 < K; k0 += 16) {
+        __syncthreads();   // the previous step's operand reads (and, on entry, the caller's use of the memory) are over
+#pragma unroll 2
+        for (int i = 0; i < BM * 16 / kBlock; i++) {
+            const int idx = tid + i * kBlock;
+            {
+                const int row = idx / 16, kk = idx % 16;
+                const int64_t m = m0 + row, k = k0 + kk;
+                A32[kk][row] = (m < g.M && k < K) ? a[m * g.sam + k * g.sak] : 0.0f;
+            }
+            {
+                const int kk = idx / BN, col = idx % BN;
+                const int64_t k = k0 + kk, n = n0 + col;
+                B32[kk][col] = (k < K && n < g.N) ? b[k * g.sbk + n * g.sbn] : 0.0f;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < 16; kk += 2) {
+            const float a0 = A32[kk + lk][wm + lm], a1 = A32[kk + lk][wm + 32 + lm];
+            const float b0 = B32[kk + lk][wn + lm], b1 = B32[kk + lk][wn + 32 + lm];
+            acc[0][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b0, acc[0][0], 0, 0, 0);
+            acc[0][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a0, b1, acc[0][1], 0, 0, 0);
+            acc[1][0] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b0, acc[1][0], 0, 0, 0);
+            acc[1][1] = __builtin_amdgcn_mfma_f32_32x32x2f32(a1, b1, acc[1][1], 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
+                const int64_t n = n0 + wn + j * 32 + lm;
+                if (m < g.M && n < g.N) c[m * g.scm + n * g.scn] = acc[i][j][r];
+            }
+}
 
 template <bool SPLIT, bool TAIL, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restrict__ c, const float* __restrict__ a, const float* __restrict__ b, GemmArgs g) {
@@ -630,6 +692,12 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
             cur ^= 1;
         }
     }
+    // an element that cannot be cut into bf16 parts was staged by some thread: the whole tile is redone on the fp32 instruction
+    if (__syncthreads_or((int)(sa.bad | sb.bad))) {
+        fp32_tile_fallback(c, a, b, g, m0, n0, K, reinterpret_cast<float (*)[BM + PAD]>(&As[0][0][0][0]),
+                           reinterpret_cast<float (*)[BN + PAD]>(&Bs[0][0][0][0]));
+        return;
+    }
     // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile
     const bool full_mn = m0 + BM <= g.M && n0 + BN <= g.N;
 #pragma unroll
@@ -705,7 +773,7 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
             a_kc = a_kc && (orig.bsa[d] % 4) == 0;
             b_kc = b_kc && (orig.bsb[d] % 4) == 0;
         }
-        x3 = g.K > 0 && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_bf16x3();
+        x3 = g.K >= kX3BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_bf16x3();
     }
     g.xcd_2d = (x3 && g.nbatch == 0 && (g.tiles_m % 2u) == 0 && (g.tiles_n % 4u) == 0 && blocks >= 64) ? 1u : 0u;
     if (splits > 1) {

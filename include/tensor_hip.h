@@ -247,9 +247,15 @@ int32_t dnh_true_indices(const DnhTensor* t_i64, const DnhTensor* src_bool, void
 /* ---------------------------------------------------------------------------------------------------
  * Dot: ITensorBackend VecVecDot / MatVecDot / MatMatDot / BatchedMatMatDot (TensorBackend.fs:137-140;
  * Host/HostBackend.fs:463-546).  The ranks of (t, a, b) select the variant exactly as Tensor.FillDot does
- * (Tensor.fs:2714-2730): (0,1,1) (1,2,1) (2,2,2) or (n,n,n) with n>2.  fp32 and fp64 on the
- * matrix cores (row-major single-precision operands: bf16 instructions on floats cut into three bf16 parts, same error bound;
- * an infinite element then gives NaN, DNH_DOT_BF16X3=0 in the environment selects the fp32 instructions); the integer types wrap like the host backend's multiply + sumAxis (HostBackend.fs:544-546); bool: status 2.
+ * (Tensor.fs:2714-2730): (0,1,1) (1,2,1) (2,2,2) or (n,n,n) with n>2.  fp32 and fp64 on the matrix cores.  Single-precision
+ * operands that are contiguous along one of their two dimensions, with K >= 16, run on the bf16 instructions with every float cut
+ * into three bf16 parts (six of the nine partial products; error within 16 u S of the exact product like an fp32 sgemm, u = 2^-24,
+ * S = sum_k |a_ik||b_kj|); tiles whose operands hold an infinite element or a nonzero element below 2^-109, which cannot be cut
+ * exactly, are computed with the fp32 instruction, so infinities and NaNs come out as IEEE arithmetic (the reference's sgemm) gives
+ * them.  DNH_DOT_BF16X3=0 in the environment keeps every product on the fp32 instruction (a tuning switch, same results contract).
+ * Denormal operands are honoured, but the single-precision matrix instruction flushes products and partial sums below 2^-126 to
+ * zero: results carry an absolute error of up to K x 2^-126 on top of the bound.  The integer types wrap like the host backend's
+ * multiply + sumAxis (HostBackend.fs:544-546); bool: status 2.
  * ------------------------------------------------------------------------------------------------- */
 int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream);
 

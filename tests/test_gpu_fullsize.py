@@ -123,7 +123,7 @@ def test_config5_mlp_block(G):
     for i in (0, 17, 63):                                        # fp64 truth on a few batches (the full fp64 product is slow on CPU)
         exact = a[i].astype(np.float64) @ b[i].astype(np.float64)
         S = np.abs(a[i]).astype(np.float64) @ np.abs(b[i]).astype(np.float64)
-        assert np.all(np.abs(cn[i] - exact) <= (2 * 512 + 64) * u * S)
+        assert np.all(np.abs(cn[i] - exact) <= 16 * u * S)      # measured 3.1 u S; a dropped partial product costs 10 u S and more
     t = c.tanh()
     mx = t.maxAxis(2)
     e = (t - mx[:, :, None]).exp()
