@@ -10,8 +10,12 @@ axis plus a full-tensor Sum (reductions) — nine backend calls through the C AB
 Every op's launches are bracketed by HIP events on the stream they run on; the `roofline` object is the op that takes
 the largest share of the step.  Consecutive ops read different 256 MiB tensors so the 256 MB Infinity Cache cannot
 serve re-reads.  `cpu_baseline` times the CPU oracle (oracle/hostref.cpp, the HostTensor restatement) on the same step.
+`configs` carries the other benchmark configurations (element-wise chain, permuted + broadcast add, double-precision
+folds, integer / bool indexing, batched dot + softmax pieces): one entry per backend call with its algorithmic bytes or
+FLOPs, the mean of >= 20 event-timed launches over rotated buffer sets and the fraction of 8 TB/s or of the fp32 / fp64
+matrix peak; `config_summary` aggregates them per configuration.  They are measured after the timed region.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-configs] [--all] [--no-cpu]
 """
 import argparse
 import ctypes as C
@@ -27,9 +31,22 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, vendor figure
 FP32_MFMA_PEAK_TFLOPS = 157.3
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (profiles/), scaled by the plain-copy calibration
-# (FETCH_SIZE x 2.0, WRITE_SIZE x 1.0): 2.0 * 262157.8 KiB + 262144.1 KiB for Add.
-TRAFFIC_BYTES = {"Add": int((2.0 * 262157.8 + 262144.1) * 1024)}
+# HBM bytes per launch of the dominant kernel are not measured by this program: they come from two rocprofv3 --pmc runs of it
+# (FETCH_SIZE, WRITE_SIZE), whose committed summary carries a line "traffic_bytes_per_launch <op> <bytes>".
+TRAFFIC_PROFILE = os.path.join("profiles", "bench_headline_fp32_8192x8192.txt")
+
+
+def profiled_traffic(op_name):
+    """(bytes, source file) of the committed counter summary for `op_name`, or (None, None) when there is none."""
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == op_name:
+                    return int(parts[2]), TRAFFIC_PROFILE
+    except OSError:
+        pass
+    return None, None
 
 
 def log(*a):
@@ -185,10 +202,14 @@ def run_cpu(repeats=1):
     return total_bytes / t_total / 1e9, H.get_threads(), per
 
 
-def run_extra(lib_mod):
-    """--all: the other benchmark configurations, reported on stderr (they are parity-test cases, not the headline)."""
+def run_configs(everything):
+    """The other benchmark configurations (not the headline): per-call lines and per-configuration sums."""
     import bench_configs
-    bench_configs.run_all(log)
+    if everything:
+        res = bench_configs.run_all(log, (1, 2, 3, 4, 5, 6, 7))
+    else:
+        res = bench_configs.run_all(log, (1, 2, 3, 4, 5), fp32_folds=False, reference_dot_shapes=False)
+    return res, bench_configs.summarise([r for r in res if r["cfg"] <= 5])
 
 
 def main():
@@ -196,7 +217,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--all", action="store_true", help="also time the other configurations (stderr)")
+    ap.add_argument("--no-configs", action="store_true", help="skip the per-configuration lines (`configs` in the JSON)")
+    ap.add_argument("--all", action="store_true", help="configurations: also the fp32 folds again, the reference's square products, "
+                                                       "the vector forms of dot and host transfers")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -218,8 +241,9 @@ def main():
     dop = ops[dom_i]
     dom_ms = float(np.mean(dop.timed_ms))
     dom_gbs = dop.bytes / (dom_ms * 1e-3) / 1e9
+    traffic, traffic_src = profiled_traffic(dop.name)
     roofline = {"bound": "hbm", "kernel": dop.kernel, "op": dop.name, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": TRAFFIC_BYTES.get(dop.name),
+                "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_src,
                 "avg_launch_ms": round(dom_ms, 5), "algorithmic_bytes": dop.bytes}
     ev_sum = sum(k["avg_ms"] for k in per_kernel)
     log(f"[bench] step: {ms_per_step:.3f} ms wall, {ev_sum:.3f} ms sum of event intervals, {value:.1f} GB/s = {100 * value / HBM_PEAK_GBS:.1f}% of HBM peak")
@@ -233,8 +257,7 @@ def main():
         for k, t in per.items():
             log(f"[bench] cpu {k:24s} {t * 1e3:9.1f} ms")
 
-    if args.all:
-        run_extra(None)
+    configs, config_summary = (None, None) if args.no_configs else run_configs(args.all)
 
     print(json.dumps({
         "metric": "achieved HBM GB/s for fp32 elementwise + axis-reduce at 64M elems",
@@ -245,6 +268,7 @@ def main():
                                "inputs resident in HBM, targets preallocated, seed 123",
                    "bytes_per_step": total_bytes, "device": info.name.decode() or info.arch.decode()},
         "roofline": roofline, "cpu_baseline": cpu, "per_kernel": per_kernel,
+        "config_summary": config_summary, "configs": configs,
     }))
 
 

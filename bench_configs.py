@@ -1,4 +1,4 @@
-"""Per-configuration timings of the HIP backend (used by `bench.py --all`): the five synthetic workloads of the
+"""Per-configuration timings of the HIP backend (used by `bench.py`, which puts them into its JSON line): the five synthetic workloads of the
 benchmark definition, one line per backend call with its algorithmic bytes (or FLOPs), HIP-event time and fraction of
 the roofline that bounds it.  Inputs come from seed 123; an op whose working set is below ~600 MB is launched over
 several independent buffer sets in rotation so that the 256 MB Infinity Cache cannot serve re-reads."""
@@ -49,17 +49,37 @@ def nsets_for(nbytes):
 
 
 def report(log, cfg, name, ms, nbytes=None, flops=None, fp64=False):
+    """One line of the per-configuration table: `frac` is the fraction of the roofline that bounds the call (8 TB/s of HBM for
+    algorithmic bytes, or the fp32 / fp64 matrix peak for a product's FLOPs)."""
     if flops:
         tf = flops / (ms * 1e-3) / 1e12
         peak = FP64_MFMA_PEAK_TFLOPS if fp64 else FP32_MFMA_PEAK_TFLOPS
         log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {tf:8.2f} TFLOP/s  {100 * tf / peak:5.1f}% of {'fp64' if fp64 else 'fp32'} MFMA peak")
-        return {"cfg": cfg, "op": name, "ms": ms, "TFLOPs": tf, "frac": tf / peak}
+        return {"cfg": cfg, "op": name, "us": round(ms * 1e3, 2), "flops": int(flops), "TFLOPs": round(tf, 2), "bound": "mfma", "frac": round(tf / peak, 4)}
     gb = nbytes / (ms * 1e-3) / 1e9
     log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {gb:8.1f} GB/s  {100 * gb / HBM_PEAK_GBS:5.1f}% of HBM peak  ({nbytes / 1e6:.1f} MB)")
-    return {"cfg": cfg, "op": name, "ms": ms, "GBps": gb, "frac": gb / HBM_PEAK_GBS}
+    return {"cfg": cfg, "op": name, "us": round(ms * 1e3, 2), "bytes": int(nbytes), "GBps": round(gb, 1), "bound": "hbm", "frac": round(gb / HBM_PEAK_GBS, 4)}
 
 
-def run_all(log, which=(1, 2, 3, 4, 5, 6)):
+def summarise(results):
+    """Per configuration: sum of algorithmic bytes over sum of time of its memory-bound calls (the composite lines — the eager
+    chain, which repeats the six calls above it — are left out), and the lowest fraction among all of its calls."""
+    out = []
+    for cfg in sorted({r["cfg"] for r in results}):
+        rows = [r for r in results if r["cfg"] == cfg and "frac" in r]
+        mem = [r for r in rows if r.get("bound") == "hbm" and not r.get("composite")]
+        entry = {"cfg": cfg, "calls": len(rows), "min_frac": min(r["frac"] for r in rows) if rows else None}
+        if mem:
+            gb = sum(r["bytes"] for r in mem) / sum(r["us"] for r in mem) / 1e3
+            entry.update({"hbm_bytes": sum(r["bytes"] for r in mem), "hbm_us": round(sum(r["us"] for r in mem), 1), "GBps": round(gb, 1),
+                          "frac": round(gb / HBM_PEAK_GBS, 4)})
+        out.append(entry)
+    return out
+
+
+def run_all(log, which=(1, 2, 3, 4, 5, 6), fp32_folds=True, reference_dot_shapes=True):
+    """fp32_folds=False leaves configuration 3's single-precision folds out (bench.py's headline step times those);
+    reference_dot_shapes=False leaves out the 1000 / 2000 / 4000 square products of the reference's own benchmark."""
     from deepnet_amd import abi, hip as G
     from deepnet_amd.backend import CAbiTensorBackend
     from deepnet_amd.tensor import Tensor
@@ -101,7 +121,7 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6)):
             ms = T.time([[s[k]] for s in sets], reps=20)
             results.append(report(log, 1, nm + " 4096x4096", ms, mult * N * 4))
         ms = T.time(sets, reps=12)
-        results.append(report(log, 1, "chain of 6 calls (eager)", ms, 14 * N * 4))
+        results.append(dict(report(log, 1, "chain of 6 calls (eager)", ms, 14 * N * 4), composite=True))
         keep.clear()
         del sets
 
@@ -125,6 +145,8 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6)):
         n = 8192
         N = n * n
         for dt, s in ((np.float32, 4), (np.float64, 8)):
+            if dt == np.float32 and not fp32_folds:
+                continue
             a = G.ofNumpy(rng.standard_normal((n, n)).astype(dt) if dt == np.float32 else rng.uniform(-1, 1, (n, n)))
             b = G.ofNumpy(G.toNumpy(a) * dt(0.5))
             srcs = [a, b]
@@ -236,7 +258,7 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6)):
             return [("binary", (abi.DNH_DIVIDE, D(c), D(a), D(sm[:, :, None].broadcastTo([Bn, n, n]))))]
         timed(5, "Divide e / rowsum (broadcast)", 2 * N * 4 + R * 4, div5)
         # the matrix sizes of the reference's own benchmark (Tensor.Benchmark/Benchmark.fs:216): few output tiles, K is split
-        for sq in (1000, 2000, 4000):
+        for sq in ((1000, 2000, 4000) if reference_dot_shapes else (4000,)):
             for dt, sz in ((np.float32, 4), (np.float64, 8)):
                 sa = G.ofNumpy(rng.standard_normal((sq, sq)).astype(dt))
                 sb = G.ofNumpy(rng.standard_normal((sq, sq)).astype(dt))
@@ -279,7 +301,7 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6)):
                     check(call())
                 ms = (time.perf_counter() - t0) / 5 * 1e3
                 log(f"[cfg7] {name} 256 MiB {kind:8s} host memory {ms:9.2f} ms  {nbytes / ms / 1e6:8.1f} GB/s")
-                results.append({"cfg": 7, "op": f"{name} {kind}", "ms": ms, "GBps": nbytes / ms / 1e6})
+                results.append({"cfg": 7, "op": f"{name} {kind}", "us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1)})
         check(lib.dnh_host_free(pinned))
     return results
 
