@@ -4,14 +4,17 @@
 //              flight per thread, one pass over HBM.
 //  map_nd    : collapsed n-d strided operands; lanes run along the target's fastest dimension (coalesced stores), 16-byte
 //              vectors when the last dimension allows it, per-item index decomposition in 32-bit arithmetic.
-//  map_tr    : a source whose unit-stride dimension differs from the target's is staged through LDS in 64x64 (32x32 for
-//              8-byte elements) tiles: global reads run along the source's fast dimension, global writes along the target's.
+//  map_tr    : a source whose unit-stride dimension differs from the target's is staged through LDS in 128x64 tiles (64x32 for
+//              8-byte elements, 256x128 for short target rows): global reads run along the source's fast dimension, global
+//              writes along the target's.
 //
 // An Op is a small functor: `using T/A/B/C` (target and source element types, `char` when absent), `NSRC`, and
 // `__device__ T operator()(A[,B[,C]]) const`.  State (a fill value) travels by value as a kernel argument.
 #pragma once
 
 #include "common.h"
+
+#include <type_traits>
 
 namespace dnh {
 
@@ -214,6 +217,7 @@ struct TrArgs {
     int64_t sa[kMaxOperands], sb[kMaxOperands];   // element strides along A and B
     int staged[kMaxOperands];                     // source k goes through LDS
     uint32_t lds_off[kMaxOperands];               // byte offset of source k's tile in dynamic LDS (staged sources only)
+    int dmode;                                    // sources that are not staged: 1 = all broadcast along B, 2 = all broadcast or in aligned vectors along B, 0 = other
 };
 
 // Direct (not LDS-staged) operand fetch of the transposing kernel for VEC consecutive positions tx.. along B at row r along A:
@@ -229,31 +233,63 @@ __device__ __forceinline__ Pack<X, VEC> tr_direct(const X* g, uint32_t r, uint32
     return v;
 }
 
-template <class Op, int TILE, int VEC>
+// Tile of TA elements along A (the staged sources' unit-stride dimension) by TB along B (the target's).  Workgroup ids walk the
+// tiles with B fastest, then A, then the outer dimensions; `xcd_chunk` (total / 8, or 0) re-numbers them so that each XCD takes a
+// contiguous range of that order.  MASK: bit k - 1 set = source k is staged through LDS (a compile-time choice: with run-time flags
+// the store loop is full of branches, and the compiler then waits for every store before it issues the next one).
+// The same fetch without a branch, for operands that are either broadcast along B (sb == 0) or run along B in aligned vectors
+// (sb == 1): one vector load (from the aligned vector that holds the element when broadcast) and one element load, then a select.
+// Branches around the loads of a loop make the compiler wait for each load before it issues the next.
+template <class X, int VEC>
+__device__ __forceinline__ Pack<X, VEC> tr_direct_fast(const X* g, uint32_t r, uint32_t tx, int64_t sa, int64_t sb) {
+    const X* q = g + (int64_t)r * sa + (int64_t)tx * sb;
+    if constexpr (VEC == 1) {
+        Pack<X, 1> v;
+        v.v[0] = *q;
+        return v;
+    } else {
+        const bool bcast = sb == 0;
+        const X* qv = bcast ? (const X*)((uintptr_t)q & ~(uintptr_t)(VEC * sizeof(X) - 1)) : q;
+        Pack<X, VEC> v = load_pack<X, VEC>(qv);
+        const X s = *q;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) v.v[e] = bcast ? s : v.v[e];
+        return v;
+    }
+}
+
+template <class Op, int TA, int TB, int VEC, int MASK>
 __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t, const typename Op::A* a, const typename Op::B* b,
-                                                        const typename Op::C* c, TrArgs p) {
+                                                        const typename Op::C* c, TrArgs p, uint32_t xcd_chunk) {
     using T = typename Op::T;
     using A = typename Op::A;
     using B = typename Op::B;
     using C = typename Op::C;
-    constexpr int TV = TILE / VEC;       // threads per tile row (each handles VEC consecutive elements)
-    constexpr int ROWS = kBlock / TV;    // tile rows covered per pass
-    constexpr int ITER = TILE / ROWS;    // passes
-    // only staged sources own an LDS tile ([TILE][TILE+1] elements each), so occupancy is not spent on unused tiles
+    constexpr bool S1 = (MASK & 1) != 0, S2 = (MASK & 2) != 0, S3 = (MASK & 4) != 0;
+    static_assert(MASK > 0 && MASK < (1 << Op::NSRC), "staged sources");
+    constexpr int TVA = TA / VEC;            // staging: threads per tile row along A
+    constexpr int ROWS_S = kBlock / TVA;     // rows (along B) staged per pass
+    constexpr int ITER_S = TB / ROWS_S;
+    constexpr int TVB = TB / VEC;            // storing: threads per tile row along B
+    constexpr int ROWS_T = kBlock / TVB;     // rows (along A) stored per pass
+    constexpr int ITER_T = TA / ROWS_T;
+    static_assert(TA % VEC == 0 && TB % VEC == 0 && kBlock % TVA == 0 && kBlock % TVB == 0 && TB % ROWS_S == 0 && TA % ROWS_T == 0, "tile shape");
+    // only staged sources own an LDS tile ([TB][TA+1] elements each), so occupancy is not spent on unused tiles
     extern __shared__ __align__(16) unsigned char tr_lds[];
-    typedef A (*TileA)[TILE + 1];
-    typedef B (*TileB)[TILE + 1];
-    typedef C (*TileC)[TILE + 1];
+    typedef A (*TileA)[TA + 1];
+    typedef B (*TileB)[TA + 1];
+    typedef C (*TileC)[TA + 1];
     TileA la = (TileA)(tr_lds + p.lds_off[1]);
     TileB lb = (TileB)(tr_lds + p.lds_off[2]);
     TileC lc = (TileC)(tr_lds + p.lds_off[3]);
 
     uint32_t bid = blockIdx.x;
+    if (xcd_chunk) bid = (bid % 8u) * xcd_chunk + bid / 8u;
     const uint32_t tb = bid % p.tiles_b;
     bid /= p.tiles_b;
     const uint32_t ta = bid % p.tiles_a;
     bid /= p.tiles_a;
-    const uint32_t a0 = ta * TILE, b0 = tb * TILE;
+    const uint32_t a0 = ta * TA, b0 = tb * TB;
     int64_t off[kMaxOperands];
 #pragma unroll
     for (int k = 0; k <= Op::NSRC; k++) off[k] = (int64_t)a0 * p.sa[k] + (int64_t)b0 * p.sb[k];
@@ -268,78 +304,129 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
     if constexpr (Op::NSRC >= 1) a += off[1];
     if constexpr (Op::NSRC >= 2) b += off[2];
     if constexpr (Op::NSRC >= 3) c += off[3];
-    const uint32_t tx = (threadIdx.x % TV) * VEC, ty = threadIdx.x / TV;
-    const uint32_t la_n = p.na - a0 < (uint32_t)TILE ? p.na - a0 : TILE;   // valid extent of this tile along A and B
-    const uint32_t lb_n = p.nb - b0 < (uint32_t)TILE ? p.nb - b0 : TILE;
+    const uint32_t la_n = p.na - a0 < (uint32_t)TA ? p.na - a0 : TA;   // valid extent of this tile along A and B
+    const uint32_t lb_n = p.nb - b0 < (uint32_t)TB ? p.nb - b0 : TB;
 
-    // stage: lanes run along A (the staged sources' unit-stride dimension); the LDS tile is [b][a]
-    if (tx < la_n) {
+    // stage: lanes run along A (the staged sources' unit-stride dimension); the LDS tile is [b][a].  All loads of a thread are
+    // issued back to back, before the first LDS store, so that they are in flight together: no branch separates them (positions
+    // outside an edge tile fetch element (0, 0) of the tile instead, and what they put into LDS is never read).
+    {
+        const uint32_t sx = (threadIdx.x % TVA) * VEC, sy = threadIdx.x / TVA;
+        const uint32_t sxc = sx < la_n ? sx : 0u;
+        Pack<A, VEC> ga[ITER_S];
+        Pack<B, VEC> gb[ITER_S];
+        Pack<C, VEC> gc[ITER_S];
 #pragma unroll
-        for (int it = 0; it < ITER; it++) {
-            const uint32_t r = ty + it * ROWS;
-            if (r < lb_n) {
+        for (int it = 0; it < ITER_S; it++) {
+            const uint32_t r = sy + it * ROWS_S;
+            const int64_t rc = r < lb_n ? (int64_t)r : 0;
+            if constexpr (Op::NSRC >= 1)
+                if constexpr (S1) ga[it] = load_pack<A, VEC>(a + rc * p.sb[1] + sxc);
+            if constexpr (Op::NSRC >= 2)
+                if constexpr (S2) gb[it] = load_pack<B, VEC>(b + rc * p.sb[2] + sxc);
+            if constexpr (Op::NSRC >= 3)
+                if constexpr (S3) gc[it] = load_pack<C, VEC>(c + rc * p.sb[3] + sxc);
+        }
+#pragma unroll
+        for (int it = 0; it < ITER_S; it++) {
+            const uint32_t r = sy + it * ROWS_S;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
                 if constexpr (Op::NSRC >= 1)
-                    if (p.staged[1]) {
-                        const Pack<A, VEC> v = load_pack<A, VEC>(a + (int64_t)r * p.sb[1] + tx);
-#pragma unroll
-                        for (int e = 0; e < VEC; e++) la[r][tx + e] = v.v[e];
-                    }
+                    if constexpr (S1) la[r][sx + e] = ga[it].v[e];
                 if constexpr (Op::NSRC >= 2)
-                    if (p.staged[2]) {
-                        const Pack<B, VEC> v = load_pack<B, VEC>(b + (int64_t)r * p.sb[2] + tx);
-#pragma unroll
-                        for (int e = 0; e < VEC; e++) lb[r][tx + e] = v.v[e];
-                    }
+                    if constexpr (S2) lb[r][sx + e] = gb[it].v[e];
                 if constexpr (Op::NSRC >= 3)
-                    if (p.staged[3]) {
-                        const Pack<C, VEC> v = load_pack<C, VEC>(c + (int64_t)r * p.sb[3] + tx);
-#pragma unroll
-                        for (int e = 0; e < VEC; e++) lc[r][tx + e] = v.v[e];
-                    }
+                    if constexpr (S3) lc[r][sx + e] = gc[it].v[e];
             }
         }
     }
-    // Operands that are not staged are read in the store pattern (lanes along B).  All of these loads are issued before
-    // the first store: on this architecture loads and stores retire through one in-order counter, so a load placed
-    // after a store would wait for that store to complete.
-    Pack<A, VEC> da[ITER];
-    Pack<B, VEC> db[ITER];
-    Pack<C, VEC> dc[ITER];
-    if (tx < lb_n) {
+    // Sources that are not staged and are broadcast along B (a bias along A, say) have one value per stored row: they are fetched
+    // here, ahead of the barrier, so that their latency is covered by the staging loads.
+    constexpr int NDIRECT = Op::NSRC - (int)S1 - (int)S2 - (int)S3;
+    [[maybe_unused]] A pa[ITER_T];
+    [[maybe_unused]] B pb[ITER_T];
+    [[maybe_unused]] C pc[ITER_T];
+    if constexpr (NDIRECT > 0 && VEC > 1) {
+        if (p.dmode == 1 && la_n == (uint32_t)TA && lb_n == (uint32_t)TB) {
+            const uint32_t ty0 = threadIdx.x / TVB;
 #pragma unroll
-        for (int it = 0; it < ITER; it++) {
-            const uint32_t r = ty + it * ROWS;
-            if (r < la_n) {
-                if constexpr (Op::NSRC >= 1)
-                    if (!p.staged[1]) da[it] = tr_direct<A, VEC>(a, r, tx, p.sa[1], p.sb[1]);
-                if constexpr (Op::NSRC >= 2)
-                    if (!p.staged[2]) db[it] = tr_direct<B, VEC>(b, r, tx, p.sa[2], p.sb[2]);
-                if constexpr (Op::NSRC >= 3)
-                    if (!p.staged[3]) dc[it] = tr_direct<C, VEC>(c, r, tx, p.sa[3], p.sb[3]);
+            for (int it = 0; it < ITER_T; it++) {
+                const uint32_t r = ty0 + it * ROWS_T;
+                const int64_t rc = r < la_n ? (int64_t)r : 0;
+                if constexpr (Op::NSRC >= 1 && !S1) pa[it] = a[rc * p.sa[1]];
+                if constexpr (Op::NSRC >= 2 && !S2) pb[it] = b[rc * p.sa[2]];
+                if constexpr (Op::NSRC >= 3 && !S3) pc[it] = c[rc * p.sa[3]];
             }
         }
     }
     __syncthreads();
-    // compute + store: lanes run along B (the target's unit-stride dimension), VEC consecutive elements per thread
-    if (tx < lb_n) {
+    // compute + store: lanes run along B (the target's unit-stride dimension), VEC consecutive elements per thread.  Operands that
+    // are not staged are read in the store pattern, a group of G rows at a time: the loads of a group are issued before its first
+    // store (loads and stores retire through one in-order counter on this architecture, so a load placed after a store waits for
+    // that store to complete; with one workgroup per CU, as for the large tile, nothing else would cover that wait).
+    constexpr int G = (NDIRECT <= 1 || ITER_T < 8) ? ITER_T : 8;   // one direct operand: all of its rows at once (at most 128 registers)
+    static_assert(ITER_T % G == 0, "tile shape");
+    const uint32_t tx = (threadIdx.x % TVB) * VEC, ty = threadIdx.x / TVB;
+    // FULL: the tile lies inside the tensor, so no row or column test is needed.  A test around each store is a divergent branch,
+    // and after such a branch the compiler waits for all outstanding memory operations, the previous store included.
+    auto store_phase = [&](auto mode_tag, auto full_tag) {
+        constexpr int MODE = decltype(mode_tag)::value;    // as TrArgs::dmode
+        constexpr bool FULL = decltype(full_tag)::value;
+#pragma unroll 1
+        for (int g0 = 0; g0 < ITER_T; g0 += G) {
+            Pack<A, VEC> da[G];
+            Pack<B, VEC> db[G];
+            Pack<C, VEC> dc[G];
+            if constexpr (MODE != 1) {
 #pragma unroll
-        for (int it = 0; it < ITER; it++) {
-            const uint32_t r = ty + it * ROWS;
-            if (r < la_n) {
-                Pack<T, VEC> res;
-#pragma unroll
-                for (int e = 0; e < VEC; e++) {
-                    A xa = A();
-                    B xb = B();
-                    C xc = C();
-                    if constexpr (Op::NSRC >= 1) xa = p.staged[1] ? la[tx + e][r] : da[it].v[e];
-                    if constexpr (Op::NSRC >= 2) xb = p.staged[2] ? lb[tx + e][r] : db[it].v[e];
-                    if constexpr (Op::NSRC >= 3) xc = p.staged[3] ? lc[tx + e][r] : dc[it].v[e];
-                    res.v[e] = apply_op(op, xa, xb, xc);
+                for (int i = 0; i < G; i++) {
+                    const uint32_t r = ty + (g0 + i) * ROWS_T;
+                    if constexpr (MODE == 2) {
+                        const uint32_t rc = (FULL || r < la_n) ? r : 0u;   // rows outside an edge tile fetch row 0, nothing of them is stored
+                        if constexpr (Op::NSRC >= 1 && !S1) da[i] = tr_direct_fast<A, VEC>(a, rc, tx, p.sa[1], p.sb[1]);
+                        if constexpr (Op::NSRC >= 2 && !S2) db[i] = tr_direct_fast<B, VEC>(b, rc, tx, p.sa[2], p.sb[2]);
+                        if constexpr (Op::NSRC >= 3 && !S3) dc[i] = tr_direct_fast<C, VEC>(c, rc, tx, p.sa[3], p.sb[3]);
+                    } else if (r < la_n) {
+                        if constexpr (Op::NSRC >= 1 && !S1) da[i] = tr_direct<A, VEC>(a, r, tx, p.sa[1], p.sb[1]);
+                        if constexpr (Op::NSRC >= 2 && !S2) db[i] = tr_direct<B, VEC>(b, r, tx, p.sa[2], p.sb[2]);
+                        if constexpr (Op::NSRC >= 3 && !S3) dc[i] = tr_direct<C, VEC>(c, r, tx, p.sa[3], p.sb[3]);
+                    }
                 }
-                store_pack<T, VEC>(t + (int64_t)r * p.sa[0] + tx, res);
+            }
+#pragma unroll
+            for (int i = 0; i < G; i++) {
+                const uint32_t r = ty + (g0 + i) * ROWS_T;
+                if (FULL || r < la_n) {
+                    Pack<T, VEC> res;
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) {
+                        A xa = A();
+                        B xb = B();
+                        C xc = C();
+                        if constexpr (Op::NSRC >= 1) xa = S1 ? la[tx + e][r] : (MODE == 1 ? pa[g0 + i] : da[i].v[e]);
+                        if constexpr (Op::NSRC >= 2) xb = S2 ? lb[tx + e][r] : (MODE == 1 ? pb[g0 + i] : db[i].v[e]);
+                        if constexpr (Op::NSRC >= 3) xc = S3 ? lc[tx + e][r] : (MODE == 1 ? pc[g0 + i] : dc[i].v[e]);
+                        res.v[e] = apply_op(op, xa, xb, xc);
+                    }
+                    store_pack<T, VEC>(t + (int64_t)r * p.sa[0] + tx, res);
+                }
             }
         }
+    };
+    using M0 = std::integral_constant<int, 0>;
+    using M1 = std::integral_constant<int, 1>;
+    using M2 = std::integral_constant<int, 2>;
+    // (the element-wise instantiation fetches single elements through any strides without a branch: mode 2 for every layout; tiles
+    // on the tensor's edge take the general path whatever the mode, which keeps the number of copies of this loop down)
+    const bool full = la_n == (uint32_t)TA && lb_n == (uint32_t)TB;
+    if constexpr (NDIRECT == 0 || VEC == 1) {
+        if (full) store_phase(M2{}, std::true_type{});
+        else if (tx < lb_n) store_phase(M2{}, std::false_type{});
+    } else {
+        if (full && p.dmode == 1) store_phase(M1{}, std::true_type{});
+        else if (full && p.dmode == 2) store_phase(M2{}, std::true_type{});
+        else if (tx < lb_n) store_phase(M0{}, std::false_type{});
     }
 }
 
@@ -424,14 +511,20 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 if (p.stride[k][d] == 1 && p.shape[d] >= 16) { dA = d; break; }
         }
         if (dA >= 0 && p.shape[last] >= 16) {
-            constexpr int TILE = (sizeof(T) > 4 || (Op::NSRC >= 1 && sizeof(A) > 4) || (Op::NSRC >= 2 && sizeof(B) > 4) ||
-                                  (Op::NSRC >= 3 && sizeof(C) > 4)) ? 32 : 64;
+            // Tile shapes (elements along A x along B), chosen from measurements of 512 MiB transposing copies on MI355X:
+            //   4-byte and narrower elements: 128 x 64 (512-byte row pieces on the read side, 256-byte on the write side; 72 % of
+            //   the HBM peak for both 256 x 524288 and 131072 x 1024 sources, against 71 % and 55 % with 64 x 64);
+            //   when the target's rows are short (at most 256 elements) and one source is staged, 256 x 128 tiles (one workgroup per
+            //   CU with 128 KB of LDS, all of a thread's 32 loads in flight): 77 % for the 256 x 524288 case;
+            //   8-byte elements: 64 x 32.
+            constexpr bool WIDE = sizeof(T) > 4 || (Op::NSRC >= 1 && sizeof(A) > 4) || (Op::NSRC >= 2 && sizeof(B) > 4) ||
+                                  (Op::NSRC >= 3 && sizeof(C) > 4);
+            constexpr int TA = WIDE ? 64 : 128, TB = WIDE ? 32 : 64;
+            constexpr int BIG_TA = 256, BIG_TB = 128;
             TrArgs q;
             memset(&q, 0, sizeof(q));
             q.na = (uint32_t)p.shape[dA];
             q.nb = (uint32_t)p.shape[last];
-            q.tiles_a = cdiv(q.na, TILE);
-            q.tiles_b = cdiv(q.nb, TILE);
             int64_t outer = 1;
             for (int d = 0; d < last; d++) {
                 if (d == dA) continue;
@@ -440,18 +533,14 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 outer *= p.shape[d];
                 q.nouter++;
             }
+            int nstaged = 0;
+            size_t staged_esize = 0;
             for (int k = 0; k < NOPS; k++) {
                 q.sa[k] = p.stride[k][dA];
                 q.sb[k] = p.stride[k][last];
                 q.staged[k] = (k >= 1 && p.stride[k][dA] == 1 && p.stride[k][last] != 0 && p.stride[k][last] != 1) ? 1 : 0;
+                if (q.staged[k]) { nstaged++; staged_esize = es[k]; }
             }
-            uint32_t lds_bytes = 0;
-            for (int k = 1; k < NOPS; k++) {
-                if (!q.staged[k]) continue;
-                q.lds_off[k] = lds_bytes;
-                lds_bytes += (uint32_t)((TILE * (TILE + 1) * es[k] + 15) / 16 * 16);
-            }
-            const int64_t blocks = (int64_t)q.tiles_a * q.tiles_b * outer;
             // vector path: every tile row a whole number of aligned vectors for the target and every staged source
             bool vec = VEC > 1 && (q.na % VEC) == 0 && (q.nb % VEC) == 0 && aligned_to(t, VEC * es[0]) && (q.sa[0] % VEC) == 0;
             for (int d = 0; d < q.nouter && vec; d++) vec = (q.ostride[0][d] % VEC) == 0;
@@ -460,9 +549,81 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 vec = aligned_to(p.ptr[k], VEC * es[k]) && (q.sb[k] % VEC) == 0;
                 for (int d = 0; d < q.nouter && vec; d++) vec = (q.ostride[k][d] % VEC) == 0;
             }
+            // sources that are not staged: all broadcast along B, or each broadcast or in aligned vectors along B, lets the kernel fetch
+            // them without branches
+            q.dmode = 1;
+            for (int k = 1; k < NOPS; k++) {
+                if (q.staged[k] || q.sb[k] == 0) continue;
+                if (q.dmode == 1) q.dmode = 2;
+                if (!vec) continue;   // the element-wise kernel fetches single elements either way
+                bool ok = q.sb[k] == 1 && aligned_to(p.ptr[k], VEC * es[k]) && (q.sa[k] % VEC) == 0;
+                for (int d = 0; d < q.nouter && ok; d++) ok = (q.ostride[k][d] % VEC) == 0;
+                if (!ok) q.dmode = 0;
+            }
+            bool big = false;
+            if constexpr (!WIDE && VEC == 4 && Op::NSRC >= 1 && Op::NSRC <= 2) {
+                big = vec && nstaged == 1 && staged_esize == 4 && q.nb <= 256 && (q.na % BIG_TA) == 0 && (q.nb % BIG_TB) == 0 &&
+                      (int64_t)(q.na / BIG_TA) * (q.nb / BIG_TB) * outer >= (int64_t)device_cus() * 8;
+            }
+            const int ta_n = big ? BIG_TA : TA, tb_n = big ? BIG_TB : TB;
+            q.tiles_a = cdiv(q.na, ta_n);
+            q.tiles_b = cdiv(q.nb, tb_n);
+            uint32_t lds_bytes = 0;
+            for (int k = 1; k < NOPS; k++) {
+                if (!q.staged[k]) continue;
+                q.lds_off[k] = lds_bytes;
+                lds_bytes += (uint32_t)(((size_t)tb_n * (ta_n + 1) * es[k] + 15) / 16 * 16);
+            }
+            const int64_t blocks = (int64_t)q.tiles_a * q.tiles_b * outer;
             if (blocks <= 0x7FFFFFFF) {
-                if (vec) hipLaunchKernelGGL((map_tr_kernel<Op, TILE, (VEC < TILE ? VEC : 1)>), dim3((unsigned)blocks), dim3(kBlock), lds_bytes, stream, op, t, a, b, c, q);
-                else hipLaunchKernelGGL((map_tr_kernel<Op, TILE, 1>), dim3((unsigned)blocks), dim3(kBlock), lds_bytes, stream, op, t, a, b, c, q);
+                const uint32_t xcd_chunk = (!big && blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
+                const int mask = (q.staged[1] ? 1 : 0) | (q.staged[2] ? 2 : 0) | (q.staged[3] ? 4 : 0);
+                int32_t st = DNH_ERR_NOT_SUPPORTED;
+                // launches map_tr_kernel<Op, TA_, TB_, V_, M_>; more than 64 KB of LDS (two or three staged sources, or the large tile)
+                // have to be asked for once per kernel
+#define DNH_TR_LAUNCH(TA_, TB_, V_, M_)                                                                                                   \
+    do {                                                                                                                                  \
+        auto kern = map_tr_kernel<Op, TA_, TB_, V_, M_>;                                                                                  \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize,                 \
+                                                          3 * (TB_ * (TA_ + 1) * (WIDE ? 8 : 4) + 16) > 160 * 1024 ? 160 * 1024           \
+                                                                                                               : 3 * (TB_ * (TA_ + 1) * (WIDE ? 8 : 4) + 16)); \
+        if (attr != hipSuccess) { st = fail(DNH_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(attr)); break; }                    \
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBlock), lds_bytes, stream, op, t, a, b, c, q, xcd_chunk);                   \
+        st = DNH_OK;                                                                                                                      \
+    } while (0)
+#define DNH_TR_MASKS(TA_, TB_, V_)                                                                       \
+    do {                                                                                                 \
+        if constexpr (Op::NSRC == 1) { DNH_TR_LAUNCH(TA_, TB_, V_, 1); }                                 \
+        else if constexpr (Op::NSRC == 2) {                                                              \
+            if (mask == 1) DNH_TR_LAUNCH(TA_, TB_, V_, 1);                                               \
+            else if (mask == 2) DNH_TR_LAUNCH(TA_, TB_, V_, 2);                                          \
+            else DNH_TR_LAUNCH(TA_, TB_, V_, 3);                                                         \
+        } else if constexpr (Op::NSRC == 3) {                                                            \
+            switch (mask) {                                                                              \
+                case 1: DNH_TR_LAUNCH(TA_, TB_, V_, 1); break;                                           \
+                case 2: DNH_TR_LAUNCH(TA_, TB_, V_, 2); break;                                           \
+                case 3: DNH_TR_LAUNCH(TA_, TB_, V_, 3); break;                                           \
+                case 4: DNH_TR_LAUNCH(TA_, TB_, V_, 4); break;                                           \
+                case 5: DNH_TR_LAUNCH(TA_, TB_, V_, 5); break;                                           \
+                case 6: DNH_TR_LAUNCH(TA_, TB_, V_, 6); break;                                           \
+                default: DNH_TR_LAUNCH(TA_, TB_, V_, 7); break;                                          \
+            }                                                                                            \
+        }                                                                                                \
+    } while (0)
+                if (big) {
+                    if constexpr (!WIDE && VEC == 4 && Op::NSRC >= 1 && Op::NSRC <= 2) {
+                        if constexpr (Op::NSRC == 1) DNH_TR_LAUNCH(BIG_TA, BIG_TB, 4, 1);
+                        else if (mask == 1) DNH_TR_LAUNCH(BIG_TA, BIG_TB, 4, 1);
+                        else DNH_TR_LAUNCH(BIG_TA, BIG_TB, 4, 2);
+                    }
+                } else if (vec) {
+                    DNH_TR_MASKS(TA, TB, VEC);
+                } else {
+                    DNH_TR_MASKS(TA, TB, 1);
+                }
+#undef DNH_TR_MASKS
+#undef DNH_TR_LAUNCH
+                DNH_TRY(st);
                 DNH_LAUNCH_CHECK();
                 return DNH_OK;
             }
