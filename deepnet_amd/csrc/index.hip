@@ -183,6 +183,273 @@ __device__ __forceinline__ uint32_t block_exclusive_scan(uint32_t c, uint32_t* t
     return base + inc - c;
 }
 
+// ---- binned scatter ------------------------------------------------------------------------------------------------------------
+// t[idx[i]] += s[i] for 32-bit integers, every tensor rank 1 with unit stride, many updates into a large table.  A random update
+// costs the memory system a 32-byte read-modify-write at the memory side (device-scope atomics do not run in the per-XCD L2):
+// 4 Mi of them into a 64 MB table take 166 us.  Here the (index, value) pairs are first sorted by bucket of kBinElems consecutive
+// target elements, then one workgroup per bucket sums its pairs in LDS and adds the bucket to the table in one coalesced pass, so
+// the table is read and written once, in whole lines:
+//   1. bin_count:   each workgroup counts its kBinChunk pairs per bucket (LDS histogram)            -> counts[workgroup][bucket]
+//   2. bin_colscan: exclusive prefix of every bucket's column of counts, and the bucket totals       -> counts (in place), totals[bucket]
+//   3. bin_move:    each workgroup ranks its pairs by bucket in LDS and writes them out in runs      -> pairs (bucket order)
+//   4. bin_apply:   one workgroup per bucket: LDS accumulate (integer adds commute: bit-exact and deterministic), then table += sums
+// An index outside the table sets the error word and is skipped, as in the direct kernel.
+constexpr int kBinShift = 14;
+constexpr uint32_t kBinElems = 1u << kBinShift;          // target elements per bucket: 64 KB of LDS
+constexpr uint32_t kBinChunk = 8192;                      // pairs per workgroup of passes 1 and 3
+constexpr uint32_t kBinMaxBuckets = 4096;                 // LDS histogram of passes 1 and 3
+constexpr int kBinThreads = 1024;                         // passes 1, 3 and 4: many wavefronts per workgroup cover the latency of their few, dependent steps
+constexpr int kBinPerThread = kBinChunk / kBinThreads;
+
+// exclusive prefix of `c` over a workgroup of kBinThreads threads; `total` receives the sum.  `wave_sum`: kBinThreads / 64 words of LDS,
+// free for reuse after the call's second barrier.
+__device__ __forceinline__ uint32_t bin_block_scan(uint32_t c, uint32_t* total, uint32_t* wave_sum) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint32_t inc = c;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const uint32_t y = (uint32_t)__shfl_up((int)inc, d, 64);
+        if (lane >= d) inc += y;
+    }
+    if (lane == 63) wave_sum[wave] = inc;
+    __syncthreads();
+    uint32_t base = 0, tot = 0;
+#pragma unroll
+    for (int w = 0; w < kBinThreads / 64; w++) {
+        const uint32_t x = wave_sum[w];
+        if (w < wave) base += x;
+        tot += x;
+    }
+    __syncthreads();
+    *total = tot;
+    return base + inc - c;
+}
+
+__global__ __launch_bounds__(kBinThreads) void bin_count_kernel(const int64_t* __restrict__ idx, uint32_t m, int64_t n, uint32_t nb, uint32_t nchunks,
+                                                                uint32_t* __restrict__ counts, int32_t* err) {
+    extern __shared__ uint32_t bin_lds[];   // nb counters
+    uint32_t* hist = bin_lds;
+    for (uint32_t b = threadIdx.x; b < nb; b += kBinThreads) hist[b] = 0;
+    const uint32_t i0 = blockIdx.x * kBinChunk;
+    bool bad = false;
+    int64_t jj[kBinPerThread];   // every load is issued before the first LDS atomic: a load inside the loop would wait for the one before it
+#pragma unroll
+    for (int e = 0; e < kBinPerThread; e++) {
+        const uint32_t i = i0 + e * kBinThreads + threadIdx.x;
+        jj[e] = i < m ? __builtin_nontemporal_load(idx + i) : 0;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < kBinPerThread; e++) {
+        const uint32_t i = i0 + e * kBinThreads + threadIdx.x;
+        if (i < m) {
+            if (jj[e] >= 0 && jj[e] < n) atomicAdd(&hist[(uint32_t)(jj[e] >> kBinShift)], 1u);
+            else bad = true;
+        }
+    }
+    if (bad) *err = 1;
+    __syncthreads();
+    for (uint32_t b = threadIdx.x; b < nb; b += kBinThreads) counts[(size_t)blockIdx.x * nb + b] = hist[b];
+}
+
+// counts is [workgroup of pass 1][bucket] (rows written and read whole); this pass replaces every column by its exclusive prefix
+// and leaves the column sums in totals.  A workgroup owns 64 adjacent buckets: lanes run along the buckets (256-byte row pieces),
+// the 16 wavefronts split a tile of 512 rows, 32 rows each (all loads of a tile in flight together), and the tiles follow one another with a running carry per bucket.
+__global__ __launch_bounds__(kBinThreads) void bin_colscan_kernel(uint32_t* __restrict__ counts, uint32_t* __restrict__ totals, uint32_t nb, uint32_t nchunks) {
+    constexpr int GROUPS = kBinThreads / 64, ROWS = 32;
+    __shared__ uint32_t gsum[GROUPS][64];
+    const uint32_t lane = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const uint32_t b = blockIdx.x * 64 + lane;
+    const bool live = b < nb;
+    uint32_t carry = 0;
+    for (uint32_t k0 = 0; k0 < nchunks; k0 += GROUPS * ROWS) {
+        uint32_t c[ROWS], sum = 0;
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            const uint32_t k = k0 + g * ROWS + r;
+            c[r] = (live && k < nchunks) ? counts[(size_t)k * nb + b] : 0u;
+        }
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) sum += c[r];
+        gsum[g][lane] = sum;
+        __syncthreads();
+        uint32_t run = carry, all = 0;
+#pragma unroll
+        for (int w = 0; w < GROUPS; w++) {
+            const uint32_t x = gsum[w][lane];
+            if (w < (int)g) run += x;
+            all += x;
+        }
+        carry += all;
+#pragma unroll
+        for (int r = 0; r < ROWS; r++) {
+            const uint32_t k = k0 + g * ROWS + r;
+            if (live && k < nchunks) counts[(size_t)k * nb + b] = run;
+            run += c[r];
+        }
+        __syncthreads();
+    }
+    if (live && g == 0) totals[b] = carry;
+}
+
+__global__ __launch_bounds__(kBinThreads) void bin_move_kernel(const int64_t* __restrict__ idx, const uint32_t* __restrict__ src, uint32_t m, int64_t n,
+                                                               uint32_t nb, uint32_t nchunks, const uint32_t* __restrict__ counts,
+                                                               const uint32_t* __restrict__ totals, uint2* __restrict__ pairs) {
+    constexpr int PER = kBinMaxBuckets / kBinThreads;   // buckets per thread in the two prefix sums
+    __shared__ uint2 sorted[kBinChunk];           // (index into the table, value), grouped by bucket; the index holds bucket and offset
+    __shared__ uint32_t wave_sum[kBinThreads / 64];
+    extern __shared__ uint32_t bin_lds[];         // 2 * nb words, sized by the launch so that two workgroups fit a CU for tables up to 64 MB
+    uint32_t* cursor = bin_lds;                   // next free slot of each bucket's group in `sorted`
+    uint32_t* gbase = bin_lds + nb;               // where this workgroup's run of each bucket starts in `pairs`, minus the group's start in `sorted`
+    for (uint32_t b = threadIdx.x; b < nb; b += kBinThreads) cursor[b] = 0;
+    // everything this workgroup reads from memory is requested here, before the first dependent step
+    const uint32_t i0 = blockIdx.x * kBinChunk;
+    int64_t jj[kBinPerThread];
+    uint32_t sv[kBinPerThread], tot[PER], off[PER];
+#pragma unroll
+    for (int e = 0; e < kBinPerThread; e++) {
+        const uint32_t i = i0 + e * kBinThreads + threadIdx.x;
+        jj[e] = i < m ? __builtin_nontemporal_load(idx + i) : -1;
+        sv[e] = i < m ? __builtin_nontemporal_load(src + i) : 0u;
+    }
+#pragma unroll
+    for (int e = 0; e < PER; e++) {
+        const uint32_t b = threadIdx.x * PER + e;
+        tot[e] = b < nb ? totals[b] : 0u;
+        off[e] = b < nb ? counts[(size_t)blockIdx.x * nb + b] : 0u;
+    }
+    __syncthreads();
+    // group sizes (recounting is cheaper than keeping the histograms of pass 1)
+#pragma unroll
+    for (int e = 0; e < kBinPerThread; e++) {
+        if (jj[e] >= n) jj[e] = -1;
+        if (jj[e] >= 0) atomicAdd(&cursor[(uint32_t)(jj[e] >> kBinShift)], 1u);
+    }
+    __syncthreads();
+    // group starts inside `sorted`, and each bucket's start in `pairs`
+    {
+        uint32_t v[PER], sum = 0, tsum = 0, total;
+#pragma unroll
+        for (int e = 0; e < PER; e++) {
+            const uint32_t b = threadIdx.x * PER + e;
+            v[e] = b < nb ? cursor[b] : 0u;
+            sum += v[e];
+            tsum += tot[e];
+        }
+        uint32_t run = bin_block_scan(sum, &total, wave_sum);
+        uint32_t trun = bin_block_scan(tsum, &total, wave_sum);
+#pragma unroll
+        for (int e = 0; e < PER; e++) {
+            const uint32_t b = threadIdx.x * PER + e;
+            if (b < nb) {
+                cursor[b] = run;
+                gbase[b] = trun + off[e] - run;
+            }
+            run += v[e];
+            trun += tot[e];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < kBinPerThread; e++) {
+        if (jj[e] >= 0) {
+            const uint32_t slot = atomicAdd(&cursor[(uint32_t)(jj[e] >> kBinShift)], 1u);
+            sorted[slot] = make_uint2((uint32_t)jj[e], sv[e]);   // table index < 2^32 here
+        }
+    }
+    __syncthreads();
+    const uint32_t valid = cursor[nb - 1];   // every group has moved up by its size: the last cursor is the number of valid pairs
+    for (uint32_t sI = threadIdx.x; sI < valid; sI += kBinThreads) {
+        const uint2 pr = sorted[sI];
+        pairs[gbase[pr.x >> kBinShift] + sI] = pr;
+    }
+}
+
+__global__ __launch_bounds__(kBinThreads) void bin_apply_kernel(uint32_t* __restrict__ t, int64_t n, uint32_t nb, const uint32_t* __restrict__ totals,
+                                                                const uint2* __restrict__ pairs) {
+    __shared__ uint32_t acc[kBinElems];
+    __shared__ uint32_t wave_sum[kBinThreads / 64];
+    const uint32_t b = blockIdx.x;
+    const uint32_t cnt = totals[b];
+    if (cnt == 0) return;               // uniform: nothing lands in this bucket
+    // the bucket's slice of the table is fetched first (whole buckets: 4 vectors per thread), so that its latency is covered by
+    // everything else the workgroup does
+    const int64_t e0 = (int64_t)b << kBinShift;
+    const uint32_t len = (uint32_t)((n - e0) < (int64_t)kBinElems ? (n - e0) : (int64_t)kBinElems);
+    uint32_t* tp = t + e0;
+    const bool whole = len == kBinElems && (((uintptr_t)tp) & 15) == 0;
+    constexpr int NV = kBinElems / 4 / kBinThreads;
+    Pack<uint32_t, 4> v[NV];
+    if (whole) {
+#pragma unroll
+        for (int k = 0; k < NV; k++) v[k] = load_pack<uint32_t, 4>(tp + (k * kBinThreads + threadIdx.x) * 4u);
+    }
+    // where the bucket's pairs start: the sum of the totals before it
+    uint32_t before = 0;
+    for (uint32_t i = threadIdx.x; i < b; i += kBinThreads) before += totals[i];
+    for (uint32_t i = threadIdx.x * 4u; i < kBinElems; i += kBinThreads * 4u) *reinterpret_cast<uint4*>(&acc[i]) = make_uint4(0, 0, 0, 0);
+    uint32_t p0;
+    (void)bin_block_scan(before, &p0, wave_sum);   // its barriers also publish the cleared accumulators
+    constexpr int U = 4;   // loads in flight per thread
+    for (uint32_t i0 = 0; i0 < cnt; i0 += kBinThreads * U) {
+        uint2 pr[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t i = i0 + u * kBinThreads + threadIdx.x;
+            const Pack<uint32_t, 2> w = load_pack<uint32_t, 2>(reinterpret_cast<const uint32_t*>(pairs + p0 + (i < cnt ? i : 0u)));
+            pr[u] = make_uint2(w.v[0], w.v[1]);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const uint32_t i = i0 + u * kBinThreads + threadIdx.x;
+            if (i < cnt) atomicAdd(&acc[pr[u].x & (kBinElems - 1u)], pr[u].y);
+        }
+    }
+    __syncthreads();
+    if (whole) {
+#pragma unroll
+        for (int k = 0; k < NV; k++) {
+            const uint32_t i = (k * kBinThreads + threadIdx.x) * 4u;
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[k].v[e] += acc[i + e];
+            store_pack<uint32_t, 4>(tp + i, v[k]);
+        }
+    } else {
+        for (uint32_t i = threadIdx.x; i < len; i += kBinThreads) tp[i] += acc[i];
+    }
+}
+
+// Takes the call when it has the binned form's shape and the binned form is the cheaper one; *status then holds its result.
+bool try_scatter_binned(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, hipStream_t stream, int32_t* err,
+                        int32_t* status) {
+    if (t->dtype != DNH_I32 && t->dtype != DNH_U32) return false;
+    if (t->ndims != 1 || src->ndims != 1 || n_idx != 1 || !idx[0] || idx[0]->ndims != 1) return false;
+    if (t->stride[0] != 1 || src->stride[0] != 1 || idx[0]->stride[0] != 1) return false;
+    const int64_t n = t->shape[0], m = src->shape[0];
+    if (m < (1 << 20) || m > 0x7FFFFFFFLL || n < 1 || n > ((int64_t)kBinMaxBuckets << kBinShift)) return false;
+    // cost model (measured on MI355X): a direct update costs about 40 ps (memory-side read-modify-write); the binned form moves the
+    // table twice and the pairs four and a half times at about 5.5 TB/s, plus three more launches
+    const double direct_us = (double)m * 40e-6, binned_us = ((double)n * 8.0 + (double)m * 36.0) / 5.5e6 + 10.0;
+    if (binned_us >= direct_us) return false;
+    const uint32_t nb = (uint32_t)((n + kBinElems - 1) >> kBinShift), nchunks = cdiv(m, kBinChunk);
+    const size_t counts_bytes = ((size_t)nb * nchunks * 4 + 255) / 256 * 256, totals_bytes = ((size_t)nb * 4 + 255) / 256 * 256;
+    char* ws = nullptr;
+    WorkspaceLease lease;
+    *status = workspace(stream, counts_bytes + totals_bytes + (size_t)m * 8, (void**)&ws, lease);
+    if (*status != DNH_OK) return true;
+    uint32_t* counts = (uint32_t*)ws;
+    uint32_t* totals = (uint32_t*)(ws + counts_bytes);
+    uint2* pairs = (uint2*)(ws + counts_bytes + totals_bytes);
+    const int64_t* ip = (const int64_t*)elem_ptr(idx[0]);
+    hipLaunchKernelGGL(bin_count_kernel, dim3(nchunks), dim3(kBinThreads), nb * 4, stream, ip, (uint32_t)m, n, nb, nchunks, counts, err);
+    hipLaunchKernelGGL(bin_colscan_kernel, dim3(cdiv(nb, 64)), dim3(kBinThreads), 0, stream, counts, totals, nb, nchunks);
+    hipLaunchKernelGGL(bin_move_kernel, dim3(nchunks), dim3(kBinThreads), nb * 8, stream, ip, (const uint32_t*)elem_ptr(src), (uint32_t)m, n, nb, nchunks,
+                       (const uint32_t*)counts, (const uint32_t*)totals, pairs);
+    hipLaunchKernelGGL(bin_apply_kernel, dim3(nb), dim3(kBinThreads), 0, stream, (uint32_t*)elem_ptr(t), n, nb, (const uint32_t*)totals, (const uint2*)pairs);
+    *status = hipGetLastError() == hipSuccess ? DNH_OK : fail(DNH_ERR_HIP, "binned scatter: launch failed");
+    return true;
+}
+
 __global__ __launch_bounds__(kBlock) void compact_count_kernel(MaskArgs m, uint32_t n, uint32_t* counts) {
     const uint32_t i0 = blockIdx.x * (uint32_t)kChunk + threadIdx.x * kItems;
     uint32_t c = 0;
@@ -595,6 +862,8 @@ extern "C" int32_t dnh_scatter(const DnhTensor* t, const DnhTensor* const* idx, 
     hipStream_t s = (hipStream_t)stream;
     int32_t* eflag = nullptr;
     DNH_TRY(error_flag_ptr(s, &eflag));
+    int32_t bst = DNH_OK;
+    if (try_scatter_binned(t, idx, n_idx, src, s, eflag, &bst)) return bst;
     const dim3 grid(cdiv(n, kBlock));
 #define CASE(DT, X) case DT: hipLaunchKernelGGL(scatter_kernel<X>, grid, dim3(kBlock), 0, s, (X*)elem_ptr(t), (const X*)elem_ptr(src), a, (uint32_t)n, eflag); break;
     switch (t->dtype) {

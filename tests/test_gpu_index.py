@@ -64,6 +64,55 @@ def test_scatter_fp_unique(H, G, rng, dt):
     assert_exact(ref, got)
 
 
+@pytest.mark.parametrize("dt", [np.int32, np.uint32])
+@pytest.mark.parametrize("m,n,kind", [
+    ((1 << 20) + 123, 300_000, "dup"),         # many updates per element; table not a whole number of buckets
+    ((1 << 21), (1 << 22) + 5, "unique"),      # the benchmark's form at a quarter of its size, ragged table
+    ((1 << 20) + 1, 16384, "dup"),             # one bucket
+    ((1 << 20) + 7, 1, "dup"),                 # one element
+    (3 << 20, 5_000_000, "skewed"),            # most updates land in a few buckets, many buckets stay empty
+])
+def test_scatter_many_updates_binned(H, G, rng, dt, m, n, kind):
+    """Large scatters of 32-bit integers are sorted by bucket of the table and summed per bucket (a different kernel sequence
+    from the direct one): bit-exact against the oracle's sequential loop and against np.add.at, sums wrapping."""
+    if kind == "unique":
+        idx = rng.permutation(n)[:m].astype(np.int64)
+    elif kind == "skewed":
+        idx = np.where(rng.random(m) < 0.9, rng.integers(0, 40_000, m), rng.integers(0, n, m)).astype(np.int64)
+    else:
+        idx = rng.integers(0, n, m).astype(np.int64)
+    src = rng.integers(0, 2 ** 31 - 1, m).astype(dt)            # large values: sums wrap
+    ref, got = both(H, G, lambda s, i: type(s).scatter([i], [n], s), src, idx)
+    assert_exact(ref, got)
+    exp = np.zeros(n, dtype=dt)
+    np.add.at(exp, idx, src)
+    assert_exact(exp, got)
+
+
+def test_scatter_many_updates_adds_to_the_target_and_reports_bad_indices(G, rng):
+    m, n = (1 << 20) + 5, 200_001
+    idx = rng.integers(0, n, m).astype(np.int64)
+    src = rng.integers(-1000, 1000, m).astype(np.int32)
+    before = rng.integers(-5, 5, n + 3).astype(np.int32)
+    t = G.ofNumpy(before)
+    view = t[3:]                                                  # a target that is not 16-byte aligned, holding values already
+    view.Backend.Scatter(view, [G.ofNumpy(idx)], G.ofNumpy(src))
+    exp = before.copy()
+    np.add.at(exp[3:], idx, src)
+    assert_exact(exp, G.toNumpy(t))
+    # indices outside the table: reported, skipped, everything else still lands
+    bad = idx.copy()
+    bad[[5, 70_000, m - 1]] = [n, -1, 2 ** 40]
+    t2 = G.zeros([n], np.int32)
+    with pytest.raises(IndexError):
+        t2.Backend.Scatter(t2, [G.ofNumpy(bad)], G.ofNumpy(src))
+    keep = np.ones(m, bool)
+    keep[[5, 70_000, m - 1]] = False
+    exp2 = np.zeros(n, np.int32)
+    np.add.at(exp2, idx[keep], src[keep])
+    assert_exact(exp2, G.toNumpy(t2))
+
+
 def test_scatter_doc_vector(H, G):
     # Guide-Index.md:118-133: first row summed into [0,3]; rows 1 and 2 swapped; row 3 stays zero
     src = np.array([[0.0, 0.1, 0.2, 0.3], [1.0, 1.1, 1.2, 1.3], [2.0, 2.1, 2.2, 2.3]])
