@@ -90,7 +90,9 @@ __device__ __forceinline__ typename Op::T apply_op(const Op& op, typename Op::A 
 constexpr uint32_t kXcdRun = 64;
 
 template <class Op, int VEC, int UNROLL>
-__global__ __launch_bounds__(kBlock) void map_flat_kernel(Op op, typename Op::T* __restrict__ t, const typename Op::A* a,
+// The target may be one of the sources (in-place ops such as FillMultiply a a b): no pointer is declared restrict, and a thread
+// reads everything it needs of an element before it writes that element.
+__global__ __launch_bounds__(kBlock) void map_flat_kernel(Op op, typename Op::T* t, const typename Op::A* a,
                                                           const typename Op::B* b, const typename Op::C* c, int sa, int sb, int sc,
                                                           int64_t n) {
     using T = typename Op::T;

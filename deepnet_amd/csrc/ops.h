@@ -171,9 +171,36 @@ template <class W> struct OpFill {
     W value;
     __device__ W operator()() const { return value; }
 };
+// ITensorBackend.Convert is an unchecked Expression.Convert (Tensor/Tensor/ScalarPrimitives.fs:50-52).  Integer -> integer wraps,
+// integer -> float rounds to nearest, float -> float rounds (overflow to infinity): the plain casts.  A float that does not fit the
+// integer target is left unspecified by the CLI standard; what the reference's runtime (64-bit x86) does is restated here, since a
+// plain cast saturates on this GPU:
+//   -> int32 / int64: truncate toward zero; NaN and values outside the range give the minimum value (the cvtt* instructions);
+//   -> int8 / uint8: as int32, then the low 8 bits;   -> uint32: as int64, then the low 32 bits;
+//   -> uint64: below 2^63 as int64 (negative values wrap), from 2^63 on (and NaN) int64(x - 2^63) + 2^63, wrapping.
+template <class F> __device__ __forceinline__ int32_t fp_to_i32(F x) {
+    return (x >= (F)-2147483648.0 && x < (F)2147483648.0) ? (int32_t)x : INT32_MIN;
+}
+template <class F> __device__ __forceinline__ int64_t fp_to_i64(F x) {
+    return (x >= (F)-9223372036854775808.0 && x < (F)9223372036854775808.0) ? (int64_t)x : INT64_MIN;
+}
 template <class TT, class TA> struct OpConvert {
     using T = TT; using A = TA; using B = char; using C = char; static constexpr int NSRC = 1;
-    __device__ TT operator()(TA a) const { return (TT)a; }
+    __device__ TT operator()(TA a) const {
+        if constexpr (kIsFp<TA> && !kIsFp<TT>) {
+            if constexpr (std::is_same<TT, int32_t>::value) return fp_to_i32(a);
+            else if constexpr (std::is_same<TT, int64_t>::value) return fp_to_i64(a);
+            else if constexpr (sizeof(TT) == 1) return (TT)(uint32_t)fp_to_i32(a);
+            else if constexpr (std::is_same<TT, uint32_t>::value) return (uint32_t)(uint64_t)fp_to_i64(a);
+            else {
+                static_assert(std::is_same<TT, uint64_t>::value, "integer target");
+                if (a < (TA)9223372036854775808.0) return (uint64_t)fp_to_i64(a);
+                return (uint64_t)fp_to_i64(a - (TA)9223372036854775808.0) + 0x8000000000000000ull;
+            }
+        } else {
+            return (TT)a;
+        }
+    }
 };
 template <class TA> struct OpToBool {
     using T = uint8_t; using A = TA; using B = char; using C = char; static constexpr int NSRC = 1;

@@ -49,6 +49,9 @@ size_t pool_round(size_t bytes) {
     return (bytes + g - 1) / g * g;
 }
 
+std::mutex g_dead_mu;
+std::vector<hipStream_t> g_dead_streams;   // handles destroyed by dnh_stream_destroy (a later dnh_stream_create may get one again)
+
 // caller holds g_pool.mu
 int32_t pool_trim_locked() {
     if (g_pool.cached_bytes == 0) return DNH_OK;
@@ -57,6 +60,26 @@ int32_t pool_trim_locked() {
         for (auto& blk : per_stream.second) (void)hipFree(blk.second);
     g_pool.free_blocks.clear();
     g_pool.cached_bytes = 0;
+    return DNH_OK;
+}
+// hipMalloc that gives the block cache back to the driver and tries once more when the driver is out of memory (the cache is
+// unbounded by default and may hold most of the device's memory).  Caller does not hold g_pool.mu.
+int32_t device_malloc(void** out, size_t bytes, const char* what) {
+    hipError_t e = hipMalloc(out, bytes);
+    if (e == hipErrorOutOfMemory) {
+        (void)hipGetLastError();
+        {
+            std::lock_guard<std::mutex> lock(g_pool.mu);
+            DNH_TRY(pool_trim_locked());
+        }
+        e = hipMalloc(out, bytes);
+    }
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        *out = nullptr;
+        if (e == hipErrorOutOfMemory) return fail(DNH_ERR_OUT_OF_MEMORY, "%s: device memory allocation of %zu MB failed", what, bytes >> 20);
+        return fail(DNH_ERR_HIP, "%s: hipMalloc(%zu): %s", what, bytes, hipGetErrorString(e));
+    }
     return DNH_OK;
 }
 }  // namespace
@@ -102,7 +125,7 @@ int32_t error_flag_ptr(hipStream_t stream, int32_t** out) {
     std::lock_guard<std::mutex> lock(g_mu);
     int32_t*& p = g_error_flags[stream];
     if (!p) {
-        DNH_HIP(hipMalloc((void**)&p, sizeof(int32_t)));
+        DNH_TRY(device_malloc((void**)&p, sizeof(int32_t), "index error word"));
         DNH_HIP(hipMemset(p, 0, sizeof(int32_t)));   // synchronous: done before any kernel that may set it is queued
     }
     *out = p;
@@ -129,7 +152,7 @@ int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& 
             w->bytes = 0;
         }
         size_t want = bytes < (size_t)(4 << 20) ? (size_t)(4 << 20) : bytes + bytes / 2;
-        DNH_HIP(hipMalloc(&w->ptr, want));
+        if (device_malloc(&w->ptr, want, "workspace") != DNH_OK) DNH_TRY(device_malloc(&w->ptr, want = bytes, "workspace"));   // without the head room
         w->bytes = want;
     }
     *out = w->ptr;
@@ -208,8 +231,7 @@ int32_t dnh_alloc(size_t bytes, void** out) {
     if (!out) return fail(DNH_ERR_INVALID_ARG, "dnh_alloc: null argument");
     DNH_TRY(ensure_init());
     *out = nullptr;
-    DNH_HIP(hipMalloc(out, bytes ? bytes : 1));
-    return DNH_OK;
+    return device_malloc(out, bytes ? bytes : 1, "dnh_alloc");
 }
 
 int32_t dnh_free(void* ptr) {
@@ -278,7 +300,15 @@ int32_t dnh_free_async(void* ptr, void* stream) {
             g_pool.live.erase(it);
             g_pool.live_bytes -= bytes;
             if (g_pool.limit_bytes == 0 || g_pool.cached_bytes + bytes <= g_pool.limit_bytes) {
-                g_pool.free_blocks[(hipStream_t)stream].emplace(bytes, ptr);
+                // a stream that dnh_stream_destroy has already retired (a finalizer running late): everything queued on it has
+                // finished, so the block is free for anyone and goes to the default stream's list instead of a dead one
+                hipStream_t owner = (hipStream_t)stream;
+                {
+                    std::lock_guard<std::mutex> dl(g_dead_mu);
+                    for (hipStream_t d : g_dead_streams)
+                        if (d == owner) owner = nullptr;
+                }
+                g_pool.free_blocks[owner].emplace(bytes, ptr);
                 g_pool.cached_bytes += bytes;
                 return DNH_OK;
             }
@@ -461,6 +491,11 @@ int32_t dnh_stream_create(void** stream) {
     DNH_TRY(ensure_init());
     hipStream_t s;
     DNH_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    {
+        std::lock_guard<std::mutex> dl(g_dead_mu);   // the driver may hand out a retired handle again
+        for (size_t i = 0; i < g_dead_streams.size(); i++)
+            if (g_dead_streams[i] == s) { g_dead_streams.erase(g_dead_streams.begin() + i); break; }
+    }
     *stream = (void*)s;
     return DNH_OK;
 }
@@ -482,6 +517,10 @@ int32_t dnh_stream_destroy(void* stream) {
         }
     }
     DNH_HIP(hipStreamDestroy((hipStream_t)stream));
+    {
+        std::lock_guard<std::mutex> dl(g_dead_mu);
+        g_dead_streams.push_back((hipStream_t)stream);
+    }
     return DNH_OK;
 }
 

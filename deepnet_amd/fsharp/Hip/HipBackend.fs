@@ -40,29 +40,58 @@ module internal Desc =
         d.Offset <- layout.Offset
         d.NDims <- layout.NDims
         d.DType <- int (dtypeOf dataType)
-        d.Shape <- Array.zeroCreate 8
-        d.Stride <- Array.zeroCreate 8
-        layout.Shape |> List.iteri (fun i s -> d.Shape.[i] <- s)
-        layout.Stride |> List.iteri (fun i s -> d.Stride.[i] <- s)
+        layout.Shape |> List.iteri (fun i s -> d.SetShape (i, s))
+        layout.Stride |> List.iteri (fun i s -> d.SetStride (i, s))
         d
+
+    /// Calls f with the address of one host element holding `value`.  bool crosses as one byte 0/1 (a bool[] is not blittable
+    /// and cannot be pinned); every other element type is pinned as a one-element array.
+    let withScalar (value: 'T) (f: nativeint -> unit) =
+        let arr : Array =
+            if typeof<'T> = typeof<bool> then [| (if (box value :?> bool) then 1uy else 0uy) |] :> Array
+            else [| value |] :> Array
+        let h = GCHandle.Alloc (arr, GCHandleType.Pinned)
+        try f (h.AddrOfPinnedObject ()) finally h.Free ()
+
+    /// Reads one element back: `f` receives the address of a one-element buffer to fill.
+    let readScalar<'T> (f: nativeint -> unit) : 'T =
+        if typeof<'T> = typeof<bool> then
+            let v = [| 0uy |]
+            let h = GCHandle.Alloc (v, GCHandleType.Pinned)
+            try f (h.AddrOfPinnedObject ()) finally h.Free ()
+            box (v.[0] <> 0uy) :?> 'T
+        else
+            let v = [| Unchecked.defaultof<'T> |]
+            let h = GCHandle.Alloc (v, GCHandleType.Pinned)
+            try f (h.AddrOfPinnedObject ()) finally h.Free ()
+            v.[0]
 
 /// Device memory owned by one tensor storage (CudaBackend.fs:54-93).
 /// The block comes from the library's stream-ordered cache under the stream current at creation.  While every use was
 /// issued on that stream the finalizer hands it back without waiting for the device (the finalizer runs after the last
 /// operation on the storage was queued, whichever thread it runs on); otherwise it uses the synchronising free.
-type TensorHipStorage<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> ValueType> (nElems: int64) =
+/// A storage made from an existing device pointer (HipTensor.usingPtr) references that memory and never frees it.
+type TensorHipStorage<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> ValueType> private (nElems: int64, external: nativeint) =
     let bytes = unativeint (max nElems 1L) * unativeint sizeof<'T>
     let stream = Cfg.Stream
+    let owned = external = IntPtr.Zero
     let mutable singleStream = true
-    let mutable ptr = IntPtr.Zero
-    do Native.check (Native.dnh_alloc_async (bytes, stream, &ptr))
+    let mutable ptr = external
+    do if owned then Native.check (Native.dnh_alloc_async (bytes, stream, &ptr))
+
+    /// allocates nElems elements on the device
+    new (nElems: int64) = TensorHipStorage<'T> (nElems, IntPtr.Zero)
+    /// references nElems elements of existing device memory; the caller keeps ownership
+    static member OfPointer (devPtr: nativeint, nElems: int64) =
+        if devPtr = IntPtr.Zero then invalidArg "devPtr" "null device pointer"
+        TensorHipStorage<'T> (nElems, devPtr)
 
     member this.Ptr =
         if Cfg.Stream <> stream then singleStream <- false
         ptr
     member this.NElems = nElems
     override this.Finalize () =
-        if ptr <> IntPtr.Zero then
+        if owned && ptr <> IntPtr.Zero then
             (if singleStream then Native.dnh_free_async (ptr, stream) else Native.dnh_free ptr) |> ignore
 
     interface ITensorStorage<'T> with
@@ -76,31 +105,53 @@ and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> Valu
         let st = t.Storage :?> TensorHipStorage<'A>
         Desc.make st.Ptr typeof<'A> t.Layout
 
+    // Every helper ends with GC.KeepAlive of the tensors it was given: `desc` copies the raw device pointer out of the storage, and
+    // without a later use of the storage object its finalizer could release the block while the native call is still running.
     static let unary op (trgt: ITensorFrontend<'R>) (a: ITensorFrontend<'A>) =
-        let mutable t, a = desc trgt, desc a
-        Native.check (Native.dnh_unary (op, &t, &a, Cfg.Stream))
+        let mutable t, ad = desc trgt, desc a
+        Native.check (Native.dnh_unary (op, &t, &ad, Cfg.Stream))
+        GC.KeepAlive trgt; GC.KeepAlive a
     static let binary op (trgt: ITensorFrontend<'R>) (a: ITensorFrontend<'A>) (b: ITensorFrontend<'A>) =
-        let mutable t, a, b = desc trgt, desc a, desc b
-        Native.check (Native.dnh_binary (op, &t, &a, &b, Cfg.Stream))
+        let mutable t, ad, bd = desc trgt, desc a, desc b
+        Native.check (Native.dnh_binary (op, &t, &ad, &bd, Cfg.Stream))
+        GC.KeepAlive trgt; GC.KeepAlive a; GC.KeepAlive b
     static let compare op (trgt: ITensorFrontend<bool>) (a: ITensorFrontend<'A>) (b: ITensorFrontend<'A>) =
-        let mutable t, a, b = desc trgt, desc a, desc b
-        Native.check (Native.dnh_compare (op, &t, &a, &b, Cfg.Stream))
+        let mutable t, ad, bd = desc trgt, desc a, desc b
+        Native.check (Native.dnh_compare (op, &t, &ad, &bd, Cfg.Stream))
+        GC.KeepAlive trgt; GC.KeepAlive a; GC.KeepAlive b
     static let reduce op (trgt: ITensorFrontend<'R>) (src: ITensorFrontend<'A>) =
-        let mutable t, s = desc trgt, desc src
-        Native.check (Native.dnh_reduce_last_axis (op, &t, &s, Cfg.Stream))
+        let mutable t, sd = desc trgt, desc src
+        Native.check (Native.dnh_reduce_last_axis (op, &t, &sd, Cfg.Stream))
+        GC.KeepAlive trgt; GC.KeepAlive src
     static let argReduce op (trgt: ITensorFrontend<int64>) (src: ITensorFrontend<'A>) =
-        let mutable t, s = desc trgt, desc src
-        Native.check (Native.dnh_arg_reduce_last_axis (op, &t, &s, Cfg.Stream))
+        let mutable t, sd = desc trgt, desc src
+        Native.check (Native.dnh_arg_reduce_last_axis (op, &t, &sd, Cfg.Stream))
+        GC.KeepAlive trgt; GC.KeepAlive src
     static let dot (trgt: ITensorFrontend<'T>) (a: ITensorFrontend<'T>) (b: ITensorFrontend<'T>) =
-        let mutable t, a, b = desc trgt, desc a, desc b
-        Native.check (Native.dnh_dot (&t, &a, &b, Cfg.Stream))
+        let mutable t, ad, bd = desc trgt, desc a, desc b
+        Native.check (Native.dnh_dot (&t, &ad, &bd, Cfg.Stream))
+        GC.KeepAlive trgt; GC.KeepAlive a; GC.KeepAlive b
 
-    /// pins optional descriptors and calls f with the array of their addresses (IntPtr.Zero for None)
+    /// Copies optional descriptors into unmanaged memory and calls f with the array of their addresses (IntPtr.Zero for None);
+    /// the library copies the descriptors before it returns.
     static let withDescs (ts: ITensorFrontend<'A> option list) (f: nativeint[] -> unit) =
-        let descs = ts |> List.map (Option.map desc)
-        let handles = descs |> List.map (Option.map (fun d -> GCHandle.Alloc (box d, GCHandleType.Pinned)))
-        try f (handles |> List.map (function Some h -> h.AddrOfPinnedObject () | None -> IntPtr.Zero) |> Array.ofList)
-        finally handles |> List.iter (Option.iter (fun h -> h.Free ()))
+        let size = Marshal.SizeOf (typeof<DnhTensor>)
+        let n = List.length ts
+        let block = Marshal.AllocHGlobal (max 1 (size * n))
+        try
+            let ptrs =
+                ts |> List.mapi (fun i t ->
+                    match t with
+                    | Some t ->
+                        let p = block + nativeint (i * size)
+                        Marshal.StructureToPtr (desc t, p, false)
+                        p
+                    | None -> IntPtr.Zero)
+                |> Array.ofList
+            f ptrs
+        finally
+            Marshal.FreeHGlobal block
+            ts |> List.iter (Option.iter (fun t -> GC.KeepAlive t))
 
     static let checkIndexError () =
         if Cfg.Stacktrace then
@@ -113,35 +164,34 @@ and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> Valu
     interface ITensorBackend<'T> with
         member this.Item
             with get idx =                                              // CudaBackend.fs:77-87: synchronous 1-element copy
-                let v = [| Unchecked.defaultof<'T> |]
-                let h = GCHandle.Alloc (v, GCHandleType.Pinned)
-                try Native.check (Native.dnh_memcpy_d2h (h.AddrOfPinnedObject (), itemAddr idx, unativeint sizeof<'T>, Cfg.Stream, 1))
-                finally h.Free ()
-                v.[0]
+                let v = Desc.readScalar<'T> (fun p -> Native.check (Native.dnh_memcpy_d2h (p, itemAddr idx, unativeint sizeof<'T>, Cfg.Stream, 1)))
+                GC.KeepAlive storage
+                v
             and set idx value =
-                let v = [| value |]
-                let h = GCHandle.Alloc (v, GCHandleType.Pinned)
-                try Native.check (Native.dnh_memcpy_h2d (itemAddr idx, h.AddrOfPinnedObject (), unativeint sizeof<'T>, Cfg.Stream, 1))
-                finally h.Free ()
+                Desc.withScalar value (fun p -> Native.check (Native.dnh_memcpy_h2d (itemAddr idx, p, unativeint sizeof<'T>, Cfg.Stream, 1)))
+                GC.KeepAlive storage
 
         member this.Copy (trgt, src) =
             let mutable t, s = desc trgt, desc src
             Native.check (Native.dnh_copy (&t, &s, Cfg.Stream))
+            GC.KeepAlive trgt; GC.KeepAlive src
         member this.Convert (trgt: ITensorFrontend<'T>, src: ITensorFrontend<'S>) =
             let mutable t, s = desc trgt, desc src
             Native.check (Native.dnh_convert (&t, &s, Cfg.Stream))
+            GC.KeepAlive trgt; GC.KeepAlive src
         member this.Transfer (trgt, src) = HipTransfer.transfer (trgt, src)   // host <-> device, as CudaBackend.fs:206-270
         member this.FillConst (value, trgt) =
             let mutable t = desc trgt
-            let h = GCHandle.Alloc ([| value |], GCHandleType.Pinned)
-            try Native.check (Native.dnh_fill_const (&t, h.AddrOfPinnedObject (), Cfg.Stream)) finally h.Free ()
-        member this.FillIncrementing (start, incr, trgt) =
+            Desc.withScalar value (fun p -> Native.check (Native.dnh_fill_const (&t, p, Cfg.Stream)))
+            GC.KeepAlive trgt
+        member this.FillIncrementing (start, incr, trgt) =               // numeric element types only, so the array is blittable
             let mutable t = desc trgt
             let h = GCHandle.Alloc ([| start; incr |], GCHandleType.Pinned)
             try
                 let p = h.AddrOfPinnedObject ()
                 Native.check (Native.dnh_fill_incrementing (&t, p, p + nativeint sizeof<'T>, Cfg.Stream))
             finally h.Free ()
+            GC.KeepAlive trgt
 
         member this.UnaryPlus (t, a) = unary 0 t a
         member this.UnaryMinus (t, a) = unary 1 t a
@@ -165,9 +215,10 @@ and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> Valu
         member this.Round (t, a) = unary 19 t a
         member this.Truncate (t, a) = unary 20 t a
         member this.Negate (t, a) = unary 21 t a
-        member this.IsFinite (trgt, a) =
-            let mutable t, a = desc trgt, desc a
+        member this.IsFinite (trgt, src) =
+            let mutable t, a = desc trgt, desc src
             Native.check (Native.dnh_is_finite (&t, &a, Cfg.Stream))
+            GC.KeepAlive trgt; GC.KeepAlive src
 
         member this.Add (t, a, b) = binary 0 t a b
         member this.Subtract (t, a, b) = binary 1 t a b
@@ -191,24 +242,30 @@ and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> Valu
         member this.IfThenElse (trgt, cond, ifTrue, ifFalse) =
             let mutable t, c, a, b = desc trgt, desc cond, desc ifTrue, desc ifFalse
             Native.check (Native.dnh_if_then_else (&t, &c, &a, &b, Cfg.Stream))
+            GC.KeepAlive trgt; GC.KeepAlive cond; GC.KeepAlive ifTrue; GC.KeepAlive ifFalse
 
         member this.Gather (trgt, srcIdxs, src) =
             let mutable t, s = desc trgt, desc src
             withDescs srcIdxs (fun p -> Native.check (Native.dnh_gather (&t, p, p.Length, &s, Cfg.Stream)))
+            GC.KeepAlive trgt; GC.KeepAlive src
             checkIndexError ()
         member this.Scatter (trgt, trgtIdxs, src) =
             let mutable t, s = desc trgt, desc src
             withDescs trgtIdxs (fun p -> Native.check (Native.dnh_scatter (&t, p, p.Length, &s, Cfg.Stream)))
+            GC.KeepAlive trgt; GC.KeepAlive src
             checkIndexError ()
         member this.MaskedGet (trgt, src, masks) =
             let mutable t, s = desc trgt, desc src
             withDescs (List.ofArray masks) (fun p -> Native.check (Native.dnh_masked_get (&t, &s, p, p.Length, Cfg.Stream)))
+            GC.KeepAlive trgt; GC.KeepAlive src
         member this.MaskedSet (trgt, masks, src) =
             let mutable t, s = desc trgt, desc src
             withDescs (List.ofArray masks) (fun p -> Native.check (Native.dnh_masked_set (&t, p, p.Length, &s, Cfg.Stream)))
+            GC.KeepAlive trgt; GC.KeepAlive src
         member this.TrueIndices (trgt, src) =
             let mutable t, s = desc trgt, desc src
             Native.check (Native.dnh_true_indices (&t, &s, Cfg.Stream))
+            GC.KeepAlive trgt; GC.KeepAlive src
 
         member this.SumLastAxis (t, s) = reduce 0 t s
         member this.ProductLastAxis (t, s) = reduce 1 t s
@@ -221,8 +278,8 @@ and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> Valu
         member this.ArgMaxLastAxis (t, s) = argReduce 1 t s
         member this.FindLastAxis (value, trgt, src) =
             let mutable t, s = desc trgt, desc src
-            let h = GCHandle.Alloc ([| value |], GCHandleType.Pinned)
-            try Native.check (Native.dnh_find_last_axis (h.AddrOfPinnedObject (), &t, &s, Cfg.Stream)) finally h.Free ()
+            Desc.withScalar value (fun p -> Native.check (Native.dnh_find_last_axis (p, &t, &s, Cfg.Stream)))
+            GC.KeepAlive trgt; GC.KeepAlive src
 
         member this.VecVecDot (t, a, b) = dot t a b
         member this.MatVecDot (t, a, b) = dot t a b
@@ -233,6 +290,7 @@ and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> Valu
         member this.BatchedInvert (trgt, src) =
             let mutable t, s = desc trgt, desc src
             Native.check (Native.dnh_batched_invert (&t, &s, Cfg.Stream))
+            GC.KeepAlive trgt; GC.KeepAlive src
         member this.BatchedSVD (trgtS, trgtUV, src) =
             let mutable s, a = desc trgtS, desc src
             match trgtUV with
@@ -241,10 +299,12 @@ and TensorHipBackend<'T when 'T: (new: unit -> 'T) and 'T: struct and 'T :> Valu
                 Native.check (Native.dnh_batched_svd (&s, &u, &v, &a, Cfg.Stream))
             | None ->
                 Native.check (Native.dnh_batched_svd_values (&s, IntPtr.Zero, IntPtr.Zero, &a, Cfg.Stream))
+            GC.KeepAlive trgtS; GC.KeepAlive trgtUV; GC.KeepAlive src
         member this.SymmetricEigenDecomposition (part, eigVals, eigVecs, src) =
             let mutable w, v, a = desc eigVals, desc eigVecs, desc src
             let part = match part with | MatrixPart.Upper -> 0 | MatrixPart.Lower -> 1
             Native.check (Native.dnh_symmetric_eig (part, &w, &v, &a, Cfg.Stream))
+            GC.KeepAlive eigVals; GC.KeepAlive eigVecs; GC.KeepAlive src
 
 /// Host <-> device copies: the source is made row-major first, a non-row-major target goes through a device temporary
 /// (CudaBackend.fs:206-270).  Returns false for pairs this backend does not handle so the frontend can try the other side
@@ -283,7 +343,8 @@ and internal HipTransfer =
 /// The device (CudaBackend.fs:497-507): new storage is uninitialised, so Zeroed = false and `zeros` launches FillConst.
 and TensorHipDevice private () =
     inherit BaseTensorDevice ()
-    static member Instance = TensorHipDevice ()
+    static let instance = TensorHipDevice ()
+    static member Instance = instance
     override this.Id = "Hip"
     override this.Create nElems = TensorHipStorage<'T> nElems :> ITensorStorage<'T>
     override this.Zeroed = false

@@ -23,17 +23,42 @@ type internal Status =
 type internal DType =
     | Bool = 0 | U8 = 1 | I8 = 2 | I32 = 3 | U32 = 4 | I64 = 5 | U64 = 6 | F32 = 7 | F64 = 8
 
-/// DnhTensor: blittable descriptor passed by reference (replaces the Reflection.Emit structs of Cuda/NativeTensor.fs:96-208).
+/// DnhTensor: descriptor passed by reference (replaces the Reflection.Emit structs of Cuda/NativeTensor.fs:96-208).
+/// Blittable: the two extents arrays of the C struct are spelled out as sixteen int64 fields (a managed int64[] marked ByValArray
+/// would make the struct non-blittable: it could not be pinned, and `byref` marshalling would copy it on every call).
 [<Struct; StructLayout(LayoutKind.Sequential)>]
 type internal DnhTensor =
     val mutable Base:   nativeint
     val mutable Offset: int64
     val mutable NDims:  int32
     val mutable DType:  int32
-    [<MarshalAs(UnmanagedType.ByValArray, SizeConst=8)>]
-    val mutable Shape:  int64[]
-    [<MarshalAs(UnmanagedType.ByValArray, SizeConst=8)>]
-    val mutable Stride: int64[]
+    val mutable Shape0: int64
+    val mutable Shape1: int64
+    val mutable Shape2: int64
+    val mutable Shape3: int64
+    val mutable Shape4: int64
+    val mutable Shape5: int64
+    val mutable Shape6: int64
+    val mutable Shape7: int64
+    val mutable Stride0: int64
+    val mutable Stride1: int64
+    val mutable Stride2: int64
+    val mutable Stride3: int64
+    val mutable Stride4: int64
+    val mutable Stride5: int64
+    val mutable Stride6: int64
+    val mutable Stride7: int64
+
+    member this.SetShape (i: int, v: int64) =
+        match i with
+        | 0 -> this.Shape0 <- v | 1 -> this.Shape1 <- v | 2 -> this.Shape2 <- v | 3 -> this.Shape3 <- v
+        | 4 -> this.Shape4 <- v | 5 -> this.Shape5 <- v | 6 -> this.Shape6 <- v | 7 -> this.Shape7 <- v
+        | _ -> invalidArg "i" "a descriptor holds at most 8 dimensions"
+    member this.SetStride (i: int, v: int64) =
+        match i with
+        | 0 -> this.Stride0 <- v | 1 -> this.Stride1 <- v | 2 -> this.Stride2 <- v | 3 -> this.Stride3 <- v
+        | 4 -> this.Stride4 <- v | 5 -> this.Stride5 <- v | 6 -> this.Stride6 <- v | 7 -> this.Stride7 <- v
+        | _ -> invalidArg "i" "a descriptor holds at most 8 dimensions"
 
 module internal Native =
     [<Literal>]

@@ -40,13 +40,17 @@ class TensorHipStorage(ITensorStorage):
     every operation on the storage is issued on that stream, release hands the block back to the cache without waiting
     for the device; once its pointer has been taken under another stream it is released with the synchronising free."""
 
-    def __init__(self, nElems: int, dtype, dev: "TensorHipDevice"):
+    def __init__(self, nElems: int, dtype, dev: "TensorHipDevice", external_ptr: int = 0):
         self.Dev = dev
         self.DataType = np.dtype(dtype)
         self.NElems = int(nElems)
         self._lib = native.load()
         self._stream = Cfg.Stream
         self._single_stream = True
+        self._owned = not external_ptr     # a storage made by usingPtr references memory it never frees
+        if external_ptr:
+            self._ptr = int(external_ptr)
+            return
         ptr = C.c_void_p()
         native.check(self._lib.dnh_alloc_async(max(self.NElems, 1) * self.DataType.itemsize, self._stream, C.byref(ptr)))
         self._ptr = ptr.value
@@ -66,7 +70,7 @@ class TensorHipStorage(ITensorStorage):
 
     def __del__(self):
         try:
-            if getattr(self, "_ptr", None):
+            if getattr(self, "_ptr", None) and getattr(self, "_owned", False):
                 if self._single_stream:
                     self._lib.dnh_free_async(self._ptr, self._stream)
                 else:
@@ -196,6 +200,21 @@ def filled(shape, value, dtype) -> Tensor: return Tensor.filled(shape, value, De
 def scalar(value, dtype) -> Tensor: return Tensor.scalar(value, Dev, dtype)
 def counting(n, dtype=np.int64) -> Tensor: return Tensor.counting(n, Dev, dtype)
 def transfer(t: Tensor) -> Tensor: return t.Transfer(Dev)
+
+
+def usingPtr(ptr: int, sizeInBytes: int, dtype, layout: TensorLayout) -> Tensor:
+    """A tensor over existing device memory (CudaTensor.usingPtr / usingPtrAndType, Cuda/CudaFrontend.fs:129-149): the data is
+    referenced, not copied, and never freed by the tensor."""
+    dt = np.dtype(dtype)
+    if not ptr:
+        raise ValueError("usingPtr: null device pointer")
+    nElems = int(sizeInBytes) // dt.itemsize
+    if layout.NElems:
+        lo = layout.Offset + sum((n - 1) * st for n, st in zip(layout.Shape, layout.Stride) if st < 0)
+        hi = layout.Offset + sum((n - 1) * st for n, st in zip(layout.Shape, layout.Stride) if st > 0)
+        if lo < 0 or hi >= nElems:
+            raise ValueError(f"usingPtr: the layout addresses elements {lo}..{hi} but the allocation holds {nElems}")
+    return Tensor(layout, TensorHipStorage(nElems, dt, Dev, external_ptr=int(ptr)))
 
 
 def synchronize():

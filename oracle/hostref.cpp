@@ -362,9 +362,33 @@ inline bool checked_addr(const Lay& l, const int64_t* pos, int64_t* out) {
     return true;
 }
 
+// Convert: the reference's unchecked Expression.Convert (ScalarPrimitives.fs:50-52).  For a float that does not fit an integer target
+// the CLI standard leaves the result unspecified; the rule below is what the reference's runtime does on 64-bit x86 (cvtt* sentinel =
+// the type's minimum for int32 / int64, narrower targets through int32, uint32 through int64, uint64 through the runtime's
+// 2^63 split), written out instead of relying on the C cast, whose out-of-range result is undefined.  Parity unpinned: no file of the
+// reference fixes these values; the tests check this function against vectors worked out from the rule by hand.
+template <class F> inline int32_t fp_to_i32(F x) { return (x >= (F)-2147483648.0 && x < (F)2147483648.0) ? (int32_t)x : INT32_MIN; }
+template <class F> inline int64_t fp_to_i64(F x) {
+    return (x >= (F)-9223372036854775808.0 && x < (F)9223372036854775808.0) ? (int64_t)x : INT64_MIN;
+}
+template <class TT, class TA> inline TT convert_elem(TA x) {
+    if constexpr (std::is_floating_point<TA>::value && !std::is_floating_point<TT>::value) {
+        if constexpr (std::is_same<TT, int32_t>::value) return fp_to_i32(x);
+        else if constexpr (std::is_same<TT, int64_t>::value) return fp_to_i64(x);
+        else if constexpr (sizeof(TT) == 1) return (TT)(uint32_t)fp_to_i32(x);
+        else if constexpr (std::is_same<TT, uint32_t>::value) return (uint32_t)(uint64_t)fp_to_i64(x);
+        else {
+            if (x < (TA)9223372036854775808.0) return (uint64_t)fp_to_i64(x);
+            return (uint64_t)fp_to_i64(x - (TA)9223372036854775808.0) + 0x8000000000000000ull;
+        }
+    } else {
+        return (TT)x;
+    }
+}
+
 template <class TT>
 int convert_from(const DnhTensor* t, const DnhTensor* a) {
-#define M(TA) return run_unary<TT, TA>(t, a, false, [](TA x) { return (TT)x; });
+#define M(TA) return run_unary<TT, TA>(t, a, false, [](TA x) { return convert_elem<TT, TA>(x); });
     switch (a->dtype) { HREF_ALL_CASES(M) default: return DNH_ERR_NOT_SUPPORTED; }
 #undef M
 }

@@ -121,3 +121,52 @@ def test_device_is_chosen_once(G):
     assert b"device" in buf.value
     x = G.ofNumpy(np.arange(6, dtype=np.int32))
     assert G.toNumpy(x + x).tolist() == [0, 2, 4, 6, 8, 10]
+
+
+def test_using_ptr_references_existing_device_memory(G):
+    """HipTensor.usingPtr (the reference's CudaTensor.usingPtr, Cuda/CudaFrontend.fs:129-149): a tensor over memory somebody else
+    owns; writes through it change the original data, and collecting it frees nothing."""
+    import ctypes as C
+    from deepnet_amd import layout as L
+    lib = native.load()
+    owner = G.ofNumpy(np.arange(24, dtype=np.float32))
+    ptr = owner.Storage.Pointer()
+    view = G.usingPtr(ptr, 24 * 4, np.float32, L.newC((4, 6)))
+    assert np.array_equal(G.toNumpy(view), np.arange(24, dtype=np.float32).reshape(4, 6))
+    view.Backend.Add(view, view, view)
+    assert np.array_equal(G.toNumpy(owner), 2 * np.arange(24, dtype=np.float32))
+    col = G.usingPtr(ptr, 24 * 4, np.float32, L.TensorLayout((4,), 1, (6,)))     # column 1 of the 4 x 6 matrix
+    assert np.array_equal(G.toNumpy(col), 2 * np.arange(24, dtype=np.float32).reshape(4, 6)[:, 1])
+    before = abi.DnhPoolStats()
+    native.check(lib.dnh_pool_stats(C.byref(before)))
+    del view, col
+    after = abi.DnhPoolStats()
+    native.check(lib.dnh_pool_stats(C.byref(after)))
+    assert (before.live_bytes, before.cached_bytes) == (after.live_bytes, after.cached_bytes)
+    assert np.array_equal(G.toNumpy(owner), 2 * np.arange(24, dtype=np.float32))
+    with pytest.raises(ValueError):
+        G.usingPtr(ptr, 24 * 4, np.float32, L.newC((5, 6)))                       # the layout does not fit the allocation
+    with pytest.raises(ValueError):
+        G.usingPtr(0, 24 * 4, np.float32, L.newC((4, 6)))
+
+
+def test_block_released_on_a_destroyed_stream_is_reused(G):
+    """A storage finalizer may run after its stream was destroyed: the block then goes to the default stream's list (everything
+    queued on the dead stream has finished) instead of being filed under a handle nobody will ask for again."""
+    import ctypes as C
+    lib = native.load()
+    st = C.c_void_p()
+    native.check(lib.dnh_stream_create(C.byref(st)))
+    p = C.c_void_p()
+    size = 3 * (1 << 20) + 4096                                   # an unusual size, so the hit below is this block
+    native.check(lib.dnh_alloc_async(size, st, C.byref(p)))
+    native.check(lib.dnh_stream_destroy(st))
+    native.check(lib.dnh_free_async(p, st))                       # late release, naming the dead stream
+    before = abi.DnhPoolStats()
+    native.check(lib.dnh_pool_stats(C.byref(before)))
+    q = C.c_void_p()
+    native.check(lib.dnh_alloc_async(size, None, C.byref(q)))     # default stream
+    after = abi.DnhPoolStats()
+    native.check(lib.dnh_pool_stats(C.byref(after)))
+    assert after.hits == before.hits + 1 and q.value == p.value
+    native.check(lib.dnh_free_async(q, None))

@@ -205,6 +205,21 @@ def test_convert(H, G, rng, src, dst):
         assert_exact(a.astype(dst), got)
 
 
+def test_convert_of_floats_outside_the_integer_range(H, G):
+    """NaN, infinities and floats that do not fit the integer target: the device follows the same stated rule as the oracle (a
+    plain cast would saturate on the GPU), checked against the hand-worked vectors and, in single precision, against the oracle."""
+    import convert_cases as cc
+    x = np.array(cc.INPUTS, dtype=np.float64)
+    for dst in cc.EXPECTED:
+        got = G.toNumpy(G.ofNumpy(x).convert(dst))
+        assert got.dtype == np.dtype(dst)
+        assert np.array_equal(got, cc.expected(dst)), (dst, got, cc.expected(dst))
+        with np.errstate(all="ignore"):
+            x32 = np.concatenate([x.astype(np.float32), np.float32([3e9, -3e9, 1.5e19, 7e18, -7e18, 2.5, -2.5])])
+        ref, dev = both(H, G, lambda t: t.convert(dst), x32)
+        assert_exact(ref, dev)
+
+
 def test_fill_and_counting(H, G):
     for dt in NUM:
         ref, got = both(H, G, lambda x: type(x).filled([5, 7], 3, x.Dev, x.DataType), np.zeros(1, dt))

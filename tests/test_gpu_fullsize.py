@@ -135,3 +135,29 @@ def test_config5_mlp_block(G):
     ref = np.exp(np.tanh(cn.astype(np.float64)) - np.tanh(cn.astype(np.float64)).max(axis=2, keepdims=True))
     ref /= ref.sum(axis=2, keepdims=True)
     assert np.allclose(p, ref, rtol=2e-5, atol=0)
+
+
+def test_in_place_elementwise_at_64M_elements(G):
+    """The target may be one of the sources (the reference's in-place forms, e.g. FillMultiply a a b,
+    Tensor.Docs/articles/Guide-Operations.md:103-115): 8192 x 8192 single precision, target = first source, target = second
+    source, and target = both, against NumPy bit for bit."""
+    rng = np.random.default_rng(5)
+    n = 8192
+    a = rng.standard_normal((n, n), dtype=np.float32)
+    b = rng.standard_normal((n, n), dtype=np.float32)
+    ta, tb = G.ofNumpy(a), G.ofNumpy(b)
+    ta.Backend.Multiply(ta, ta, tb)            # a <- a * b
+    assert_exact(a * b, G.toNumpy(ta))
+    tb.Backend.Subtract(tb, ta, tb)            # b <- (a * b) - b
+    assert_exact(a * b - b, G.toNumpy(tb))
+    ta.Backend.Add(ta, ta, ta)                 # a <- 2 (a * b)
+    assert_exact((a * b) + (a * b), G.toNumpy(ta))
+    ta.Backend.Tanh(ta, ta)
+    ref = np.tanh(((a * b) + (a * b)).astype(np.float64)).astype(np.float32)
+    got = G.toNumpy(ta)
+    assert np.all(np.abs(got - ref) <= 1e-6 * np.abs(ref) + 1e-37)
+    # a transposed view of the tensor itself as a source goes through a temporary on the host side of the interface as in the
+    # reference; in place with the identical layout is the supported overlap
+    tv = G.ofNumpy(a)
+    tv.T.Backend.Abs(tv.T, tv.T)
+    assert_exact(np.abs(a), G.toNumpy(tv))

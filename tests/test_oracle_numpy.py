@@ -214,3 +214,17 @@ def test_errors_mirror_the_reference(H):
         H.ofNumpy(np.zeros(3, np.int32)).tanh()
     with pytest.raises(IndexError):
         a.sumAxis(2)
+
+
+def test_convert_of_floats_outside_the_integer_range(H):
+    """Pins the oracle's Convert rule for NaN, infinities and out-of-range floats against vectors worked out by hand
+    (tests/convert_cases.py); in-range values truncate toward zero like a C cast."""
+    import convert_cases as cc
+    x = np.array(cc.INPUTS, dtype=np.float64)
+    for dst in cc.EXPECTED:
+        got = H.toNumpy(H.ofNumpy(x).convert(dst))
+        assert got.dtype == np.dtype(dst)
+        assert np.array_equal(got, cc.expected(dst)), (dst, got, cc.expected(dst))
+    r = np.random.default_rng(2).uniform(-100, 100, 1000)
+    for dst in (np.int32, np.int64, np.int8):
+        assert np.array_equal(H.toNumpy(H.ofNumpy(r).convert(dst)), np.trunc(r).astype(dst))
