@@ -151,14 +151,39 @@ __global__ __launch_bounds__(kBlock) void map_flat_kernel(Op op, typename Op::T*
 
 // ---- n-d ----------------------------------------------------------------------------------------------------------------
 
+// Division of a 32-bit index by an extent known on the host: q = (t + ((n - t) >> s1)) >> s2 with t = mulhi(n, m), exact for every
+// n < 2^32 (m = floor(2^32 (2^l - d) / d) + 1, l = ceil(log2 d), s1 = min(l, 1), s2 = max(l - 1, 0)).  Five instructions instead of
+// the twenty-odd of a hardware-free 32-bit division, once per thread and dimension.
+struct FastDiv {
+    uint32_t m, s1, s2, d;
+};
+inline FastDiv make_fast_div(uint32_t d) {
+    FastDiv f;
+    if (d == 0) d = 1;
+    uint32_t l = 0;
+    while (l < 32 && ((uint64_t)1 << l) < d) l++;
+    f.m = (uint32_t)((((uint64_t)1 << 32) * (((uint64_t)1 << l) - d)) / d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l > 1 ? l - 1 : 0;
+    f.d = d;
+    return f;
+}
+__device__ __forceinline__ uint32_t fast_div(uint32_t n, const FastDiv& f) {
+    const uint32_t t = __umulhi(n, f.m);
+    return (t + ((n - t) >> f.s1)) >> f.s2;
+}
+
 struct NdArgs {
     int nd;                                      // >= 1
+    FastDiv div[DNH_MAX_DIMS];                   // division by shape[d]
     uint32_t shape[DNH_MAX_DIMS];                // shape[nd-1] counts items of VEC elements
     int64_t stride[kMaxOperands][DNH_MAX_DIMS];  // element strides; last dimension already multiplied by VEC
     int vecload[kMaxOperands];                   // source k is read as a vector (last-dim stride 1) rather than splat (stride 0)
 };
 
-template <class Op, int VEC, int UNROLL>
+// ND > 0: the collapsed rank is known at compile time (2 for a matrix with a row- or column-broadcast operand, the commonest
+// case), so the index loop unrolls and its extents and strides stay in scalar registers; ND = 0: any rank, read from p.nd.
+template <class Op, int VEC, int UNROLL, int ND>
 __global__ __launch_bounds__(kBlock) void map_nd_kernel(Op op, typename Op::T* t, const typename Op::A* a, const typename Op::B* b,
                                                         const typename Op::C* c, NdArgs p, uint32_t nitems) {
     using T = typename Op::T;
@@ -176,8 +201,10 @@ __global__ __launch_bounds__(kBlock) void map_nd_kernel(Op op, typename Op::T* t
         ot[u] = oa[u] = ob[u] = oc[u] = 0;
         if (item < nitems) {
             uint32_t rem = item;
-            for (int d = p.nd - 1; d >= 0; d--) {
-                uint32_t q = (d == 0) ? 0u : rem / p.shape[d];
+            const int nd = ND > 0 ? ND : p.nd;
+#pragma unroll
+            for (int d = nd - 1; d >= 0; d--) {
+                uint32_t q = (d == 0) ? 0u : fast_div(rem, p.div[d]);
                 uint32_t idx = rem - q * p.shape[d];
                 rem = q;
                 ot[u] += (int64_t)idx * p.stride[0][d];
@@ -649,17 +676,19 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
         for (int k = 0; k < NOPS; k++)
             if (p.stride[k][last] == 1) vec = vec && (p.stride[k][d] % VEC) == 0;
     constexpr int UNROLL = 1;
+    if (vec) q.shape[last] = (uint32_t)(p.shape[last] / VEC);
+    for (int d = 0; d < q.nd; d++) q.div[d] = make_fast_div(q.shape[d]);
     if (vec) {
-        q.shape[last] = (uint32_t)(p.shape[last] / VEC);
         for (int k = 0; k < NOPS; k++) {
             q.vecload[k] = p.stride[k][last] == 1;
             q.stride[k][last] = p.stride[k][last] * VEC;
         }
         const uint32_t nitems = (uint32_t)(p.total / VEC);
-        hipLaunchKernelGGL((map_nd_kernel<Op, VEC, UNROLL>), dim3(cdiv(nitems, kBlock * UNROLL)), dim3(kBlock), 0, stream, op, t, a, b, c, q, nitems);
+        if (q.nd == 2) hipLaunchKernelGGL((map_nd_kernel<Op, VEC, UNROLL, 2>), dim3(cdiv(nitems, kBlock * UNROLL)), dim3(kBlock), 0, stream, op, t, a, b, c, q, nitems);
+        else hipLaunchKernelGGL((map_nd_kernel<Op, VEC, UNROLL, 0>), dim3(cdiv(nitems, kBlock * UNROLL)), dim3(kBlock), 0, stream, op, t, a, b, c, q, nitems);
     } else {
         const uint32_t nitems = (uint32_t)p.total;
-        hipLaunchKernelGGL((map_nd_kernel<Op, 1, UNROLL>), dim3(cdiv(nitems, kBlock * UNROLL)), dim3(kBlock), 0, stream, op, t, a, b, c, q, nitems);
+        hipLaunchKernelGGL((map_nd_kernel<Op, 1, UNROLL, 0>), dim3(cdiv(nitems, kBlock * UNROLL)), dim3(kBlock), 0, stream, op, t, a, b, c, q, nitems);
     }
     DNH_LAUNCH_CHECK();
     return DNH_OK;
