@@ -62,23 +62,27 @@ struct RCountTrue {
     __device__ int64_t extract(int64_t s) const { return s; }
 };
 
-template <class X> struct ArgState {
+template <class X, class P> struct ArgState {
     X val;
-    int64_t pos;
+    P pos;
 };
 // State starts at (NotFound, minValue|maxValue) and is replaced only by a strictly better value, so a position is set
 // only together with a value better than the initial one; equal values therefore are either both unset or both set, and
 // taking the smaller position on a tie reproduces "first index wins" under any combine order.
-template <class X, bool MAX> struct RArg {
-    using In = X; using State = ArgState<X>; using Out = int64_t;
+// P: the position's type inside the state.  int64, or uint32 (with 0xFFFFFFFF for NotFound) for 4-byte elements on axes shorter than
+// 2^32 - 1: the state is then 8 bytes instead of 16, which halves the partial results of two-pass folds and lets the column kernel
+// take its 256-lane form.
+template <class X, bool MAX, class P> struct RArg {
+    using In = X; using State = ArgState<X, P>; using Out = int64_t;
+    static constexpr P kNone = std::is_same<P, int64_t>::value ? (P)DNH_NOT_FOUND : (P)0xFFFFFFFFu;
     __device__ static bool better(X a, X b) { return MAX ? a > b : a < b; }
-    __device__ State init() const { return State{MAX ? std::numeric_limits<X>::lowest() : std::numeric_limits<X>::max(), DNH_NOT_FOUND}; }
-    __device__ State step(State s, X v, int64_t i) const { return better(v, s.val) ? State{v, i} : s; }
+    __device__ State init() const { return State{MAX ? std::numeric_limits<X>::lowest() : std::numeric_limits<X>::max(), kNone}; }
+    __device__ State step(State s, X v, int64_t i) const { return better(v, s.val) ? State{v, (P)i} : s; }
     __device__ State combine(State a, State b) const {
         const bool takeb = better(b.val, a.val) || (b.val == a.val && b.pos < a.pos);
         return takeb ? b : a;
     }
-    __device__ int64_t extract(State s) const { return s.pos; }
+    __device__ int64_t extract(State s) const { return s.pos == kNone ? DNH_NOT_FOUND : (int64_t)s.pos; }
 };
 template <class X> struct RFind {
     using In = X; using State = int64_t; using Out = int64_t;
@@ -110,15 +114,16 @@ int32_t run_numeric(const DnhTensor* t, const DnhTensor* s, hipStream_t st, cons
 
 template <bool MAX>
 int32_t run_arg(const DnhTensor* t, const DnhTensor* s, hipStream_t st, const char* what) {
+    const bool short_axis = s->ndims >= 1 && s->shape[s->ndims - 1] < 0xFFFFFFFFLL;
     switch (s->dtype) {
-        case DNH_U8: return launch_reduce(RArg<uint8_t, MAX>{}, t, s, st, what);
-        case DNH_I8: return launch_reduce(RArg<int8_t, MAX>{}, t, s, st, what);
-        case DNH_I32: return launch_reduce(RArg<int32_t, MAX>{}, t, s, st, what);
-        case DNH_U32: return launch_reduce(RArg<uint32_t, MAX>{}, t, s, st, what);
-        case DNH_I64: return launch_reduce(RArg<int64_t, MAX>{}, t, s, st, what);
-        case DNH_U64: return launch_reduce(RArg<uint64_t, MAX>{}, t, s, st, what);
-        case DNH_F32: return launch_reduce(RArg<float, MAX>{}, t, s, st, what);
-        case DNH_F64: return launch_reduce(RArg<double, MAX>{}, t, s, st, what);
+        case DNH_U8: return launch_reduce(RArg<uint8_t, MAX, int64_t>{}, t, s, st, what);
+        case DNH_I8: return launch_reduce(RArg<int8_t, MAX, int64_t>{}, t, s, st, what);
+        case DNH_I32: return short_axis ? launch_reduce(RArg<int32_t, MAX, uint32_t>{}, t, s, st, what) : launch_reduce(RArg<int32_t, MAX, int64_t>{}, t, s, st, what);
+        case DNH_U32: return short_axis ? launch_reduce(RArg<uint32_t, MAX, uint32_t>{}, t, s, st, what) : launch_reduce(RArg<uint32_t, MAX, int64_t>{}, t, s, st, what);
+        case DNH_I64: return launch_reduce(RArg<int64_t, MAX, int64_t>{}, t, s, st, what);
+        case DNH_U64: return launch_reduce(RArg<uint64_t, MAX, int64_t>{}, t, s, st, what);
+        case DNH_F32: return short_axis ? launch_reduce(RArg<float, MAX, uint32_t>{}, t, s, st, what) : launch_reduce(RArg<float, MAX, int64_t>{}, t, s, st, what);
+        case DNH_F64: return launch_reduce(RArg<double, MAX, int64_t>{}, t, s, st, what);
     }
     return fail(DNH_ERR_NOT_SUPPORTED, "%s is not defined for %s", what, dtype_name(s->dtype));
 }
