@@ -22,7 +22,7 @@ DNH_ERR_SINGULAR_MATRIX = 7
 DNH_ERR_NO_CONVERGENCE = 8
 
 # DnhDType
-DNH_BOOL, DNH_U8, DNH_I8, DNH_I32, DNH_U32, DNH_I64, DNH_U64, DNH_F32, DNH_F64 = range(9)
+DNH_BOOL, DNH_U8, DNH_I8, DNH_I32, DNH_U32, DNH_I64, DNH_U64, DNH_F32, DNH_F64, DNH_I16, DNH_U16 = range(11)
 
 DTYPE_TO_NUMPY = {
     DNH_BOOL: np.dtype(np.bool_),
@@ -34,6 +34,8 @@ DTYPE_TO_NUMPY = {
     DNH_U64: np.dtype(np.uint64),
     DNH_F32: np.dtype(np.float32),
     DNH_F64: np.dtype(np.float64),
+    DNH_I16: np.dtype(np.int16),
+    DNH_U16: np.dtype(np.uint16),
 }
 NUMPY_TO_DTYPE = {v: k for k, v in DTYPE_TO_NUMPY.items()}
 

@@ -155,6 +155,8 @@ template <class T> struct DTypeOf;
 template <> struct DTypeOf<bool> { static constexpr int value = DNH_BOOL; };
 template <> struct DTypeOf<uint8_t> { static constexpr int value = DNH_U8; };
 template <> struct DTypeOf<int8_t> { static constexpr int value = DNH_I8; };
+template <> struct DTypeOf<int16_t> { static constexpr int value = DNH_I16; };
+template <> struct DTypeOf<uint16_t> { static constexpr int value = DNH_U16; };
 template <> struct DTypeOf<int32_t> { static constexpr int value = DNH_I32; };
 template <> struct DTypeOf<uint32_t> { static constexpr int value = DNH_U32; };
 template <> struct DTypeOf<int64_t> { static constexpr int value = DNH_I64; };

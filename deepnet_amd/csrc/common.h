@@ -75,16 +75,17 @@ int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& 
 inline int dtype_size(int dt) {
     switch (dt) {
         case DNH_BOOL: case DNH_U8: case DNH_I8: return 1;
+        case DNH_I16: case DNH_U16: return 2;
         case DNH_I32: case DNH_U32: case DNH_F32: return 4;
         case DNH_I64: case DNH_U64: case DNH_F64: return 8;
     }
     return 0;
 }
 inline bool dtype_is_fp(int dt) { return dt == DNH_F32 || dt == DNH_F64; }
-inline bool dtype_is_signed(int dt) { return dt == DNH_I8 || dt == DNH_I32 || dt == DNH_I64 || dtype_is_fp(dt); }
+inline bool dtype_is_signed(int dt) { return dt == DNH_I8 || dt == DNH_I16 || dt == DNH_I32 || dt == DNH_I64 || dtype_is_fp(dt); }
 inline bool dtype_is_numeric(int dt) { return dt > DNH_BOOL && dt < DNH_DTYPE_COUNT; }
 inline const char* dtype_name(int dt) {
-    static const char* n[] = {"bool", "uint8", "int8", "int32", "uint32", "int64", "uint64", "single", "double"};
+    static const char* n[] = {"bool", "uint8", "int8", "int32", "uint32", "int64", "uint64", "single", "double", "int16", "uint16"};
     return (dt >= 0 && dt < DNH_DTYPE_COUNT) ? n[dt] : "?";
 }
 

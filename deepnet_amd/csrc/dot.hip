@@ -1191,7 +1191,7 @@ extern "C" int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTens
         }
 #define DNH_INT_DOT(DT, CT) case DT: return launch_gemm_int<CT>(g, (CT*)elem_ptr(t), (const CT*)elem_ptr(a), (const CT*)elem_ptr(b), batch, s);
         switch (t->dtype) {
-            DNH_INT_DOT(DNH_U8, uint8_t) DNH_INT_DOT(DNH_I8, int8_t) DNH_INT_DOT(DNH_I32, int32_t) DNH_INT_DOT(DNH_U32, uint32_t)
+            DNH_INT_DOT(DNH_U8, uint8_t) DNH_INT_DOT(DNH_I8, int8_t) DNH_INT_DOT(DNH_I16, int16_t) DNH_INT_DOT(DNH_U16, uint16_t) DNH_INT_DOT(DNH_I32, int32_t) DNH_INT_DOT(DNH_U32, uint32_t)
             DNH_INT_DOT(DNH_I64, int64_t) DNH_INT_DOT(DNH_U64, uint64_t)
         }
 #undef DNH_INT_DOT

@@ -11,6 +11,8 @@ int32_t run_numeric(int dt, const MapPlan& p, hipStream_t s) {
     switch (dt) {
         case DNH_U8: return launch_map(OpT<uint8_t>{}, p, s);
         case DNH_I8: return launch_map(OpT<int8_t>{}, p, s);
+        case DNH_I16: return launch_map(OpT<int16_t>{}, p, s);
+        case DNH_U16: return launch_map(OpT<uint16_t>{}, p, s);
         case DNH_I32: return launch_map(OpT<int32_t>{}, p, s);
         case DNH_U32: return launch_map(OpT<uint32_t>{}, p, s);
         case DNH_I64: return launch_map(OpT<int64_t>{}, p, s);

@@ -11,6 +11,8 @@ int32_t run_cmp(int dt, const MapPlan& p, hipStream_t s) {
     switch (dt) {
         case DNH_BOOL: case DNH_U8: return launch_map(OpT<uint8_t>{}, p, s);
         case DNH_I8: return launch_map(OpT<int8_t>{}, p, s);
+        case DNH_I16: return launch_map(OpT<int16_t>{}, p, s);
+        case DNH_U16: return launch_map(OpT<uint16_t>{}, p, s);
         case DNH_I32: return launch_map(OpT<int32_t>{}, p, s);
         case DNH_U32: return launch_map(OpT<uint32_t>{}, p, s);
         case DNH_I64: return launch_map(OpT<int64_t>{}, p, s);
@@ -52,6 +54,7 @@ extern "C" int32_t dnh_if_then_else(const DnhTensor* t, const DnhTensor* c, cons
     hipStream_t s = (hipStream_t)stream;
     switch (dtype_size(t->dtype)) {
         case 1: return launch_map(OpSelect<uint8_t>{}, p, s);
+        case 2: return launch_map(OpSelect<uint16_t>{}, p, s);
         case 4: return launch_map(OpSelect<uint32_t>{}, p, s);
         case 8: return launch_map(OpSelect<uint64_t>{}, p, s);
     }

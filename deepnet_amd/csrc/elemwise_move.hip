@@ -34,6 +34,8 @@ int32_t convert_to(int sdt, const MapPlan& p, hipStream_t s) {
     switch (sdt) {
         case DNH_BOOL: case DNH_U8: return launch_map(OpConvert<TT, uint8_t>{}, p, s);
         case DNH_I8: return launch_map(OpConvert<TT, int8_t>{}, p, s);
+        case DNH_I16: return launch_map(OpConvert<TT, int16_t>{}, p, s);
+        case DNH_U16: return launch_map(OpConvert<TT, uint16_t>{}, p, s);
         case DNH_I32: return launch_map(OpConvert<TT, int32_t>{}, p, s);
         case DNH_U32: return launch_map(OpConvert<TT, uint32_t>{}, p, s);
         case DNH_I64: return launch_map(OpConvert<TT, int64_t>{}, p, s);
@@ -47,6 +49,7 @@ int32_t convert_to(int sdt, const MapPlan& p, hipStream_t s) {
 int32_t convert_to_bool(int sdt, const MapPlan& p, hipStream_t s) {
     switch (sdt) {
         case DNH_BOOL: case DNH_U8: case DNH_I8: return launch_map(OpToBool<uint8_t>{}, p, s);
+        case DNH_I16: case DNH_U16: return launch_map(OpToBool<uint16_t>{}, p, s);
         case DNH_I32: case DNH_U32: return launch_map(OpToBool<uint32_t>{}, p, s);
         case DNH_I64: case DNH_U64: return launch_map(OpToBool<uint64_t>{}, p, s);
         case DNH_F32: return launch_map(OpToBool<float>{}, p, s);
@@ -66,6 +69,7 @@ extern "C" int32_t dnh_fill_const(const DnhTensor* t, const void* value, void* s
     hipStream_t s = (hipStream_t)stream;
     switch (dtype_size(t->dtype)) {
         case 1: { uint8_t v; memcpy(&v, value, 1); if (t->dtype == DNH_BOOL) v = v ? 1 : 0; return launch_map(OpFill<uint8_t>{v}, p, s); }
+        case 2: { uint16_t v; memcpy(&v, value, 2); return launch_map(OpFill<uint16_t>{v}, p, s); }
         case 4: { uint32_t v; memcpy(&v, value, 4); return launch_map(OpFill<uint32_t>{v}, p, s); }
         case 8: { uint64_t v; memcpy(&v, value, 8); return launch_map(OpFill<uint64_t>{v}, p, s); }
     }
@@ -91,7 +95,7 @@ extern "C" int32_t dnh_fill_incrementing(const DnhTensor* t, const void* start, 
 #define CASE(DT, X) case DT: { X s0, inc; memcpy(&s0, start, sizeof(X)); memcpy(&inc, incr, sizeof(X)); \
         hipLaunchKernelGGL(fill_inc_kernel<X>, dim3(blocks), dim3(kBlock), 0, s, (X*)elem_ptr(t), s0, inc, p, (uint32_t)n); break; }
     switch (t->dtype) {
-        CASE(DNH_U8, uint8_t) CASE(DNH_I8, int8_t) CASE(DNH_I32, int32_t) CASE(DNH_U32, uint32_t)
+        CASE(DNH_U8, uint8_t) CASE(DNH_I8, int8_t) CASE(DNH_I16, int16_t) CASE(DNH_U16, uint16_t) CASE(DNH_I32, int32_t) CASE(DNH_U32, uint32_t)
         CASE(DNH_I64, int64_t) CASE(DNH_U64, uint64_t) CASE(DNH_F32, float) CASE(DNH_F64, double)
         default: return fail(DNH_ERR_NOT_SUPPORTED, "dnh_fill_incrementing on %s", dtype_name(t->dtype));
     }
@@ -109,6 +113,7 @@ extern "C" int32_t dnh_copy(const DnhTensor* t, const DnhTensor* src, void* stre
     hipStream_t s = (hipStream_t)stream;
     switch (dtype_size(t->dtype)) {
         case 1: return launch_map(OpIdentity<uint8_t>{}, p, s);
+        case 2: return launch_map(OpIdentity<uint16_t>{}, p, s);
         case 4: return launch_map(OpIdentity<uint32_t>{}, p, s);
         case 8: return launch_map(OpIdentity<uint64_t>{}, p, s);
     }
@@ -127,6 +132,8 @@ extern "C" int32_t dnh_convert(const DnhTensor* t, const DnhTensor* src, void* s
         case DNH_BOOL: return convert_to_bool(src->dtype, p, s);
         case DNH_U8: return convert_to<uint8_t>(src->dtype, p, s);
         case DNH_I8: return convert_to<int8_t>(src->dtype, p, s);
+        case DNH_I16: return convert_to<int16_t>(src->dtype, p, s);
+        case DNH_U16: return convert_to<uint16_t>(src->dtype, p, s);
         case DNH_I32: return convert_to<int32_t>(src->dtype, p, s);
         case DNH_U32: return convert_to<uint32_t>(src->dtype, p, s);
         case DNH_I64: return convert_to<int64_t>(src->dtype, p, s);

@@ -20,6 +20,7 @@ template <template <class> class OpT>
 int32_t run_signed(int dt, const MapPlan& p, hipStream_t s, bool with_i8) {
     switch (dt) {
         case DNH_I8: if (with_i8) return run1<OpT, int8_t>(p, s); break;
+        case DNH_I16: return run1<OpT, int16_t>(p, s);
         case DNH_I32: return run1<OpT, int32_t>(p, s);
         case DNH_I64: return run1<OpT, int64_t>(p, s);
         case DNH_F32: return run1<OpT, float>(p, s);
@@ -48,6 +49,7 @@ extern "C" int32_t dnh_unary(int32_t op, const DnhTensor* t, const DnhTensor* a,
             // identity on any numeric type: move by element width
             switch (dtype_size(dt)) {
                 case 1: return run1<OpIdentity, uint8_t>(p, s);
+                case 2: return run1<OpIdentity, uint16_t>(p, s);
                 case 4: return run1<OpIdentity, uint32_t>(p, s);
                 default: return run1<OpIdentity, uint64_t>(p, s);
             }

@@ -106,6 +106,18 @@ template <> __device__ __forceinline__ void atomic_add_any<uint8_t>(uint8_t* p, 
     } while (old != assumed);
 }
 
+// two-byte integers: the same on the containing 32-bit word
+template <> __device__ __forceinline__ void atomic_add_any<uint16_t>(uint16_t* p, uint16_t v) {
+    uint32_t* w = (uint32_t*)((uintptr_t)p & ~(uintptr_t)3);
+    const unsigned sh = ((uintptr_t)p & 2) * 8;
+    uint32_t old = *w, assumed;
+    do {
+        assumed = old;
+        const uint32_t b = ((assumed >> sh) + v) & 0xFFFFu;
+        old = atomicCAS(w, assumed, (assumed & ~(0xFFFFu << sh)) | (b << sh));
+    } while (old != assumed);
+}
+
 template <class X>
 __global__ __launch_bounds__(kBlock) void scatter_kernel(X* t, const X* s, IndexArgs a, uint32_t n, int32_t* err) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
@@ -783,6 +795,7 @@ bool try_compaction_fast(const MaskArgs& m, void* full, void* out, const Lay& ol
     if ((n % vec) != 0 || !aligned_to(full, 16) || !aligned_to(m.mask[0], 16)) return false;
     switch (esize) {
         case 1: *status = run_compaction_fast<uint8_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
+        case 2: *status = run_compaction_fast<uint16_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
         case 4: *status = run_compaction_fast<uint32_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
         case 8: *status = run_compaction_fast<uint64_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
     }
@@ -805,6 +818,7 @@ int32_t run_compaction(const MaskArgs& m, void* full, void* out, const Lay& olay
     DNH_LAUNCH_CHECK();
     switch (esize) {
         case 1: hipLaunchKernelGGL((compact_move_kernel<uint8_t, MODE>), dim3(nb), dim3(kBlock), 0, stream, m, (uint8_t*)full, (uint8_t*)out, olay, n, nout, counts); break;
+        case 2: hipLaunchKernelGGL((compact_move_kernel<uint16_t, MODE>), dim3(nb), dim3(kBlock), 0, stream, m, (uint16_t*)full, (uint16_t*)out, olay, n, nout, counts); break;
         case 4: hipLaunchKernelGGL((compact_move_kernel<uint32_t, MODE>), dim3(nb), dim3(kBlock), 0, stream, m, (uint32_t*)full, (uint32_t*)out, olay, n, nout, counts); break;
         case 8: hipLaunchKernelGGL((compact_move_kernel<uint64_t, MODE>), dim3(nb), dim3(kBlock), 0, stream, m, (uint64_t*)full, (uint64_t*)out, olay, n, nout, counts); break;
         default: return fail(DNH_ERR_NOT_SUPPORTED, "masked op: unsupported element width");
@@ -844,6 +858,7 @@ extern "C" int32_t dnh_gather(const DnhTensor* t, const DnhTensor* const* idx, i
     const dim3 grid(cdiv(n, kBlock));
     switch (dtype_size(t->dtype)) {
         case 1: hipLaunchKernelGGL(gather_kernel<uint8_t>, grid, dim3(kBlock), 0, s, (uint8_t*)elem_ptr(t), (const uint8_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
+        case 2: hipLaunchKernelGGL(gather_kernel<uint16_t>, grid, dim3(kBlock), 0, s, (uint16_t*)elem_ptr(t), (const uint16_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
         case 4: hipLaunchKernelGGL(gather_kernel<uint32_t>, grid, dim3(kBlock), 0, s, (uint32_t*)elem_ptr(t), (const uint32_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
         case 8: hipLaunchKernelGGL(gather_kernel<uint64_t>, grid, dim3(kBlock), 0, s, (uint64_t*)elem_ptr(t), (const uint64_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
         default: return fail(DNH_ERR_NOT_SUPPORTED, "dnh_gather: unsupported element width");
@@ -869,6 +884,7 @@ extern "C" int32_t dnh_scatter(const DnhTensor* t, const DnhTensor* const* idx, 
     switch (t->dtype) {
         CASE(DNH_U8, uint8_t)
         case DNH_I8: hipLaunchKernelGGL(scatter_kernel<uint8_t>, grid, dim3(kBlock), 0, s, (uint8_t*)elem_ptr(t), (const uint8_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
+        case DNH_I16: case DNH_U16: hipLaunchKernelGGL(scatter_kernel<uint16_t>, grid, dim3(kBlock), 0, s, (uint16_t*)elem_ptr(t), (const uint16_t*)elem_ptr(src), a, (uint32_t)n, eflag); break;
         CASE(DNH_I32, int32_t) CASE(DNH_U32, uint32_t) CASE(DNH_I64, int64_t) CASE(DNH_U64, uint64_t) CASE(DNH_F32, float) CASE(DNH_F64, double)
         default: return fail(DNH_ERR_NOT_SUPPORTED, "dnh_scatter on %s", dtype_name(t->dtype));
     }

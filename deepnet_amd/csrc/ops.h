@@ -101,9 +101,10 @@ template <class X> struct OpDiv {
         if constexpr (kIsFp<X>) return a / b;
         else {
             bool bad = b == 0;
-            if constexpr (std::is_signed<X>::value) bad = bad || (a == std::numeric_limits<X>::min() && b == X(-1));
+            // (8- and 16-bit operands are widened to 32 bits before the division, so MinValue / -1 does not overflow: it wraps when stored)
+            if constexpr (std::is_signed<X>::value && sizeof(X) >= 4) bad = bad || (a == std::numeric_limits<X>::min() && b == X(-1));
             const X bb = bad ? X(1) : b;
-            const X q = (X)(a / bb);
+            const X q = (X)(a / bb);   // narrow types: int arithmetic, truncated
             return bad ? X(0) : q;
         }
     }
@@ -115,7 +116,8 @@ template <class X> struct OpMod {
         else if constexpr (std::is_same<X, double>::value) return fmod(a, b);
         else {
             bool bad = b == 0;
-            if constexpr (std::is_signed<X>::value) bad = bad || (a == std::numeric_limits<X>::min() && b == X(-1));
+            // (8- and 16-bit operands are widened to 32 bits before the division, so MinValue / -1 does not overflow: it wraps when stored)
+            if constexpr (std::is_signed<X>::value && sizeof(X) >= 4) bad = bad || (a == std::numeric_limits<X>::min() && b == X(-1));
             const X bb = bad ? X(1) : b;
             const X r = (X)(a % bb);
             return bad ? X(0) : r;
@@ -176,7 +178,7 @@ template <class W> struct OpFill {
 // integer target is left unspecified by the CLI standard; what the reference's runtime (64-bit x86) does is restated here, since a
 // plain cast saturates on this GPU:
 //   -> int32 / int64: truncate toward zero; NaN and values outside the range give the minimum value (the cvtt* instructions);
-//   -> int8 / uint8: as int32, then the low 8 bits;   -> uint32: as int64, then the low 32 bits;
+//   -> int8 / uint8 / int16 / uint16: as int32, then the low 8 / 16 bits;   -> uint32: as int64, then the low 32 bits;
 //   -> uint64: below 2^63 as int64 (negative values wrap), from 2^63 on (and NaN) int64(x - 2^63) + 2^63, wrapping.
 template <class F> __device__ __forceinline__ int32_t fp_to_i32(F x) {
     return (x >= (F)-2147483648.0 && x < (F)2147483648.0) ? (int32_t)x : INT32_MIN;
@@ -190,7 +192,7 @@ template <class TT, class TA> struct OpConvert {
         if constexpr (kIsFp<TA> && !kIsFp<TT>) {
             if constexpr (std::is_same<TT, int32_t>::value) return fp_to_i32(a);
             else if constexpr (std::is_same<TT, int64_t>::value) return fp_to_i64(a);
-            else if constexpr (sizeof(TT) == 1) return (TT)(uint32_t)fp_to_i32(a);
+            else if constexpr (sizeof(TT) <= 2) return (TT)(uint32_t)fp_to_i32(a);
             else if constexpr (std::is_same<TT, uint32_t>::value) return (uint32_t)(uint64_t)fp_to_i64(a);
             else {
                 static_assert(std::is_same<TT, uint64_t>::value, "integer target");

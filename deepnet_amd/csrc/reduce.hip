@@ -102,6 +102,8 @@ int32_t run_numeric(const DnhTensor* t, const DnhTensor* s, hipStream_t st, cons
     switch (s->dtype) {
         case DNH_U8: return launch_reduce(RT<uint8_t>{}, t, s, st, what, ps);
         case DNH_I8: return launch_reduce(RT<int8_t>{}, t, s, st, what, ps);
+        case DNH_I16: return launch_reduce(RT<int16_t>{}, t, s, st, what, ps);
+        case DNH_U16: return launch_reduce(RT<uint16_t>{}, t, s, st, what, ps);
         case DNH_I32: return launch_reduce(RT<int32_t>{}, t, s, st, what, ps);
         case DNH_U32: return launch_reduce(RT<uint32_t>{}, t, s, st, what, ps);
         case DNH_I64: return launch_reduce(RT<int64_t>{}, t, s, st, what, ps);
@@ -118,6 +120,8 @@ int32_t run_arg(const DnhTensor* t, const DnhTensor* s, hipStream_t st, const ch
     switch (s->dtype) {
         case DNH_U8: return launch_reduce(RArg<uint8_t, MAX, int64_t>{}, t, s, st, what);
         case DNH_I8: return launch_reduce(RArg<int8_t, MAX, int64_t>{}, t, s, st, what);
+        case DNH_I16: return launch_reduce(RArg<int16_t, MAX, int64_t>{}, t, s, st, what);
+        case DNH_U16: return launch_reduce(RArg<uint16_t, MAX, int64_t>{}, t, s, st, what);
         case DNH_I32: return short_axis ? launch_reduce(RArg<int32_t, MAX, uint32_t>{}, t, s, st, what) : launch_reduce(RArg<int32_t, MAX, int64_t>{}, t, s, st, what);
         case DNH_U32: return short_axis ? launch_reduce(RArg<uint32_t, MAX, uint32_t>{}, t, s, st, what) : launch_reduce(RArg<uint32_t, MAX, int64_t>{}, t, s, st, what);
         case DNH_I64: return launch_reduce(RArg<int64_t, MAX, int64_t>{}, t, s, st, what);
@@ -214,7 +218,7 @@ extern "C" int32_t dnh_find_last_axis(const void* value, const DnhTensor* t, con
     hipStream_t st = (hipStream_t)stream;
 #define CASE(DT, X) case DT: { X v; memcpy(&v, value, sizeof(X)); return launch_reduce(RFind<X>{v}, t, src, st, "FindLastAxis"); }
     switch (src->dtype) {
-        CASE(DNH_BOOL, uint8_t) CASE(DNH_U8, uint8_t) CASE(DNH_I8, int8_t) CASE(DNH_I32, int32_t) CASE(DNH_U32, uint32_t)
+        CASE(DNH_BOOL, uint8_t) CASE(DNH_U8, uint8_t) CASE(DNH_I8, int8_t) CASE(DNH_I16, int16_t) CASE(DNH_U16, uint16_t) CASE(DNH_I32, int32_t) CASE(DNH_U32, uint32_t)
         CASE(DNH_I64, int64_t) CASE(DNH_U64, uint64_t) CASE(DNH_F32, float) CASE(DNH_F64, double)
     }
 #undef CASE

@@ -31,6 +31,7 @@ module internal Desc =
         if   t = typeof<bool>   then DType.Bool elif t = typeof<byte>   then DType.U8  elif t = typeof<sbyte>  then DType.I8
         elif t = typeof<int32>  then DType.I32  elif t = typeof<uint32> then DType.U32 elif t = typeof<int64>  then DType.I64
         elif t = typeof<uint64> then DType.U64  elif t = typeof<single> then DType.F32 elif t = typeof<double> then DType.F64
+        elif t = typeof<int16>  then DType.I16  elif t = typeof<uint16> then DType.U16
         else raise (NotSupportedException (sprintf "element type %s is not supported by the HIP backend" t.Name))
 
     let make (basePtr: nativeint) (dataType: Type) (layout: TensorLayout) =

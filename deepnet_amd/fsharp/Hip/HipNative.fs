@@ -21,7 +21,7 @@ type internal Status =
 
 /// DnhDType — the element types the reference marshals to kernels (Cuda/NativeTensor.fs:22-34).
 type internal DType =
-    | Bool = 0 | U8 = 1 | I8 = 2 | I32 = 3 | U32 = 4 | I64 = 5 | U64 = 6 | F32 = 7 | F64 = 8
+    | Bool = 0 | U8 = 1 | I8 = 2 | I32 = 3 | U32 = 4 | I64 = 5 | U64 = 6 | F32 = 7 | F64 = 8 | I16 = 9 | U16 = 10
 
 /// DnhTensor: descriptor passed by reference (replaces the Reflection.Emit structs of Cuda/NativeTensor.fs:96-208).
 /// Blittable: the two extents arrays of the C struct are spelled out as sixteen int64 fields (a managed int64[] marked ByValArray

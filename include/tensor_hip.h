@@ -45,7 +45,8 @@ typedef enum DnhStatus {
     DNH_ERR_NO_CONVERGENCE = 8    /* -> "SVD did not converge" (Host/HostBackend.fs:598)             */
 } DnhStatus;
 
-/* Element types: the set the reference marshals to kernels (Cuda/NativeTensor.fs:22-34). bool is one byte 0/1. */
+/* Element types: the set the reference marshals to kernels (Cuda/NativeTensor.fs:22-34) plus the 16-bit integers its host device
+ * also handles (Sgn.fs:11-15, Host/ScalarOps.fs).  bool is one byte 0/1.  Values are part of the ABI: new types are appended. */
 typedef enum DnhDType {
     DNH_BOOL = 0,
     DNH_U8 = 1,
@@ -56,7 +57,9 @@ typedef enum DnhDType {
     DNH_U64 = 6,
     DNH_F32 = 7,
     DNH_F64 = 8,
-    DNH_DTYPE_COUNT = 9
+    DNH_I16 = 9,
+    DNH_U16 = 10,
+    DNH_DTYPE_COUNT = 11
 } DnhDType;
 
 /* Replaces the by-value kernel argument struct Tensor<T,N> (Cuda/Kernels/Tensor.cuh:7-16,

@@ -212,7 +212,7 @@ template <class T> inline T safe_div(T a, T b) {
     if constexpr (is_fp<T>) return a / b;
     else {
         if (b == 0) return 0;
-        if constexpr (std::is_signed<T>::value)
+        if constexpr (std::is_signed<T>::value && sizeof(T) >= 4)   // narrower operands divide as int32 and wrap when stored (IL div, conv.i2)
             if (a == std::numeric_limits<T>::min() && b == T(-1)) return 0;
         return (T)(a / b);
     }
@@ -221,7 +221,7 @@ template <class T> inline T safe_mod(T a, T b) {
     if constexpr (is_fp<T>) return (T)std::fmod(a, b);
     else {
         if (b == 0) return 0;
-        if constexpr (std::is_signed<T>::value)
+        if constexpr (std::is_signed<T>::value && sizeof(T) >= 4)   // narrower operands divide as int32 and wrap when stored (IL div, conv.i2)
             if (a == std::numeric_limits<T>::min() && b == T(-1)) return 0;
         return (T)(a % b);
     }
@@ -234,13 +234,15 @@ template <class T> inline T max_value() { return std::numeric_limits<T>::max(); 
 // ---- dtype dispatch ---------------------------------------------------------------------------------------------------
 
 #define HREF_NUMERIC_CASES(M) \
-    case DNH_U8: M(uint8_t) break; case DNH_I8: M(int8_t) break; case DNH_I32: M(int32_t) break; case DNH_U32: M(uint32_t) break; \
+    case DNH_U8: M(uint8_t) break; case DNH_I8: M(int8_t) break; case DNH_I16: M(int16_t) break; case DNH_U16: M(uint16_t) break; \
+    case DNH_I32: M(int32_t) break; case DNH_U32: M(uint32_t) break; \
     case DNH_I64: M(int64_t) break; case DNH_U64: M(uint64_t) break; case DNH_F32: M(float) break; case DNH_F64: M(double) break;
 #define HREF_ALL_CASES(M) case DNH_BOOL: M(uint8_t) break; HREF_NUMERIC_CASES(M)
 
 inline int dtype_size(int dt) {
     switch (dt) {
         case DNH_BOOL: case DNH_U8: case DNH_I8: return 1;
+        case DNH_I16: case DNH_U16: return 2;
         case DNH_I32: case DNH_U32: case DNH_F32: return 4;
         case DNH_I64: case DNH_U64: case DNH_F64: return 8;
     }
@@ -375,7 +377,7 @@ template <class TT, class TA> inline TT convert_elem(TA x) {
     if constexpr (std::is_floating_point<TA>::value && !std::is_floating_point<TT>::value) {
         if constexpr (std::is_same<TT, int32_t>::value) return fp_to_i32(x);
         else if constexpr (std::is_same<TT, int64_t>::value) return fp_to_i64(x);
-        else if constexpr (sizeof(TT) == 1) return (TT)(uint32_t)fp_to_i32(x);
+        else if constexpr (sizeof(TT) <= 2) return (TT)(uint32_t)fp_to_i32(x);
         else if constexpr (std::is_same<TT, uint32_t>::value) return (uint32_t)(uint64_t)fp_to_i64(x);
         else {
             if (x < (TA)9223372036854775808.0) return (uint64_t)fp_to_i64(x);
@@ -464,7 +466,7 @@ int32_t href_unary(int32_t op, const DnhTensor* t, const DnhTensor* a) {
     if (!valid(t) || !valid(a) || t->dtype != a->dtype) return DNH_ERR_INVALID_ARG;
     int dt = t->dtype;
     bool fp = dt == DNH_F32 || dt == DNH_F64;
-    bool sgnd = fp || dt == DNH_I8 || dt == DNH_I32 || dt == DNH_I64;
+    bool sgnd = fp || dt == DNH_I8 || dt == DNH_I16 || dt == DNH_I32 || dt == DNH_I64;
     if (op == DNH_NEGATE) {
         if (dt != DNH_BOOL) return DNH_ERR_NOT_SUPPORTED;
         return run_unary<uint8_t, uint8_t>(t, a, false, [](uint8_t x) { return (uint8_t)(x ? 0 : 1); });
@@ -478,18 +480,18 @@ int32_t href_unary(int32_t op, const DnhTensor* t, const DnhTensor* a) {
         case DNH_UNARY_MINUS:
             if (!sgnd) return DNH_ERR_NOT_SUPPORTED;
 #define M(T) return run_unary<T, T>(t, a, true, [](T x) { return wrap_neg<T>(x); });
-            switch (dt) { case DNH_I8: M(int8_t) case DNH_I32: M(int32_t) case DNH_I64: M(int64_t) case DNH_F32: M(float) case DNH_F64: M(double) }
+            switch (dt) { case DNH_I8: M(int8_t) case DNH_I16: M(int16_t) case DNH_I32: M(int32_t) case DNH_I64: M(int64_t) case DNH_F32: M(float) case DNH_F64: M(double) }
             return DNH_ERR_NOT_SUPPORTED;
 #undef M
         case DNH_ABS:
             if (!sgnd) return DNH_ERR_NOT_SUPPORTED;
 #define M(T) return run_unary<T, T>(t, a, true, [](T x) { return wrap_abs<T>(x); });
-            switch (dt) { case DNH_I8: M(int8_t) case DNH_I32: M(int32_t) case DNH_I64: M(int64_t) case DNH_F32: M(float) case DNH_F64: M(double) }
+            switch (dt) { case DNH_I8: M(int8_t) case DNH_I16: M(int16_t) case DNH_I32: M(int32_t) case DNH_I64: M(int64_t) case DNH_F32: M(float) case DNH_F64: M(double) }
             return DNH_ERR_NOT_SUPPORTED;
 #undef M
         case DNH_SGN:  // Sgn.fs implements int16/int32/int64/single/double only
 #define M(T) return run_unary<T, T>(t, a, false, [](T x) { return sgn_of<T>(x); });
-            switch (dt) { case DNH_I32: M(int32_t) case DNH_I64: M(int64_t) case DNH_F32: M(float) case DNH_F64: M(double) }
+            switch (dt) { case DNH_I16: M(int16_t) case DNH_I32: M(int32_t) case DNH_I64: M(int64_t) case DNH_F32: M(float) case DNH_F64: M(double) }
             return DNH_ERR_NOT_SUPPORTED;
 #undef M
         default: break;
@@ -517,7 +519,8 @@ int32_t href_is_finite(const DnhTensor* t, const DnhTensor* a) {
         case DNH_F32: return run_unary<uint8_t, float>(t, a, false, [](float x) { return (uint8_t)(std::isfinite(x) ? 1 : 0); });
         case DNH_F64: return run_unary<uint8_t, double>(t, a, false, [](double x) { return (uint8_t)(std::isfinite(x) ? 1 : 0); });
 #define M(T) return run_unary<uint8_t, T>(t, a, false, [](T) { return (uint8_t)1; });
-        case DNH_U8: M(uint8_t) case DNH_I8: M(int8_t) case DNH_I32: M(int32_t) case DNH_U32: M(uint32_t) case DNH_I64: M(int64_t) case DNH_U64: M(uint64_t)
+        case DNH_U8: M(uint8_t) case DNH_I8: M(int8_t) case DNH_I16: M(int16_t) case DNH_U16: M(uint16_t) case DNH_I32: M(int32_t) case DNH_U32: M(uint32_t)
+        case DNH_I64: M(int64_t) case DNH_U64: M(uint64_t)
 #undef M
     }
     return DNH_ERR_NOT_SUPPORTED;

@@ -1,6 +1,6 @@
 """Known-answer vectors for Convert of floats that do not fit the integer target, worked out by hand from the rule the backends
-state (truncate toward zero; NaN and out-of-range values give the minimum of int32 / int64; int8 / uint8 go through int32 and
-uint32 through int64, keeping the low bits; uint64 splits at 2^63).  Inputs are doubles that are exactly representable."""
+state (truncate toward zero; NaN and out-of-range values give the minimum of int32 / int64; the 8- and 16-bit types go through int32
+and uint32 through int64, keeping the low bits; uint64 splits at 2^63).  Inputs are doubles that are exactly representable."""
 import numpy as np
 
 I32_MIN, I64_MIN = -2 ** 31, -2 ** 63
@@ -16,6 +16,8 @@ EXPECTED = {
                10 ** 10, -10 ** 10, I64_MIN, I64_MIN, I64_MIN, I64_MIN],
     np.uint8: [0, 0, 0, 255, 0, 255, 0, 44, 127, 255, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0],
     np.int8: [0, 0, 0, -1, 0, -1, 0, 44, 127, -1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0],
+    np.uint16: [0, 0, 0, 65535, 0, 255, 256, 300, 65407, 65535, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0],
+    np.int16: [0, 0, 0, -1, 0, 255, 256, 300, -129, -1, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0],
     np.uint32: [0, 0, 0, 4294967295, 0, 255, 256, 300, 4294967167, 2147483647, 2147483648, 2147483648, 2147483647, 5, 1410065408,
                 2884901888, 0, 0, 0, 0],
     np.uint64: [0, 0, 2 ** 63, U64 - 1, 0, 255, 256, 300, U64 - 129, 2147483647, 2147483648, U64 - 2147483648, U64 - 2147483649,

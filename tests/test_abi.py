@@ -37,7 +37,7 @@ def test_descriptor_layout_matches_the_header():
 int main(void) {
   printf("%zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(DnhTensor), offsetof(DnhTensor, base), offsetof(DnhTensor, offset),
          offsetof(DnhTensor, ndims), offsetof(DnhTensor, dtype), offsetof(DnhTensor, shape), offsetof(DnhTensor, stride), sizeof(DnhDeviceInfo));
-  printf("%d %d %d %d %d %lld\n", DNH_F64, DNH_NEGATE, DNH_XOR, DNH_GREATER_OR_EQUAL, DNH_COUNT_TRUE, (long long)DNH_NOT_FOUND);
+  printf("%d %d %d %d %d %d %d %lld\n", DNH_F64, DNH_I16, DNH_U16, DNH_NEGATE, DNH_XOR, DNH_GREATER_OR_EQUAL, DNH_COUNT_TRUE, (long long)DNH_NOT_FOUND);
   return 0; }'''
     with tempfile.TemporaryDirectory() as d:
         c = os.path.join(d, "t.c")
@@ -49,7 +49,7 @@ int main(void) {
     T = abi.DnhTensor
     assert vals[:8] == [C.sizeof(T), T.base.offset, T.offset.offset, T.ndims.offset, T.dtype.offset, T.shape.offset, T.stride.offset,
                         C.sizeof(abi.DnhDeviceInfo)]
-    assert vals[8:] == [abi.DNH_F64, abi.DNH_NEGATE, abi.DNH_XOR, abi.DNH_GREATER_OR_EQUAL, abi.DNH_COUNT_TRUE, abi.NOT_FOUND]
+    assert vals[8:] == [abi.DNH_F64, abi.DNH_I16, abi.DNH_U16, abi.DNH_NEGATE, abi.DNH_XOR, abi.DNH_GREATER_OR_EQUAL, abi.DNH_COUNT_TRUE, abi.NOT_FOUND]
 
 
 def test_oracle_exports_the_same_operator_set():

@@ -155,7 +155,7 @@ def test_bool_dot_not_supported(G):
         a @ a
 
 
-@pytest.mark.parametrize("dt", [np.uint8, np.int8, np.int32, np.uint32, np.int64, np.uint64])
+@pytest.mark.parametrize("dt", [np.uint8, np.int8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64])
 def test_integer_dot_wraps_like_the_host_backend(H, G, rng, dt):
     """The reference's host backend computes dot of the types BLAS does not cover as multiply + sumAxis in the element type
     (Host/HostBackend.fs:544-546): wrapping arithmetic, so the result is bit-exact whatever the summation order."""

@@ -9,7 +9,7 @@ from util import both, assert_exact, assert_rel
 
 pytestmark = pytest.mark.gpu
 
-NUM = [np.uint8, np.int8, np.int32, np.uint32, np.int64, np.uint64, np.float32, np.float64]
+NUM = [np.uint8, np.int8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64, np.float32, np.float64]
 
 
 def rand(rng, dt, shape, lo=-50, hi=50):
@@ -66,7 +66,7 @@ def test_special_values_fp(H, G):
         assert_exact(ref, got)
 
 
-@pytest.mark.parametrize("dt", [np.int8, np.int32, np.int64])
+@pytest.mark.parametrize("dt", [np.int8, np.int16, np.int32, np.int64])
 def test_unary_int(H, G, rng, dt):
     a = rand(rng, dt, (100, 17))
     for fn in ["__neg__", "abs", "__pos__"] + (["sgn"] if dt != np.int8 else []):
@@ -98,6 +98,22 @@ def test_integer_wraparound(H, G):
     assert got.tolist() == [-1, 1, -1, 1]
 
 
+@pytest.mark.parametrize("dt", [np.int8, np.int16, np.int32, np.int64, np.uint16, np.uint64])
+def test_integer_division_corner_cases(H, G, dt):
+    """A zero divisor gives 0.  MinValue / -1: 0 for int32 / int64 (the quotient does not exist); the narrower types divide as
+    int32 and wrap when the quotient is stored, so MinValue comes back."""
+    info = np.iinfo(dt)
+    a = np.array([info.min, info.max, 7, info.min, 0], dtype=dt)
+    b = np.array([0, 0, 0, info.max if info.min == 0 else -1, 0], dtype=dt)
+    ref, got = both(H, G, lambda x, y: x / y, a, b)
+    assert_exact(ref, got)
+    narrow_signed = info.min < 0 and np.dtype(dt).itemsize < 4
+    assert got.tolist() == [0, 0, 0, info.min if narrow_signed else 0, 0]
+    ref, got = both(H, G, lambda x, y: x % y, a, b)
+    assert_exact(ref, got)
+    assert got.tolist() == [0, 0, 0, 0, 0]
+
+
 @pytest.mark.parametrize("dt", [np.bool_] + NUM)
 def test_compare(H, G, rng, dt):
     a = rand(rng, dt, (63, 70), -3, 3)
@@ -115,7 +131,7 @@ def test_logic(H, G, rng):
         assert_exact(ref, got)
 
 
-@pytest.mark.parametrize("dt", [np.bool_, np.int8, np.int32, np.float32, np.int64, np.float64])
+@pytest.mark.parametrize("dt", [np.bool_, np.int8, np.uint16, np.int32, np.float32, np.int64, np.float64])
 def test_if_then_else(H, G, rng, dt):
     c = rand(rng, np.bool_, (33, 65))
     a = rand(rng, dt, (33, 65))
@@ -137,7 +153,7 @@ def test_scalar_broadcast_and_power(H, G, rng):
     assert_exact(ai > 0, got)
 
 
-@pytest.mark.parametrize("dt", [np.float32, np.float64, np.int32, np.uint8])
+@pytest.mark.parametrize("dt", [np.float32, np.float64, np.int32, np.uint8, np.int16])
 def test_strided_and_broadcast_views(H, G, rng, dt):
     x = rand(rng, dt, (6, 20, 70))
     v = rand(rng, dt, (70,))
@@ -203,6 +219,17 @@ def test_convert(H, G, rng, src, dst):
     assert_exact(ref, got)
     if np.dtype(dst) != np.bool_:
         assert_exact(a.astype(dst), got)
+
+
+@pytest.mark.parametrize("src", [np.int16, np.uint16, np.int32, np.int64, np.uint64])
+def test_convert_between_integers_keeps_the_low_bits(H, G, rng, src):
+    info = np.iinfo(src)
+    a = rng.integers(info.min, info.max, size=5000, dtype=src, endpoint=True)
+    a[:4] = [info.min, info.max, 0, info.max // 2 + 1]
+    for dst in (np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64):
+        ref, got = both(H, G, lambda x: x.convert(dst), a)
+        assert_exact(ref, got)
+        assert_exact(a.astype(dst), got)            # NumPy's integer casts wrap as well
 
 
 def test_convert_of_floats_outside_the_integer_range(H, G):

@@ -8,7 +8,7 @@ from util import both, assert_exact
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("dt", [np.int32, np.float32, np.int64, np.float64, np.uint8, np.bool_])
+@pytest.mark.parametrize("dt", [np.int32, np.float32, np.int64, np.float64, np.uint8, np.bool_, np.int16])
 def test_gather_1d(H, G, rng, dt):
     src = (rng.integers(0, 2, 100000) > 0) if dt == np.bool_ else rng.integers(-1000, 1000, 100000).astype(dt)
     idx = rng.integers(0, src.size, 30011).astype(np.int64)
@@ -45,7 +45,7 @@ def test_gather_out_of_range_raises(H, G):
     assert G.toNumpy(ok).tolist() == [9, 0]
 
 
-@pytest.mark.parametrize("dt", [np.int32, np.int64, np.uint32, np.uint64, np.uint8, np.int8])
+@pytest.mark.parametrize("dt", [np.int32, np.int64, np.uint32, np.uint64, np.uint8, np.int8, np.int16, np.uint16])
 def test_scatter_int_with_duplicates(H, G, rng, dt):
     src = rng.integers(0, 100, 50000).astype(dt)
     idx = rng.integers(0, 777, 50000).astype(np.int64)          # heavy duplication: sums, wrapping for narrow types
@@ -135,7 +135,7 @@ def test_masked_get_1d(H, G, rng, n):
     assert_exact(a[m], got)
 
 
-@pytest.mark.parametrize("dt", [np.float32, np.float64, np.uint8, np.bool_])
+@pytest.mark.parametrize("dt", [np.float32, np.float64, np.uint8, np.bool_, np.uint16])
 def test_masked_get_set_nd(H, G, rng, dt):
     a = (rng.random((37, 41)) < 0.5) if dt == np.bool_ else rng.integers(0, 100, (37, 41)).astype(dt)
     m = rng.random((37, 41)) < 0.3

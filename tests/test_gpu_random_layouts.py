@@ -56,9 +56,9 @@ def make_operands(rng, H, G, dtype, max_elems=200_000):
 def test_random_views_elementwise_and_folds(H, G, seed):
     rng = np.random.default_rng(1000 + seed)
     for case in range(25):
-        dtype = [np.int32, np.int64, np.uint8, np.int8][int(rng.integers(0, 4))]
+        dtype = [np.int32, np.int64, np.uint8, np.int8, np.int16, np.uint16][int(rng.integers(0, 6))]
         a_np = make_operands(rng, H, G, dtype)
-        b_np = rng.integers(-50, 50, size=a_np.shape).astype(dtype) if dtype != np.uint8 else rng.integers(0, 100, size=a_np.shape).astype(dtype)
+        b_np = rng.integers(-50, 50, size=a_np.shape).astype(dtype) if dtype not in (np.uint8, np.uint16) else rng.integers(0, 100, size=a_np.shape).astype(dtype)
         state = rng.bit_generator.state
         outs = []
         for M in (H, G):

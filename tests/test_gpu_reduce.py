@@ -41,7 +41,7 @@ def test_sum_max_min_fp_all_axes(H, G, rng, dt, shape):
         assert_exact(np.max(x, axis=ax), G.toNumpy(G.ofNumpy(x).maxAxis(ax)))
 
 
-@pytest.mark.parametrize("dt", [np.int32, np.int64, np.uint8, np.int8, np.uint32, np.uint64])
+@pytest.mark.parametrize("dt", [np.int32, np.int64, np.uint8, np.int8, np.int16, np.uint16, np.uint32, np.uint64])
 def test_int_folds_exact(H, G, rng, dt):
     x = rng.integers(0, 100, size=(33, 1030)).astype(dt)
     for ax in (0, 1):

@@ -7,7 +7,7 @@ import pytest
 from util import assert_exact, run_on
 
 NOT_FOUND = -(2 ** 63) + 4
-NUM = [np.uint8, np.int8, np.int32, np.uint32, np.int64, np.uint64, np.float32, np.float64]
+NUM = [np.uint8, np.int8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64, np.float32, np.float64]
 
 
 def rnd(rng, dt, shape, lo=-50, hi=50):
@@ -45,6 +45,19 @@ def test_integer_overflow_wraps(H):
     assert run_on(H, lambda x, y: x + y, [a, b]).tolist() == [-2 ** 31, 2 ** 31 - 1, 2 ** 30 + 4]
     assert run_on(H, lambda x, y: x * y, [a, b]).tolist() == [2 ** 31 - 1, -2 ** 31, 0]
     assert run_on(H, lambda x: x.sumAxis(0), [np.array([200, 100], np.uint8)]).tolist() == 44
+
+
+def test_narrow_integer_division_follows_int32_arithmetic(H):
+    """int16 (and int8) operands are divided as int32 and the quotient is truncated when stored (IL `div` then `conv.i2`): MinValue / -1
+    wraps to MinValue, where the 32- and 64-bit types have no quotient (defined as 0, like a zero divisor)."""
+    for dt, want in ((np.int16, -2 ** 15), (np.int8, -2 ** 7), (np.int32, 0), (np.int64, 0)):
+        lo = np.iinfo(dt).min
+        a, b = np.array([lo, lo, 5], dtype=dt), np.array([-1, 0, 0], dtype=dt)
+        assert run_on(H, lambda x, y: x / y, [a, b]).tolist() == [want, 0, 0]
+        assert run_on(H, lambda x, y: x % y, [a, b]).tolist() == [0, 0, 0]
+    s = np.array([-300, 0, 17, -2 ** 15], dtype=np.int16)
+    assert run_on(H, lambda x: x.sgn(), [s]).tolist() == [-1, 0, 1, -1]
+    assert run_on(H, lambda x: abs(x), [s]).tolist() == [300, 0, 17, -2 ** 15]
 
 
 def test_round_is_ties_to_even_and_sgn_abs(H):
@@ -226,5 +239,5 @@ def test_convert_of_floats_outside_the_integer_range(H):
         assert got.dtype == np.dtype(dst)
         assert np.array_equal(got, cc.expected(dst)), (dst, got, cc.expected(dst))
     r = np.random.default_rng(2).uniform(-100, 100, 1000)
-    for dst in (np.int32, np.int64, np.int8):
+    for dst in (np.int32, np.int64, np.int8, np.int16):
         assert np.array_equal(H.toNumpy(H.ofNumpy(r).convert(dst)), np.trunc(r).astype(dst))
