@@ -446,6 +446,9 @@ __global__ __launch_bounds__(64 * SG) void gemm_split_finish_kernel(T* __restric
 // rounded fp32 product) stay on the fp32 instructions.  DNH_DOT_BF16X3=0 in the environment keeps every product there.
 // Every operand that is contiguous along one of its two dimensions (row-major or transposed; 16-byte aligned rows when k is the
 // contiguous one), K splits included; accumulating products and operands strided in both dimensions take gemm_kernel.
+// Two forms: 128 x 128 tiles, 256 threads, two workgroups per CU (gemm_bf16x3_kernel: every size, K splits), and 256 x 256 tiles,
+// 512 threads, one workgroup per CU (gemm_bf16x3_big_kernel: half the staging and LDS traffic per matrix instruction; taken when
+// the product has about a CU's worth of such tiles, use_big_tiles; DNH_DOT_BIG=0 / 1 in the environment forces the choice).
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kX3BK = 16;
@@ -471,25 +474,26 @@ __device__ __forceinline__ void split3_bf16(const float (&v)[8], u32x4& hi, u32x
     }
 }
 
-// Staging of one operand tile (128 rows x 16 k; "row" is m for A and n for B) from memory into the three bf16 tiles in LDS.
+// Staging of one operand tile (ROWS rows x 16 k; "row" is m for A and n for B) by 2 * ROWS threads from memory into the three bf16 tiles in LDS.
 //   KC: k is the contiguous direction.  Four lanes cover the 16 k of a row with one 16-byte load each (a wavefront reads 16 rows of
-//       64 contiguous bytes); a thread takes the same 4 k of rows r and r + 64 and writes 8 bytes per part and row.
+//       64 contiguous bytes); a thread takes the same 4 k of rows r and r + ROWS / 2 and writes 8 bytes per part and row.
 //   otherwise the rows are contiguous (row-major B, transposed A): a thread takes one row and 8 consecutive k with element loads
 //       (the lanes of a wavefront read 256 consecutive bytes) and writes 16 bytes per part.
-template <bool KC>
+template <bool KC, int ROWS = BM>
 struct X3Stage {
+    static constexpr int HALF = ROWS / 2;   // 2 * ROWS threads stage a tile
     int row, kofs;      // first row and first k of this thread inside the tile
     bool ok0, ok1;      // row (and for KC row + 64) inside the matrix
     const float *p0, *p1;   // element (row, k = 0) of those rows; row 0 of the matrix when outside
     int64_t ks;
     bool bad;           // an element staged so far is infinite or too small to cut into bf16 parts
     __device__ __forceinline__ void init(const float* base, int64_t row0, int64_t limit, int64_t rs, int64_t kstride, int tid) {
-        row = KC ? tid >> 2 : tid & 127;
-        kofs = KC ? (tid & 3) * 4 : (tid >> 7) * 8;
+        row = KC ? tid >> 2 : tid & (ROWS - 1);
+        kofs = KC ? (tid & 3) * 4 : (tid / ROWS) * 8;
         ok0 = row0 + row < limit;
-        ok1 = KC && row0 + row + 64 < limit;
+        ok1 = KC && row0 + row + HALF < limit;
         p0 = base + (ok0 ? (row0 + row) * rs : 0);
-        p1 = base + (ok1 ? (row0 + row + 64) * rs : 0);
+        p1 = base + (ok1 ? (row0 + row + HALF) * rs : 0);
         ks = KC ? 1 : kstride;
         bad = false;
     }
@@ -519,7 +523,7 @@ struct X3Stage {
         }
     }
     // cuts the staged elements into their parts and writes them to tile[part][row][k]
-    __device__ __forceinline__ void store(float (&r)[8], __bf16 (*tile)[BM][kX3Row]) {
+    __device__ __forceinline__ void store(float (&r)[8], __bf16 (*tile)[ROWS][kX3Row]) {
 #pragma unroll
         for (int e = 0; e < 8; e++) r[e] = ((KC && e >= 4) ? ok1 : ok0) ? r[e] : 0.0f;
         // +-inf stays infinite under the scaling; |x| < 2^-109 (x != 0) becomes denormal; zero stays zero
@@ -533,20 +537,64 @@ struct X3Stage {
             if constexpr (KC) {
                 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
                 *reinterpret_cast<u32x2*>(&tile[s][row][kofs]) = u32x2{part[s][0], part[s][1]};
-                *reinterpret_cast<u32x2*>(&tile[s][row + 64][kofs]) = u32x2{part[s][2], part[s][3]};
+                *reinterpret_cast<u32x2*>(&tile[s][row + HALF][kofs]) = u32x2{part[s][2], part[s][3]};
             } else {
                 *reinterpret_cast<u32x4*>(&tile[s][row][kofs]) = part[s];
             }
         }
     }
+    // The same work as store() in 16 pieces of a few instructions each, for a caller that places them between its matrix instructions:
+    // piece 2e cuts element e, piece 2e + 1 classifies it, packs a finished pair and writes finished groups to LDS.
+    uint32_t hw[2], mw[2], lw[2];
+    u32x4 part[3];
+    template <int Q>
+    __device__ __forceinline__ void piece(float (&r)[8], __bf16 (*tile)[ROWS][kX3Row]) {
+        constexpr int e = Q / 2;
+        if constexpr (Q % 2 == 0) {
+            const float v = ((KC && e >= 4) ? ok1 : ok0) ? r[e] : 0.0f;
+            r[e] = v;
+            const uint32_t h = __float_as_uint(v);
+            const float r1 = v - __uint_as_float(h & 0xFFFF0000u);
+            const uint32_t m = __float_as_uint(r1);
+            const float r2 = r1 - __uint_as_float(m & 0xFFFF0000u);
+            hw[e & 1] = h;
+            mw[e & 1] = m;
+            lw[e & 1] = __float_as_uint(r2);
+        } else {
+            constexpr int kClassInfOrDenormal = (1 << 2) | (1 << 4) | (1 << 7) | (1 << 9);
+            bad |= __builtin_amdgcn_classf(r[e] * 0x1p-17f, kClassInfOrDenormal);
+            if constexpr (e % 2 == 1) {
+                part[0][e / 2] = __builtin_amdgcn_perm(hw[1], hw[0], 0x07060302u);
+                part[1][e / 2] = __builtin_amdgcn_perm(mw[1], mw[0], 0x07060302u);
+                part[2][e / 2] = __builtin_amdgcn_perm(lw[1], lw[0], 0x07060302u);
+            }
+            if constexpr (KC && e % 4 == 3) {
+                typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+#pragma unroll
+                for (int s = 0; s < 3; s++)
+                    *reinterpret_cast<u32x2*>(&tile[s][row + (e / 4) * HALF][kofs]) = u32x2{part[s][e / 2 - 1], part[s][e / 2]};
+            }
+            if constexpr (!KC && e == 7) {
+#pragma unroll
+                for (int s = 0; s < 3; s++) *reinterpret_cast<u32x4*>(&tile[s][row][kofs]) = part[s];
+            }
+        }
+    }
 };
+
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>()), ...); }
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>()); }
 
 // One 128 x 128 tile of c = a . b over k in [0, K) on v_mfma_f32_32x32x2_f32, operands fetched element by element through their
 // strides: the slow, IEEE-faithful path of a workgroup of gemm_bf16x3_kernel whose operands hold infinite or very small elements.
 // A32 / B32: [16][BM + PAD] floats of LDS each; every thread of the block calls it.
+// tid: 0..255, the thread's number among the 256 that share this tile (a larger workgroup runs several tiles side by side, each group
+// with its own A32 / B32; the barriers are the whole workgroup's, so every group must make the same number of K steps).
 __device__ __forceinline__ void fp32_tile_fallback(float* c, const float* a, const float* b, const GemmArgs& g, int64_t m0, int64_t n0, int64_t K,
-                                                float (*A32)[BM + PAD], float (*B32)[BN + PAD]) {
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+                                                float (*A32)[BM + PAD], float (*B32)[BN + PAD], int tid) {
+    const int wave = tid >> 6, lane = tid & 63;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64, lk = lane >> 5, lm = lane & 31;
     f32x16 acc[2][2];
 #pragma unroll
@@ -639,14 +687,6 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
     sa.init(a, m0, g.M, g.sam, g.sak, tid);
     sb.init(b, n0, g.N, g.sbn, g.sbk, tid);
     float ra[8], rb[8];
-    auto load_tiles = [&](int64_t k0) {
-        sa.template load<TAIL>(k0, K, ra);
-        sb.template load<TAIL>(k0, K, rb);
-    };
-    auto store_tiles = [&](int buf) {
-        sa.store(ra, As[buf]);
-        sb.store(rb, Bs[buf]);
-    };
 
     const int wave = tid >> 6, lane = tid & 63;
     const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
@@ -659,43 +699,63 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
 
-    load_tiles(0);
-    store_tiles(0);
-    __syncthreads();
+    // One K step: the 24 matrix instructions of the tiles in LDS buffer cur and, when NEXT, the fetch of the next step's elements
+    // (first), their cutting into parts and the writes to the other buffer (32 pieces, X3Stage::piece, two behind each of the last 16
+    // matrix instructions).  The order is pinned by scheduling barriers: left alone, the compiler puts the fetches after most of the
+    // matrix instructions and the cutting after all of them, and each wavefront waits for memory with the matrix pipe idle.
     int cur = 0;
-    for (int64_t k0 = 0; k0 < K; k0 += kX3BK) {
-        const bool more = k0 + kX3BK < K;
-        if (more) load_tiles(k0 + kX3BK);
+    auto k_step = [&](auto next_tag, auto tail_tag, int64_t k_next) {
+        constexpr bool NEXT = decltype(next_tag)::value, TL = decltype(tail_tag)::value;
+        if constexpr (NEXT) {
+            sa.template load<TL>(k_next, K, ra);
+            sb.template load<TL>(k_next, K, rb);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         bf16x8 av[2][3], bv[2][3];
 #pragma unroll
-        for (int i = 0; i < 2; i++)
+        for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int s = 0; s < 3; s++) {
-                av[i][s] = *reinterpret_cast<const bf16x8*>(&As[cur][s][wm + i * 32 + lm][lk * 8]);
-                bv[i][s] = *reinterpret_cast<const bf16x8*>(&Bs[cur][s][wn + i * 32 + lm][lk * 8]);
+            for (int s = 0; s < 3; s++) bv[j][s] = *reinterpret_cast<const bf16x8*>(&Bs[cur][s][wn + j * 32 + lm][lk * 8]);
+#pragma unroll
+        for (int s = 0; s < 3; s++) av[0][s] = *reinterpret_cast<const bf16x8*>(&As[cur][s][wm + lm][lk * 8]);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<24>([&](auto tt) {
+            constexpr int t = decltype(tt)::value, i = t / 12, j = (t % 12) / 6, p = t % 6;
+            constexpr int pa = p == 0 ? 1 : p == 1 ? 0 : p == 2 ? 2 : p == 3 ? 0 : p == 4 ? 1 : 0;   // smallest products first
+            constexpr int pb = p == 0 ? 1 : p == 1 ? 2 : p == 2 ? 0 : p == 3 ? 1 : p == 4 ? 0 : 0;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][pa], bv[j][pb], acc[i][j], 0, 0, 0);
+            if constexpr (t < 3) av[1][t] = *reinterpret_cast<const bf16x8*>(&As[cur][t][wm + 32 + lm][lk * 8]);
+            if constexpr (NEXT && t >= 8) {
+                constexpr int q = (t - 8) * 2;
+                if constexpr (q < 16) {
+                    sa.template piece<q>(ra, As[cur ^ 1]);
+                    sa.template piece<q + 1>(ra, As[cur ^ 1]);
+                } else {
+                    sb.template piece<q - 16>(rb, Bs[cur ^ 1]);
+                    sb.template piece<q - 15>(rb, Bs[cur ^ 1]);
+                }
             }
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
-                // smallest products first
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][1], bv[j][1], acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][0], bv[j][2], acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][2], bv[j][0], acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][0], bv[j][1], acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][1], bv[j][0], acc[i][j], 0, 0, 0);
-                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][0], bv[j][0], acc[i][j], 0, 0, 0);
-            }
-        if (more) {
-            store_tiles(cur ^ 1);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (NEXT) {
             __syncthreads();
             cur ^= 1;
         }
-    }
+    };
+    const int64_t nsteps = (K + kX3BK - 1) / kX3BK;
+    sa.template load<TAIL>(0, K, ra);
+    sb.template load<TAIL>(0, K, rb);
+    sa.store(ra, As[0]);
+    sb.store(rb, Bs[0]);
+    __syncthreads();
+    // K steps 1 .. nsteps - 2 are whole; the last one may be partial (TAIL)
+    for (int64_t s = 0; s + 2 < nsteps; s++) k_step(std::true_type(), std::false_type(), (s + 1) * kX3BK);
+    if (nsteps >= 2) k_step(std::true_type(), std::integral_constant<bool, TAIL>(), (nsteps - 1) * kX3BK);
+    k_step(std::false_type(), std::false_type(), 0);
     // an element that cannot be cut into bf16 parts was staged by some thread: the whole tile is redone on the fp32 instruction
     if (__syncthreads_or((int)(sa.bad | sb.bad))) {
         fp32_tile_fallback(c, a, b, g, m0, n0, K, reinterpret_cast<float (*)[BM + PAD]>(&As[0][0][0][0]),
-                           reinterpret_cast<float (*)[BN + PAD]>(&Bs[0][0][0][0]));
+                           reinterpret_cast<float (*)[BN + PAD]>(&Bs[0][0][0][0]), tid);
         return;
     }
     // accumulator register r of lane l holds row 8*(r/4) + 4*(l/32) + r%4, column l%32 of its 32x32 tile
@@ -710,6 +770,170 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
                 const int64_t n = n0 + wn + j * 32 + lm;
                 if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
             }
+}
+
+// The same product on 256 x 256 tiles: 512 threads = 8 wavefronts in a 2 x 4 arrangement, each owning 128 x 64 (eight 32 x 32
+// accumulators).  Against the 128 x 128 kernel every staged element (cut into parts once per workgroup that needs it) and every LDS
+// operand fetch feeds twice as many matrix instructions: 48 per wavefront and K step against 18 LDS reads and 16 staged elements.
+// One workgroup per CU (144 KB of LDS, two wavefronts per SIMD); chosen when the product has at least a CU's worth of such tiles.
+// The K loop keeps one shape per iteration (no branch inside: the last K step and the K tail are peeled), so that the cutting of the
+// next step's elements can be scheduled between the matrix instructions of the current one.
+constexpr int XBM = 256, XBN = 256, kBigThreads = 512;
+constexpr size_t kBigLdsBytes = (size_t)2 * 2 * 3 * XBM * kX3Row * sizeof(__bf16);
+
+template <bool TAIL, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kBigThreads) void gemm_bf16x3_big_kernel(float* c, const float* a, const float* b, GemmArgs g) {
+    extern __shared__ __align__(16) unsigned char x3_lds[];
+    typedef __bf16 (*Tiles)[3][XBM][kX3Row];                      // [buffer][part][row][k]
+    Tiles As = reinterpret_cast<Tiles>(x3_lds);
+    Tiles Bs = reinterpret_cast<Tiles>(x3_lds + kBigLdsBytes / 2);
+
+    uint32_t bid = blockIdx.x, tm, tn;
+    if (g.xcd_2d) {
+        const uint32_t xcd = bid % 8u, local = bid / 8u, regw = g.tiles_n / 4u, regh = g.tiles_m / 2u;
+        tm = (xcd / 4u) * regh + local / regw;
+        tn = (xcd % 4u) * regw + local % regw;
+        bid = 0;
+    } else {
+        if (g.xcd_chunk) bid = (bid % 8u) * g.xcd_chunk + bid / 8u;
+        tn = bid % g.tiles_n;
+        bid /= g.tiles_n;
+        tm = bid % g.tiles_m;
+        bid /= g.tiles_m;
+    }
+    int64_t oa = 0, ob = 0, oc = 0;
+    for (int d = g.nbatch - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
+        const uint32_t i = bid - q * g.bshape[d];
+        bid = q;
+        oa += (int64_t)i * g.bsa[d];
+        ob += (int64_t)i * g.bsb[d];
+        oc += (int64_t)i * g.bsc[d];
+    }
+    const int64_t K = g.K;
+    const int64_t m0 = (int64_t)tm * XBM, n0 = (int64_t)tn * XBN;
+    a += oa;
+    b += ob;
+    c += oc;
+    const int tid = threadIdx.x;
+
+    X3Stage<A_KC, XBM> sa;
+    X3Stage<B_KC, XBN> sb;
+    sa.init(a, m0, g.M, g.sam, g.sak, tid);
+    sb.init(b, n0, g.N, g.sbn, g.sbk, tid);
+    float ra[8], rb[8];
+
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 2) * 128, wn = (wave & 3) * 64;
+    const int lm = lane & 31, lk = lane >> 5;
+    f32x16 acc[4][2];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.0f;
+
+    // the matrix instructions of one K step on LDS buffer `buf`
+    auto compute = [&](int buf) {
+        bf16x8 bv[2][3];
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int s = 0; s < 3; s++) bv[j][s] = *reinterpret_cast<const bf16x8*>(&Bs[buf][s][wn + j * 32 + lm][lk * 8]);
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            bf16x8 av[3];
+#pragma unroll
+            for (int s = 0; s < 3; s++) av[s] = *reinterpret_cast<const bf16x8*>(&As[buf][s][wm + i * 32 + lm][lk * 8]);
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                // smallest products first
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][1], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][2], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[2], bv[j][0], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][1], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[1], bv[j][0], acc[i][j], 0, 0, 0);
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[0], bv[j][0], acc[i][j], 0, 0, 0);
+            }
+        }
+    };
+
+    const int64_t nsteps = (K + kX3BK - 1) / kX3BK;
+    sa.template load<TAIL>(0, K, ra);
+    sb.template load<TAIL>(0, K, rb);
+    sa.store(ra, As[0]);
+    sb.store(rb, Bs[0]);
+    __syncthreads();
+    int cur = 0;
+    // One K step: fetch the next step's elements, multiply the current step's tiles, cut the fetched elements into parts and write them
+    // to the other buffer.  The instruction order is pinned by scheduling barriers (left alone, the compiler puts the fetches after most
+    // of the matrix instructions and the cutting after all of them: each wavefront then waits for memory with the matrix pipe idle):
+    // fetches first; the LDS reads of B and of the first 32 rows of A; then the 48 matrix instructions, the remaining LDS reads behind
+    // the first nine, and behind the later ones the 32 pieces of the cutting (X3Stage::piece) with their LDS writes.
+    auto k_step = [&](auto tail_tag, int64_t k_next) {
+        constexpr bool TL = decltype(tail_tag)::value;
+        sa.template load<TL>(k_next, K, ra);
+        sb.template load<TL>(k_next, K, rb);
+        __builtin_amdgcn_sched_barrier(0);
+        bf16x8 av[4][3], bv[2][3];
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int s = 0; s < 3; s++) bv[j][s] = *reinterpret_cast<const bf16x8*>(&Bs[cur][s][wn + j * 32 + lm][lk * 8]);
+#pragma unroll
+        for (int s = 0; s < 3; s++) av[0][s] = *reinterpret_cast<const bf16x8*>(&As[cur][s][wm + lm][lk * 8]);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<48>([&](auto tt) {
+            constexpr int t = decltype(tt)::value, i = t / 12, j = (t % 12) / 6, p = t % 6;
+            constexpr int pa = p == 0 ? 1 : p == 1 ? 0 : p == 2 ? 2 : p == 3 ? 0 : p == 4 ? 1 : 0;   // smallest products first
+            constexpr int pb = p == 0 ? 1 : p == 1 ? 2 : p == 2 ? 0 : p == 3 ? 1 : p == 4 ? 0 : 0;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][pa], bv[j][pb], acc[i][j], 0, 0, 0);
+            if constexpr (t < 9) av[1 + t / 3][t % 3] = *reinterpret_cast<const bf16x8*>(&As[cur][t % 3][wm + (1 + t / 3) * 32 + lm][lk * 8]);
+            if constexpr (t >= 16 && t < 32) sa.template piece<t - 16>(ra, As[cur ^ 1]);   // pieces 0-15 cut A, 16-31 cut B
+            if constexpr (t >= 32) sb.template piece<t - 32>(rb, Bs[cur ^ 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        __syncthreads();
+        cur ^= 1;
+    };
+    // K steps 1 .. nsteps - 2 are whole
+    for (int64_t s = 0; s + 2 < nsteps; s++) k_step(std::false_type(), (s + 1) * kX3BK);
+    if (nsteps >= 2) k_step(std::integral_constant<bool, TAIL>(), (nsteps - 1) * kX3BK);
+    compute(cur);
+
+    // an element that cannot be cut into bf16 parts was staged by some thread: the four 128 x 128 quarters of the tile are redone on the
+    // fp32 instruction, two at a time (threads 0-255 take the upper two, threads 256-511 the lower two)
+    if (__syncthreads_or((int)(sa.bad | sb.bad))) {
+        const int grp = tid >> 8;
+        float* lds = reinterpret_cast<float*>(x3_lds) + grp * 2 * 16 * (BM + PAD);
+        for (int q = 0; q < 2; q++)
+            fp32_tile_fallback(c, a, b, g, m0 + grp * 128, n0 + q * 128, K, reinterpret_cast<float (*)[BM + PAD]>(lds),
+                               reinterpret_cast<float (*)[BN + PAD]>(lds + 16 * (BM + PAD)), tid & 255);
+        return;
+    }
+    const bool full_mn = m0 + XBM <= g.M && n0 + XBN <= g.N;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
+                const int64_t n = n0 + wn + j * 32 + lm;
+                if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
+            }
+}
+
+// 256 x 256 tiles, one workgroup per CU: when they fill the CUs about as evenly as 128 x 128 tiles at two per CU would
+bool use_big_tiles(int64_t M, int64_t N, int64_t batch) {
+    static const int mode = [] { const char* e = getenv("DNH_DOT_BIG"); return e ? atoi(e) : -1; }();   // 0 / 1 force the choice
+    if (mode >= 0) return mode != 0;
+    const int64_t cus = device_cus();
+    const int64_t big = cdiv(M, (int64_t)XBM) * cdiv(N, (int64_t)XBN) * batch, small = cdiv(M, (int64_t)BM) * cdiv(N, (int64_t)BN) * batch;
+    const double eff_big = (double)big / (double)(cdiv(big, cus) * cus), eff_small = (double)small / (double)(cdiv(small, 2 * cus) * 2 * cus);
+    const double waste_big = (double)(M * N * batch) / ((double)big * XBM * XBN), waste_small = (double)(M * N * batch) / ((double)small * BM * BN);
+    return eff_big * waste_big * 1.1 >= eff_small * waste_small;
 }
 
 bool use_bf16x3() {
@@ -776,6 +1000,27 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         x3 = g.K >= kX3BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_bf16x3();
     }
     g.xcd_2d = (x3 && g.nbatch == 0 && (g.tiles_m % 2u) == 0 && (g.tiles_n % 4u) == 0 && blocks >= 64) ? 1u : 0u;
+    if constexpr (sizeof(T) == 4) {
+        if (x3 && splits == 1 && use_big_tiles(g.M, g.N, batch)) {
+            g.tiles_m = (uint32_t)cdiv(g.M, (int64_t)XBM);
+            g.tiles_n = (uint32_t)cdiv(g.N, (int64_t)XBN);
+            blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
+            g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
+            g.xcd_2d = (g.nbatch == 0 && (g.tiles_m % 2u) == 0 && (g.tiles_n % 4u) == 0 && blocks >= 64) ? 1u : 0u;
+#define DNH_BIG_LAUNCH(TL, AK, BK_) do { \
+                static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_bf16x3_big_kernel<TL, AK, BK_>), \
+                                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLdsBytes); \
+                if (attr != hipSuccess) return fail(DNH_ERR_HIP, "dnh_dot: %s", hipGetErrorString(attr)); \
+                hipLaunchKernelGGL((gemm_bf16x3_big_kernel<TL, AK, BK_>), dim3((unsigned)blocks), dim3(kBigThreads), kBigLdsBytes, stream, c, a, b, g); } while (0)
+#define DNH_BIG_AB(TL) do { if (a_kc) { if (b_kc) DNH_BIG_LAUNCH(TL, true, true); else DNH_BIG_LAUNCH(TL, true, false); } \
+                            else { if (b_kc) DNH_BIG_LAUNCH(TL, false, true); else DNH_BIG_LAUNCH(TL, false, false); } } while (0)
+            if (g.K % kX3BK) DNH_BIG_AB(true); else DNH_BIG_AB(false);
+#undef DNH_BIG_AB
+#undef DNH_BIG_LAUNCH
+            DNH_LAUNCH_CHECK();
+            return DNH_OK;
+        }
+    }
     if (splits > 1) {
         if (x3) {
             if constexpr (sizeof(T) == 4) DNH_X3(true);

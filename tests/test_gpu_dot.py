@@ -404,3 +404,43 @@ print("ok")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=300)
     assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
+
+
+@pytest.mark.parametrize("ta,tb", STAGINGS)
+@pytest.mark.parametrize("m,k,n", [(4096, 48, 4096),     # 256 tiles of 256 x 256: the large-tile kernel by the library's own choice
+                                   (4000, 40, 4090)])    # edge tiles on both sides and a partial last K step
+def test_single_precision_large_tiles(G, rng, ta, tb, m, k, n):
+    """Products with at least a CU's worth of 256 x 256 tiles run the large-tile form of the bf16-parts kernel: same parts, same six
+    products, so the same 16 u S; an infinite element sends its tile to the fp32 instructions, quarter by quarter."""
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    b = rng.standard_normal((k, n)).astype(np.float32)
+    x, y = _views(G, a, b, ta, tb)
+    assert _err_over_uS(a, b, G.toNumpy(x @ y)).max() <= 16
+    a[300, 5] = np.inf           # tile row 1: quarter (1, *) of every tile in that row
+    b[7, 1000] = -np.inf
+    b[5, 2000] = 0.0             # inf x 0
+    with np.errstate(all="ignore"):
+        want = a @ b
+    x, y = _views(G, a, b, ta, tb)
+    got = G.toNumpy(x @ y)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    assert np.array_equal(np.isposinf(got), np.isposinf(want)) and np.array_equal(np.isneginf(got), np.isneginf(want))
+    fin = np.isfinite(want)
+    af, bf = np.where(np.isfinite(a), a, 0), np.where(np.isfinite(b), b, 0)
+    assert _err_over_uS(af, bf, np.where(fin, got, 0))[fin].max() <= 16
+
+
+def test_large_tile_kernel_on_every_shape_of_this_file():
+    """DNH_DOT_BIG=1 sends every product that the bf16-parts kernel takes in one launch to its large-tile form, whatever the size
+    (the switch is read once per process, so the tests of this file run again in a child process)."""
+    import os
+    import subprocess
+    import sys
+    if os.environ.get("DNH_DOT_BIG") is not None:
+        pytest.skip("already running under the switch")
+    env = dict(os.environ, DNH_DOT_BIG="1")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-m", "gpu", "-p", "no:cacheprovider", os.path.abspath(__file__),
+                          "-k", "single_precision or matmat or batched or split_k or config5"],
+                         env=env, cwd=root, capture_output=True, text=True, timeout=900)
+    assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-2000:]
