@@ -781,7 +781,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
 constexpr int XBM = 256, XBN = 256, kBigThreads = 512;
 constexpr size_t kBigLdsBytes = (size_t)2 * 2 * 3 * XBM * kX3Row * sizeof(__bf16);
 
-template <bool TAIL, bool A_KC, bool B_KC>
+template <bool SPLIT, bool TAIL, bool A_KC, bool B_KC>
 __global__ __launch_bounds__(kBigThreads) void gemm_bf16x3_big_kernel(float* c, const float* a, const float* b, GemmArgs g) {
     extern __shared__ __align__(16) unsigned char x3_lds[];
     typedef __bf16 (*Tiles)[3][XBM][kX3Row];                      // [buffer][part][row][k]
@@ -802,6 +802,7 @@ __global__ __launch_bounds__(kBigThreads) void gemm_bf16x3_big_kernel(float* c, 
         bid /= g.tiles_m;
     }
     int64_t oa = 0, ob = 0, oc = 0;
+    uint32_t chunk_id = 0;
     for (int d = g.nbatch - 1; d >= 0; d--) {
         const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
         const uint32_t i = bid - q * g.bshape[d];
@@ -809,8 +810,10 @@ __global__ __launch_bounds__(kBigThreads) void gemm_bf16x3_big_kernel(float* c, 
         oa += (int64_t)i * g.bsa[d];
         ob += (int64_t)i * g.bsb[d];
         oc += (int64_t)i * g.bsc[d];
+        if (SPLIT && d == g.nbatch - 1) chunk_id = i;
     }
-    const int64_t K = g.K;
+    // this block's extent along k: the whole of K, or one chunk of it (SPLIT: the innermost batch dimension counts the chunks)
+    const int64_t K = SPLIT ? min(g.kchunk, g.K - (int64_t)chunk_id * g.kchunk) : g.K;
     const int64_t m0 = (int64_t)tm * XBM, n0 = (int64_t)tn * XBN;
     a += oa;
     b += ob;
@@ -925,20 +928,57 @@ __global__ __launch_bounds__(kBigThreads) void gemm_bf16x3_big_kernel(float* c, 
             }
 }
 
-// 256 x 256 tiles, one workgroup per CU: when they fill the CUs about as evenly as 128 x 128 tiles at two per CU would
-bool use_big_tiles(int64_t M, int64_t N, int64_t batch) {
-    static const int mode = [] { const char* e = getenv("DNH_DOT_BIG"); return e ? atoi(e) : -1; }();   // 0 / 1 force the choice
-    if (mode >= 0) return mode != 0;
-    const int64_t cus = device_cus();
-    const int64_t big = cdiv(M, (int64_t)XBM) * cdiv(N, (int64_t)XBN) * batch, small = cdiv(M, (int64_t)BM) * cdiv(N, (int64_t)BN) * batch;
-    const double eff_big = (double)big / (double)(cdiv(big, cus) * cus), eff_small = (double)small / (double)(cdiv(small, 2 * cus) * 2 * cus);
-    const double waste_big = (double)(M * N * batch) / ((double)big * XBM * XBN), waste_small = (double)(M * N * batch) / ((double)small * BM * BN);
-    return eff_big * waste_big * 1.1 >= eff_small * waste_small;
-}
-
 bool use_bf16x3() {
     static const bool on = [] { const char* e = getenv("DNH_DOT_BF16X3"); return !e || e[0] != '0'; }();
     return on;
+}
+
+// Tile form and number of K chunks of a product on the bf16-parts kernels: the cheapest of both forms at 1 .. 32 chunks under a
+// model of the two kernels fitted to measurements (1000^3 .. 4096^3, 512 x 8192 x 512, 4 .. 64 x 512^3 / 1024^3: the model's pick is
+// the measured best or within 9 % of it).  Per K step of 16: 128 x 128 tiles take 1.56 us with two workgroups on a CU, 1.09 - 1.29 us
+// with one (the more CUs are busy, the lower the clock); 256 x 256 tiles take 1.75 - 2.5 us at one per CU.  A workgroup costs 8 / 10 us
+// on top (launch, first fetch, epilogue), the summing launch 5 us plus its traffic at 5 TB/s.  DNH_DOT_BIG=0 / 1 and DNH_DOT_SPLITS=n
+// in the environment force either choice (for measurements and tests).
+void choose_x3_plan(int64_t M, int64_t N, int64_t batch, int64_t steps, bool can_split, bool* big, int64_t* want) {
+    static const int force_big = [] { const char* e = getenv("DNH_DOT_BIG"); return e ? atoi(e) : -1; }();
+    static const int force_splits = [] { const char* e = getenv("DNH_DOT_SPLITS"); return e ? atoi(e) : 0; }();
+    const int64_t cus = device_cus();
+    const int64_t nbig = cdiv(M, (int64_t)XBM) * cdiv(N, (int64_t)XBN) * batch, nsmall = cdiv(M, (int64_t)BM) * cdiv(N, (int64_t)BN) * batch;
+    const double out_bytes = (double)batch * (double)M * (double)N * 4.0;
+    auto cost = [&](bool bg, int64_t sp) {
+        const int64_t chunk = cdiv(steps, sp), real = cdiv(steps, chunk);
+        const int64_t n = (bg ? nbig : nsmall) * real;
+        double us;
+        if (bg) {
+            const int64_t full = n / cus, rem = n % cus;
+            us = (double)full * ((double)chunk * 2.5 + 10.0) + (rem ? (double)chunk * (1.75 + 0.75 * (double)rem / (double)cus) + 10.0 : 0.0);
+        } else {
+            const int64_t full = n / (2 * cus), rem = n % (2 * cus);
+            const double ts = rem <= cus ? 1.09 + 0.2 * (double)rem / (double)cus : 1.29 + 0.27 * (double)(rem - cus) / (double)cus;
+            us = (double)full * ((double)chunk * 1.56 + 8.0) + (rem ? (double)chunk * ts + 8.0 : 0.0);
+        }
+        if (real > 1) us = (us + 5.0 + (double)(real + 1) * out_bytes / 5.0e6) * 1.03;   // a split must pay for itself
+        return us;
+    };
+    // chunks of at least 4 steps; the partial sums of a split stay below 32 x 64 MB
+    const int64_t max_sp = (can_split && nsmall <= 4 * cus) ? std::min<int64_t>(32, steps / 4) : 1;
+    bool best_big = false;
+    int64_t best_sp = 1;
+    double best = -1.0;
+    for (int form = 0; form < 2; form++) {
+        if (force_big >= 0 && form != (force_big ? 1 : 0)) continue;
+        for (int64_t sp = 1; sp <= std::max<int64_t>(max_sp, 1); sp++) {
+            const double us = cost(form == 1, sp);
+            if (best < 0.0 || us < best) {
+                best = us;
+                best_big = form == 1;
+                best_sp = sp;
+            }
+        }
+    }
+    if (force_splits > 0 && can_split && batch * M * N < (1ll << 31)) best_sp = std::min<int64_t>(force_splits, std::max<int64_t>(steps / 2, 1));
+    *big = best_big;
+    *want = best_sp;
 }
 
 template <class T>
@@ -956,8 +996,30 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
     T* target = c;
     int64_t splits = 1;
     const int64_t steps = (g.K + kBK<T> - 1) / kBK<T>;
-    const int64_t want = (g.nbatch < DNH_MAX_DIMS && blocks <= 4 * (int64_t)device_cus()) ? choose_k_splits<T>(blocks, steps, batch * g.M * g.N) : 1;
-    if (want > 1) {   // implies steps >= 8: the chunk below is not empty
+    bool x3 = false, big = false;
+    bool a_kc = false, b_kc = false;
+    if constexpr (sizeof(T) == 4) {
+        // each operand either k-contiguous with 16-byte aligned rows, or contiguous along its other dimension
+        a_kc = g.sak == 1 && (g.sam % 4) == 0 && aligned_to(a, 16);
+        b_kc = g.sbk == 1 && (g.sbn % 4) == 0 && aligned_to(b, 16);
+        for (int d = 0; d < g.nbatch; d++) {
+            a_kc = a_kc && (g.bsa[d] % 4) == 0;
+            b_kc = b_kc && (g.bsb[d] % 4) == 0;
+        }
+        x3 = g.K >= kX3BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_bf16x3();
+    }
+    int64_t want = 1;
+    if (x3) {
+        choose_x3_plan(g.M, g.N, batch, steps, g.nbatch < DNH_MAX_DIMS, &big, &want);
+        if (big) {
+            g.tiles_m = (uint32_t)cdiv(g.M, (int64_t)XBM);
+            g.tiles_n = (uint32_t)cdiv(g.N, (int64_t)XBN);
+            blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
+        }
+    } else if (g.nbatch < DNH_MAX_DIMS && blocks <= 4 * (int64_t)device_cus()) {
+        want = choose_k_splits<T>(blocks, steps, batch * g.M * g.N);
+    }
+    if (want > 1) {   // the choosers keep chunks of at least 2 steps: the chunk below is not empty
         const int64_t kchunk = ((steps + want - 1) / want) * kBK<T>;
         splits = (g.K + kchunk - 1) / kchunk;
         if (splits > 1) {
@@ -987,41 +1049,23 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
                                else { if (b_kc) DNH_X3_LAUNCH(SP, TL, false, true); else DNH_X3_LAUNCH(SP, TL, false, false); } } while (0)
 #define DNH_X3(SP) do { if (g.K % kX3BK) DNH_X3_AB(SP, true); else DNH_X3_AB(SP, false); } while (0)
 #define DNH_GEMM(FASTF, ACCF, SPLITF) hipLaunchKernelGGL((gemm_kernel<T, FASTF, ACCF, SPLITF>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, c, a, b, g)
-    bool x3 = false;
-    bool a_kc = false, b_kc = false;
-    if constexpr (sizeof(T) == 4) {
-        // each operand either k-contiguous with 16-byte aligned rows, or contiguous along its other dimension
-        a_kc = g.sak == 1 && (g.sam % 4) == 0 && aligned_to(a, 16);
-        b_kc = g.sbk == 1 && (g.sbn % 4) == 0 && aligned_to(b, 16);
-        for (int d = 0; d < orig.nbatch; d++) {
-            a_kc = a_kc && (orig.bsa[d] % 4) == 0;
-            b_kc = b_kc && (orig.bsb[d] % 4) == 0;
-        }
-        x3 = g.K >= kX3BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_bf16x3();
-    }
     g.xcd_2d = (x3 && g.nbatch == 0 && (g.tiles_m % 2u) == 0 && (g.tiles_n % 4u) == 0 && blocks >= 64) ? 1u : 0u;
+#define DNH_BIG_LAUNCH(SP, TL, AK, BK_) do { \
+        static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_bf16x3_big_kernel<SP, TL, AK, BK_>), \
+                                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLdsBytes); \
+        if (attr != hipSuccess) return fail(DNH_ERR_HIP, "dnh_dot: %s", hipGetErrorString(attr)); \
+        hipLaunchKernelGGL((gemm_bf16x3_big_kernel<SP, TL, AK, BK_>), dim3((unsigned)blocks), dim3(kBigThreads), kBigLdsBytes, stream, c, a, b, g); } while (0)
+#define DNH_BIG_AB(SP, TL) do { if (a_kc) { if (b_kc) DNH_BIG_LAUNCH(SP, TL, true, true); else DNH_BIG_LAUNCH(SP, TL, true, false); } \
+                                else { if (b_kc) DNH_BIG_LAUNCH(SP, TL, false, true); else DNH_BIG_LAUNCH(SP, TL, false, false); } } while (0)
+#define DNH_BIG(SP) do { if (g.K % kX3BK) DNH_BIG_AB(SP, true); else DNH_BIG_AB(SP, false); } while (0)
     if constexpr (sizeof(T) == 4) {
-        if (x3 && splits == 1 && use_big_tiles(g.M, g.N, batch)) {
-            g.tiles_m = (uint32_t)cdiv(g.M, (int64_t)XBM);
-            g.tiles_n = (uint32_t)cdiv(g.N, (int64_t)XBN);
-            blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
-            g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
-            g.xcd_2d = (g.nbatch == 0 && (g.tiles_m % 2u) == 0 && (g.tiles_n % 4u) == 0 && blocks >= 64) ? 1u : 0u;
-#define DNH_BIG_LAUNCH(TL, AK, BK_) do { \
-                static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_bf16x3_big_kernel<TL, AK, BK_>), \
-                                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLdsBytes); \
-                if (attr != hipSuccess) return fail(DNH_ERR_HIP, "dnh_dot: %s", hipGetErrorString(attr)); \
-                hipLaunchKernelGGL((gemm_bf16x3_big_kernel<TL, AK, BK_>), dim3((unsigned)blocks), dim3(kBigThreads), kBigLdsBytes, stream, c, a, b, g); } while (0)
-#define DNH_BIG_AB(TL) do { if (a_kc) { if (b_kc) DNH_BIG_LAUNCH(TL, true, true); else DNH_BIG_LAUNCH(TL, true, false); } \
-                            else { if (b_kc) DNH_BIG_LAUNCH(TL, false, true); else DNH_BIG_LAUNCH(TL, false, false); } } while (0)
-            if (g.K % kX3BK) DNH_BIG_AB(true); else DNH_BIG_AB(false);
-#undef DNH_BIG_AB
-#undef DNH_BIG_LAUNCH
-            DNH_LAUNCH_CHECK();
-            return DNH_OK;
+        if (big) {
+            if (splits > 1) DNH_BIG(true); else DNH_BIG(false);
         }
     }
-    if (splits > 1) {
+    if (big) {
+        // launched above
+    } else if (splits > 1) {
         if (x3) {
             if constexpr (sizeof(T) == 4) DNH_X3(true);
         } else if (fast) DNH_GEMM(true, false, true);
@@ -1035,6 +1079,9 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         else DNH_GEMM(false, false, false);
     }
 #undef DNH_GEMM
+#undef DNH_BIG
+#undef DNH_BIG_AB
+#undef DNH_BIG_LAUNCH
 #undef DNH_X3
 #undef DNH_X3_AB
 #undef DNH_X3_LAUNCH
