@@ -933,18 +933,191 @@ bool use_bf16x3() {
     return on;
 }
 
-// Tile form and number of K chunks of a product on the bf16-parts kernels: the cheapest of both forms at 1 .. 32 chunks under a
-// model of the two kernels fitted to measurements (1000^3 .. 4096^3, 512 x 8192 x 512, 4 .. 64 x 512^3 / 1024^3: the model's pick is
-// the measured best or within 9 % of it).  Per K step of 16: 128 x 128 tiles take 1.56 us with two workgroups on a CU, 1.09 - 1.29 us
-// with one (the more CUs are busy, the lower the clock); 256 x 256 tiles take 1.75 - 2.5 us at one per CU.  A workgroup costs 8 / 10 us
-// on top (launch, first fetch, epilogue), the summing launch 5 us plus its traffic at 5 TB/s.  DNH_DOT_BIG=0 / 1 and DNH_DOT_SPLITS=n
-// in the environment force either choice (for measurements and tests).
-void choose_x3_plan(int64_t M, int64_t N, int64_t batch, int64_t steps, bool can_split, bool* big, int64_t* want) {
+// ---- double precision with a pinned instruction order ------------------------------------------------------------------------
+// The 128 x 128 tile of gemm_kernel<double> (K step 8, sixteen 16 x 16 accumulators per wavefront on v_mfma_f64_16x16x4_f64) for
+// operands that are each contiguous along one of their two dimensions, with the loop written as the bf16-parts kernels write theirs:
+// branch-free fetches of the next K step first (rows beyond the matrix read row 0 and are zeroed on their way to LDS), then the 32
+// matrix instructions with the second half's LDS reads behind the first eight and the LDS writes of the fetched elements behind the
+// last sixteen, one barrier per step.  gemm_kernel keeps the other layouts and the accumulating form.
+constexpr int kF64BK = 8;
+
+// Staging of one operand tile (128 rows x 8 k) by 256 threads: four doubles per thread.
+//   KC (k contiguous, 16-byte aligned rows): four lanes cover the 8 k of a row with one 16-byte load each; a thread takes rows r, r + 64.
+//   otherwise (rows contiguous): a thread takes one row and 4 consecutive k with element loads (a wavefront reads 512 contiguous bytes).
+template <bool KC>
+struct F64Stage {
+    int row, kofs;
+    bool ok0, ok1;
+    const double *p0, *p1;
+    int64_t ks;
+    __device__ __forceinline__ void init(const double* base, int64_t row0, int64_t limit, int64_t rs, int64_t kstride, int tid) {
+        row = KC ? tid >> 2 : tid & 127;
+        kofs = KC ? (tid & 3) * 2 : (tid >> 7) * 4;
+        ok0 = row0 + row < limit;
+        ok1 = KC && row0 + row + 64 < limit;
+        p0 = base + (ok0 ? (row0 + row) * rs : 0);
+        p1 = base + (ok1 ? (row0 + row + 64) * rs : 0);
+        ks = KC ? 1 : kstride;
+    }
+    template <bool TAIL>
+    __device__ __forceinline__ void load(int64_t k0, int64_t K, double (&r)[4]) const {
+        if (!TAIL || k0 + kF64BK <= K) {
+            if constexpr (KC) {
+                const Pack<double, 2> v0 = load_pack<double, 2>(p0 + k0 + kofs), v1 = load_pack<double, 2>(p1 + k0 + kofs);
+                r[0] = v0.v[0];
+                r[1] = v0.v[1];
+                r[2] = v1.v[0];
+                r[3] = v1.v[1];
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; e++) r[e] = p0[(k0 + kofs + e) * ks];
+            }
+        } else {
+            // the partial last K step: element loads from addresses clamped into the row, zeros beyond K
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int64_t k = k0 + kofs + (KC ? (e & 1) : e);
+                const double* p = (KC && e >= 2) ? p1 : p0;
+                const double v = p[(k < K ? k : K - 1) * ks];
+                r[e] = k < K ? v : 0.0;
+            }
+        }
+    }
+    // element e of the staged four goes to tile[k][row]
+    template <int E>
+    __device__ __forceinline__ void put(const double (&r)[4], double (*tile)[BM + PAD]) const {
+        const double v = ((KC && E >= 2) ? ok1 : ok0) ? r[E] : 0.0;
+        if constexpr (KC) tile[kofs + (E & 1)][row + (E >> 1) * 64] = v;
+        else tile[kofs + E][row] = v;
+    }
+    __device__ __forceinline__ void store(const double (&r)[4], double (*tile)[BM + PAD]) const {
+        put<0>(r, tile);
+        put<1>(r, tile);
+        put<2>(r, tile);
+        put<3>(r, tile);
+    }
+};
+
+template <bool SPLIT, bool TAIL, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kBlock, 2) void gemm_f64_kernel(double* c, const double* a, const double* b, GemmArgs g) {
+    __shared__ __align__(16) double As[2][kF64BK][BM + PAD];
+    __shared__ __align__(16) double Bs[2][kF64BK][BN + PAD];
+
+    uint32_t bid = blockIdx.x;
+    if (g.xcd_chunk) bid = (bid % 8u) * g.xcd_chunk + bid / 8u;
+    const uint32_t tn = bid % g.tiles_n;
+    bid /= g.tiles_n;
+    const uint32_t tm = bid % g.tiles_m;
+    bid /= g.tiles_m;
+    int64_t oa = 0, ob = 0, oc = 0;
+    uint32_t chunk_id = 0;
+    for (int d = g.nbatch - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
+        const uint32_t i = bid - q * g.bshape[d];
+        bid = q;
+        oa += (int64_t)i * g.bsa[d];
+        ob += (int64_t)i * g.bsb[d];
+        oc += (int64_t)i * g.bsc[d];
+        if (SPLIT && d == g.nbatch - 1) chunk_id = i;
+    }
+    const int64_t K = SPLIT ? min(g.kchunk, g.K - (int64_t)chunk_id * g.kchunk) : g.K;
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    a += oa;
+    b += ob;
+    c += oc;
+    const int tid = threadIdx.x;
+
+    F64Stage<A_KC> sa;
+    F64Stage<B_KC> sb;
+    sa.init(a, m0, g.M, g.sam, g.sak, tid);
+    sb.init(b, n0, g.N, g.sbn, g.sbk, tid);
+    double ra[4], rb[4];
+
+    // operand lane l supplies A[l % 16][l / 16] and B[l / 16][l % 16]; accumulator register r of lane l holds row 4 r + l / 16,
+    // column l % 16 of its 16 x 16 tile
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
+    const int lk = lane >> 4, lm = lane & 15;
+    f64x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) acc[i][j][r] = 0.0;
+
+    int cur = 0;
+    auto k_step = [&](auto next_tag, auto tail_tag, int64_t k_next) {
+        constexpr bool NEXT = decltype(next_tag)::value, TL = decltype(tail_tag)::value;
+        if constexpr (NEXT) {
+            sa.template load<TL>(k_next, K, ra);
+            sb.template load<TL>(k_next, K, rb);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        double av[2][4], bv[2][4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) av[0][i] = As[cur][lk][wm + i * 16 + lm];
+#pragma unroll
+        for (int j = 0; j < 4; j++) bv[0][j] = Bs[cur][lk][wn + j * 16 + lm];
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<32>([&](auto tt) {
+            constexpr int t = decltype(tt)::value, h = t / 16, i = (t % 16) / 4, j = t % 4;
+            acc[i][j] = __builtin_amdgcn_mfma_f64_16x16x4f64(av[h][i], bv[h][j], acc[i][j], 0, 0, 0);
+            if constexpr (t < 4) av[1][t] = As[cur][4 + lk][wm + t * 16 + lm];
+            else if constexpr (t < 8) bv[1][t - 4] = Bs[cur][4 + lk][wn + (t - 4) * 16 + lm];
+            if constexpr (NEXT && t >= 16 && t < 32 && t % 2 == 0) {
+                constexpr int q = (t - 16) / 2;   // eight elements: four of A, four of B
+                if constexpr (q < 4) sa.template put<q>(ra, As[cur ^ 1]);
+                else sb.template put<q - 4>(rb, Bs[cur ^ 1]);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (NEXT) {
+            __syncthreads();
+            cur ^= 1;
+        }
+    };
+    const int64_t nsteps = (K + kF64BK - 1) / kF64BK;
+    sa.template load<TAIL>(0, K, ra);
+    sb.template load<TAIL>(0, K, rb);
+    sa.store(ra, As[0]);
+    sb.store(rb, Bs[0]);
+    __syncthreads();
+    for (int64_t s = 0; s + 2 < nsteps; s++) k_step(std::true_type(), std::false_type(), (s + 1) * kF64BK);
+    if (nsteps >= 2) k_step(std::true_type(), std::integral_constant<bool, TAIL>(), (nsteps - 1) * kF64BK);
+    k_step(std::false_type(), std::false_type(), 0);
+
+    const bool full_mn = m0 + BM <= g.M && n0 + BN <= g.N;
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const int64_t m = m0 + wm + i * 16 + 4 * r + lk, n = n0 + wn + j * 16 + lm;
+                if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = acc[i][j][r];
+            }
+}
+
+bool use_f64_pinned() {
+    static const bool on = [] { const char* e = getenv("DNH_DOT_F64_PINNED"); return !e || e[0] != '0'; }();   // 0: gemm_kernel<double> for every layout
+    return on;
+}
+
+// Tile form and number of K chunks of a product on the kernels with a pinned instruction order: the cheapest of the available forms
+// at 1 .. 32 chunks under a model fitted to measurements (1000^3 .. 4096^3, 512 x 8192 x 512, 2048 x 512 x 2048, 4 .. 64 x 512^3 /
+// 1024^3: the model's pick is the measured best or within 9 % of it).  Per K step, in microseconds:
+//   bf16 parts (K step 16), 128 x 128 tiles: 1.56 with two workgroups on a CU, 1.09 - 1.29 with one (the more CUs are busy, the
+//       lower the clock); 256 x 256 tiles, one per CU: 1.75 - 2.5;
+//   double precision (K step 8), 128 x 128 tiles: 2.05 with two workgroups on a CU, 1.10 - 1.26 with one.
+// A round of workgroups costs 8 / 10 / 13 us on top (launch, first fetch, epilogue), the summing launch 5 us plus its traffic at
+// 5 TB/s.  DNH_DOT_BIG=0 / 1 and DNH_DOT_SPLITS=n in the environment force either choice (for measurements and tests).
+void choose_plan(bool f64, int64_t M, int64_t N, int64_t batch, int64_t steps, bool can_split, bool* big, int64_t* want) {
     static const int force_big = [] { const char* e = getenv("DNH_DOT_BIG"); return e ? atoi(e) : -1; }();
     static const int force_splits = [] { const char* e = getenv("DNH_DOT_SPLITS"); return e ? atoi(e) : 0; }();
     const int64_t cus = device_cus();
     const int64_t nbig = cdiv(M, (int64_t)XBM) * cdiv(N, (int64_t)XBN) * batch, nsmall = cdiv(M, (int64_t)BM) * cdiv(N, (int64_t)BN) * batch;
-    const double out_bytes = (double)batch * (double)M * (double)N * 4.0;
+    const double out_bytes = (double)batch * (double)M * (double)N * (f64 ? 8.0 : 4.0);
     auto cost = [&](bool bg, int64_t sp) {
         const int64_t chunk = cdiv(steps, sp), real = cdiv(steps, chunk);
         const int64_t n = (bg ? nbig : nsmall) * real;
@@ -954,19 +1127,21 @@ void choose_x3_plan(int64_t M, int64_t N, int64_t batch, int64_t steps, bool can
             us = (double)full * ((double)chunk * 2.5 + 10.0) + (rem ? (double)chunk * (1.75 + 0.75 * (double)rem / (double)cus) + 10.0 : 0.0);
         } else {
             const int64_t full = n / (2 * cus), rem = n % (2 * cus);
-            const double ts = rem <= cus ? 1.09 + 0.2 * (double)rem / (double)cus : 1.29 + 0.27 * (double)(rem - cus) / (double)cus;
-            us = (double)full * ((double)chunk * 1.56 + 8.0) + (rem ? (double)chunk * ts + 8.0 : 0.0);
+            const double r = (double)rem / (double)cus;
+            const double ts2 = f64 ? 2.05 : 1.56, fix = f64 ? 13.0 : 8.0;
+            const double ts = f64 ? (rem <= cus ? 1.10 + 0.16 * r : 1.26 + 0.79 * (r - 1.0)) : (rem <= cus ? 1.09 + 0.2 * r : 1.29 + 0.27 * (r - 1.0));
+            us = (double)full * ((double)chunk * ts2 + fix) + (rem ? (double)chunk * ts + fix : 0.0);
         }
         if (real > 1) us = (us + 5.0 + (double)(real + 1) * out_bytes / 5.0e6) * 1.03;   // a split must pay for itself
         return us;
     };
-    // chunks of at least 4 steps; the partial sums of a split stay below 32 x 64 MB
+    // chunks of at least 4 steps; the partial sums of a split stay below 32 x 64 (128) MB
     const int64_t max_sp = (can_split && nsmall <= 4 * cus) ? std::min<int64_t>(32, steps / 4) : 1;
     bool best_big = false;
     int64_t best_sp = 1;
     double best = -1.0;
-    for (int form = 0; form < 2; form++) {
-        if (force_big >= 0 && form != (force_big ? 1 : 0)) continue;
+    for (int form = 0; form < (f64 ? 1 : 2); form++) {
+        if (!f64 && force_big >= 0 && form != (force_big ? 1 : 0)) continue;
         for (int64_t sp = 1; sp <= std::max<int64_t>(max_sp, 1); sp++) {
             const double us = cost(form == 1, sp);
             if (best < 0.0 || us < best) {
@@ -1008,9 +1183,19 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         }
         x3 = g.K >= kX3BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_bf16x3();
     }
+    bool f64p = false;   // double precision on gemm_f64_kernel: each operand contiguous along one of its dimensions
+    if constexpr (sizeof(T) == 8) {
+        a_kc = g.sak == 1 && (g.sam % 2) == 0 && aligned_to(a, 16);
+        b_kc = g.sbk == 1 && (g.sbn % 2) == 0 && aligned_to(b, 16);
+        for (int d = 0; d < g.nbatch; d++) {
+            a_kc = a_kc && (g.bsa[d] % 2) == 0;
+            b_kc = b_kc && (g.bsb[d] % 2) == 0;
+        }
+        f64p = g.K >= kF64BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_f64_pinned();
+    }
     int64_t want = 1;
-    if (x3) {
-        choose_x3_plan(g.M, g.N, batch, steps, g.nbatch < DNH_MAX_DIMS, &big, &want);
+    if (x3 || f64p) {
+        choose_plan(f64p, g.M, g.N, batch, steps, g.nbatch < DNH_MAX_DIMS, &big, &want);
         if (big) {
             g.tiles_m = (uint32_t)cdiv(g.M, (int64_t)XBM);
             g.tiles_n = (uint32_t)cdiv(g.N, (int64_t)XBN);
@@ -1018,6 +1203,8 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         }
     } else if (g.nbatch < DNH_MAX_DIMS && blocks <= 4 * (int64_t)device_cus()) {
         want = choose_k_splits<T>(blocks, steps, batch * g.M * g.N);
+        static const int force_splits = [] { const char* e = getenv("DNH_DOT_SPLITS"); return e ? atoi(e) : 0; }();
+        if (force_splits > 0) want = std::min<int64_t>(force_splits, std::max<int64_t>(steps / 2, 1));
     }
     if (want > 1) {   // the choosers keep chunks of at least 2 steps: the chunk below is not empty
         const int64_t kchunk = ((steps + want - 1) / want) * kBK<T>;
@@ -1063,7 +1250,19 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
             if (splits > 1) DNH_BIG(true); else DNH_BIG(false);
         }
     }
-    if (big) {
+#define DNH_F64_LAUNCH(SP, TL, AK, BK_) hipLaunchKernelGGL((gemm_f64_kernel<SP, TL, AK, BK_>), dim3((unsigned)blocks), dim3(kBlock), 0, stream, (double*)c, (const double*)a, (const double*)b, g)
+#define DNH_F64_AB(SP, TL) do { if (a_kc) { if (b_kc) DNH_F64_LAUNCH(SP, TL, true, true); else DNH_F64_LAUNCH(SP, TL, true, false); } \
+                                else { if (b_kc) DNH_F64_LAUNCH(SP, TL, false, true); else DNH_F64_LAUNCH(SP, TL, false, false); } } while (0)
+#define DNH_F64(SP) do { if (g.K % kF64BK) DNH_F64_AB(SP, true); else DNH_F64_AB(SP, false); } while (0)
+    if constexpr (sizeof(T) == 8) {
+        if (f64p) {
+            if (splits > 1) DNH_F64(true); else DNH_F64(false);
+        }
+    }
+#undef DNH_F64
+#undef DNH_F64_AB
+#undef DNH_F64_LAUNCH
+    if (big || f64p) {
         // launched above
     } else if (splits > 1) {
         if (x3) {
