@@ -218,7 +218,16 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_finish_kernel(R r, const t
     State st = r.init();
     if (col < nc) {
         const State* p = partial + (int64_t)other * splits * nc + col;
-        for (uint32_t s = y; s < splits; s += NY) st = r.combine(st, p[(int64_t)s * nc]);
+        constexpr uint32_t U = 8;   // loads in flight per thread; combined in split order
+        uint32_t s = y;
+        for (; s + (U - 1) * NY < splits; s += U * NY) {
+            State v[U];
+#pragma unroll
+            for (uint32_t u = 0; u < U; u++) v[u] = p[(int64_t)(s + u * NY) * nc];
+#pragma unroll
+            for (uint32_t u = 0; u < U; u++) st = r.combine(st, v[u]);
+        }
+        for (; s < splits; s += NY) st = r.combine(st, p[(int64_t)s * nc]);
     }
     __shared__ State sh[NY][WX];
     sh[y][x] = st;
@@ -430,7 +439,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
 #undef DNH_COLS
             DNH_LAUNCH_CHECK();
             if (splits > 1) {
-                constexpr int FW = 16;
+                constexpr int FW = 32;   // (16 and 64 columns per finishing workgroup measured 1-2 % slower on 8192 x 8192)
                 const uint32_t ftiles = cdiv(nc, FW);
                 hipLaunchKernelGGL((reduce_cols_finish_kernel<R, FW>), dim3(ftiles * others), dim3(kBlock), 0, stream, r, (const State*)partial, out,
                                    oo, ftiles, nc, tc_stride, splits);

@@ -444,3 +444,30 @@ def test_large_tile_kernel_on_every_shape_of_this_file():
                           "-k", "single_precision or matmat or batched or split_k or config5"],
                          env=env, cwd=root, capture_output=True, text=True, timeout=900)
     assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-2000:]
+
+
+@pytest.mark.parametrize("ta,tb", STAGINGS)
+@pytest.mark.parametrize("m,k,n", [(256, 8, 256), (257, 100, 130), (1100, 44, 1500), (300, 2049, 200)])
+def test_double_precision_stagings(H, G, rng, ta, tb, m, k, n):
+    """Double precision with row-major or transposed operands (the kernel's two stagings per operand), whole and partial K steps,
+    edge tiles, one launch or chunks along K: IEEE products and sums in some order, so the K-term bound against the oracle and
+    the exact product; an operand strided in both dimensions takes the general kernel and must agree as well."""
+    a = rng.standard_normal((m, k))
+    b = rng.standard_normal((k, n))
+    x, y = _views(G, a, b, ta, tb)
+    got = G.toNumpy(x @ y)
+    ref = H.toNumpy(H.ofNumpy(a) @ H.ofNumpy(b))
+    check_dot(ref, got, a, b)
+    a[3, 5], b[5, 7] = np.inf, 0.0
+    a[9, 1] = np.nan
+    x, y = _views(G, a, b, ta, tb)
+    got = G.toNumpy(x @ y)
+    with np.errstate(all="ignore"):
+        want = a @ b
+    assert np.array_equal(np.isnan(got), np.isnan(want)) and np.array_equal(np.isposinf(got), np.isposinf(want))
+    assert np.array_equal(np.isneginf(got), np.isneginf(want))
+    # one plane of a 3-d tensor: strided in both dimensions
+    wide = rng.standard_normal((m, k, 2))
+    b2 = np.where(np.isfinite(b), b, 0.0)
+    got = G.toNumpy(G.ofNumpy(wide)[:, :, 0] @ G.ofNumpy(b2))
+    check_dot(wide[:, :, 0] @ b2, got, wide[:, :, 0], b2)
