@@ -483,17 +483,16 @@ template <bool KC, int ROWS = BM>
 struct X3Stage {
     static constexpr int HALF = ROWS / 2;   // 2 * ROWS threads stage a tile
     int row, kofs;      // first row and first k of this thread inside the tile
-    bool ok0, ok1;      // row (and for KC row + 64) inside the matrix
-    const float *p0, *p1;   // element (row, k = 0) of those rows; row 0 of the matrix when outside
+    // element (row, k = 0) of this thread's rows (KC: row and row + ROWS / 2).  A row beyond the matrix reads row 0 instead: what it
+    // contributes lands in rows (columns) of the tile's result that lie beyond the matrix as well and are never stored.
+    const float *p0, *p1;
     int64_t ks;
     bool bad;           // an element staged so far is infinite or too small to cut into bf16 parts
     __device__ __forceinline__ void init(const float* base, int64_t row0, int64_t limit, int64_t rs, int64_t kstride, int tid) {
         row = KC ? tid >> 2 : tid & (ROWS - 1);
         kofs = KC ? (tid & 3) * 4 : (tid / ROWS) * 8;
-        ok0 = row0 + row < limit;
-        ok1 = KC && row0 + row + HALF < limit;
-        p0 = base + (ok0 ? (row0 + row) * rs : 0);
-        p1 = base + (ok1 ? (row0 + row + HALF) * rs : 0);
+        p0 = base + (row0 + row < limit ? (row0 + row) * rs : 0);
+        p1 = base + (KC && row0 + row + HALF < limit ? (row0 + row + HALF) * rs : 0);
         ks = KC ? 1 : kstride;
         bad = false;
     }
@@ -524,8 +523,6 @@ struct X3Stage {
     }
     // cuts the staged elements into their parts and writes them to tile[part][row][k]
     __device__ __forceinline__ void store(float (&r)[8], __bf16 (*tile)[ROWS][kX3Row]) {
-#pragma unroll
-        for (int e = 0; e < 8; e++) r[e] = ((KC && e >= 4) ? ok1 : ok0) ? r[e] : 0.0f;
         // +-inf stays infinite under the scaling; |x| < 2^-109 (x != 0) becomes denormal; zero stays zero
         constexpr int kClassInfOrDenormal = (1 << 2) | (1 << 4) | (1 << 7) | (1 << 9);
 #pragma unroll
@@ -551,8 +548,7 @@ struct X3Stage {
     __device__ __forceinline__ void piece(float (&r)[8], __bf16 (*tile)[ROWS][kX3Row]) {
         constexpr int e = Q / 2;
         if constexpr (Q % 2 == 0) {
-            const float v = ((KC && e >= 4) ? ok1 : ok0) ? r[e] : 0.0f;
-            r[e] = v;
+            const float v = r[e];
             const uint32_t h = __float_as_uint(v);
             const float r1 = v - __uint_as_float(h & 0xFFFF0000u);
             const uint32_t m = __float_as_uint(r1);
@@ -936,7 +932,7 @@ bool use_bf16x3() {
 // ---- double precision with a pinned instruction order ------------------------------------------------------------------------
 // The 128 x 128 tile of gemm_kernel<double> (K step 8, sixteen 16 x 16 accumulators per wavefront on v_mfma_f64_16x16x4_f64) for
 // operands that are each contiguous along one of their two dimensions, with the loop written as the bf16-parts kernels write theirs:
-// branch-free fetches of the next K step first (rows beyond the matrix read row 0 and are zeroed on their way to LDS), then the 32
+// branch-free fetches of the next K step first (rows beyond the matrix read row 0; their products are never stored), then the 32
 // matrix instructions with the second half's LDS reads behind the first eight and the LDS writes of the fetched elements behind the
 // last sixteen, one barrier per step.  gemm_kernel keeps the other layouts and the accumulating form.
 constexpr int kF64BK = 8;
@@ -947,16 +943,13 @@ constexpr int kF64BK = 8;
 template <bool KC>
 struct F64Stage {
     int row, kofs;
-    bool ok0, ok1;
-    const double *p0, *p1;
+    const double *p0, *p1;   // a row beyond the matrix reads row 0: its products land beyond the matrix too and are never stored
     int64_t ks;
     __device__ __forceinline__ void init(const double* base, int64_t row0, int64_t limit, int64_t rs, int64_t kstride, int tid) {
         row = KC ? tid >> 2 : tid & 127;
         kofs = KC ? (tid & 3) * 2 : (tid >> 7) * 4;
-        ok0 = row0 + row < limit;
-        ok1 = KC && row0 + row + 64 < limit;
-        p0 = base + (ok0 ? (row0 + row) * rs : 0);
-        p1 = base + (ok1 ? (row0 + row + 64) * rs : 0);
+        p0 = base + (row0 + row < limit ? (row0 + row) * rs : 0);
+        p1 = base + (KC && row0 + row + 64 < limit ? (row0 + row + 64) * rs : 0);
         ks = KC ? 1 : kstride;
     }
     template <bool TAIL>
@@ -986,7 +979,7 @@ struct F64Stage {
     // element e of the staged four goes to tile[k][row]
     template <int E>
     __device__ __forceinline__ void put(const double (&r)[4], double (*tile)[BM + PAD]) const {
-        const double v = ((KC && E >= 2) ? ok1 : ok0) ? r[E] : 0.0;
+        const double v = r[E];
         if constexpr (KC) tile[kofs + (E & 1)][row + (E >> 1) * 64] = v;
         else tile[kofs + E][row] = v;
     }
