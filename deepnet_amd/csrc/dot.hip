@@ -13,6 +13,9 @@
 //     reference's BLAS paths (Tensor/Tensor/BlasSupport.fs:173-190, Cuda/CudaBLAS.fs:28-38).
 // The "fast" instantiation (row-major, 16-byte aligned A and B) uses 16-byte global loads on interior tiles and guarded
 // scalar loads on edge tiles; every other layout runs the same kernel with guarded scalar loads throughout.
+// This kernel is the general form (operands strided in both dimensions, accumulation, K < one step).  Operands that are contiguous
+// along one of their dimensions take the kernels further down: gemm_bf16x3_kernel / gemm_bf16x3_big_kernel (single precision on the
+// bf16 matrix instructions) and gemm_f64_kernel (double precision), whose K loops have a hand-pinned instruction order.
 #include "map_kernels.h"
 
 using namespace dnh;
@@ -771,7 +774,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_bf16x3_kernel(float* __restric
 // The same product on 256 x 256 tiles: 512 threads = 8 wavefronts in a 2 x 4 arrangement, each owning 128 x 64 (eight 32 x 32
 // accumulators).  Against the 128 x 128 kernel every staged element (cut into parts once per workgroup that needs it) and every LDS
 // operand fetch feeds twice as many matrix instructions: 48 per wavefront and K step against 18 LDS reads and 16 staged elements.
-// One workgroup per CU (144 KB of LDS, two wavefronts per SIMD); chosen when the product has at least a CU's worth of such tiles.
+// One workgroup per CU (144 KB of LDS, two wavefronts per SIMD); choose_plan picks the form (and the chunks along K) per product.
 // The K loop keeps one shape per iteration (no branch inside: the last K step and the K tail are peeled), so that the cutting of the
 // next step's elements can be scheduled between the matrix instructions of the current one.
 constexpr int XBM = 256, XBN = 256, kBigThreads = 512;
