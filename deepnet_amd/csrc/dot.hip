@@ -1579,8 +1579,222 @@ __global__ __launch_bounds__(256) void gemm_int_kernel(T* __restrict__ c, const 
         }
 }
 
+// 32-bit integers on the int8 matrix instruction.  Modulo 2^32 an element is the sum of four signed bytes d_i 2^(8 i) (the bytes of
+// (u + 0x80808080) ^ 0x80808080: adding 128 to every byte with carries, then taking 128 off each byte), so a.b = sum over i, j of
+// 2^(8 (i + j)) sum_k da_i db_j, of which the ten terms with i + j <= 3 survive the modulus.  v_mfma_i32_32x32x32_i8 forms the byte
+// products exactly and adds them in int32, whose wrap-around is the modulus itself: one accumulator per shift i + j, combined at the
+// end as acc0 + (acc1 << 8) + (acc2 << 16) + (acc3 << 24).  Bit-identical to the wrapping multiply + sum of the host backend for any
+// K.  128 x 128 tile, K step 32, 512 threads = 8 wavefronts 2 x 4, each owning 64 x 32 (two 32 x 32 sub-tiles x four shifts); the four
+// byte planes of both operands lie in LDS k-contiguous, [plane][row][32 + 16 bytes], double buffered.  20 matrix instructions per
+// wavefront and K step replace 64 x 32 x 32 / 64 lanes = 1024 integer multiply-adds per lane.
+typedef int i32x4v __attribute__((ext_vector_type(4)));
+typedef int i32x16v __attribute__((ext_vector_type(16)));
+constexpr int kI8BK = 32, kI8Row = 48, kI8Threads = 512;
+constexpr size_t kI8LdsBytes = (size_t)2 * 2 * 4 * BM * kI8Row;
+
+// four elements (consecutive k) -> one dword of each byte plane
+__device__ __forceinline__ void cut4_i8(const uint32_t (&w)[4], uint32_t (&plane)[4]) {
+    uint32_t d[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) d[e] = (w[e] + 0x80808080u) ^ 0x80808080u;
+    const uint32_t lo01 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);
+    const uint32_t lo23 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+    plane[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+    plane[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+    plane[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+    plane[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+}
+
+// Staging of one operand tile (128 rows x 32 k) by 512 threads, eight elements per thread.
+//   KC (k contiguous, 16-byte aligned rows): eight lanes cover the 32 k of a row with one 16-byte load each; a thread takes rows r, r + 64.
+//   otherwise (rows contiguous): a thread takes one row and 8 consecutive k with element loads.
+template <bool KC>
+struct I8Stage {
+    int row, kofs;
+    const uint32_t *p0, *p1;   // a row beyond the matrix reads row 0: its products land beyond the matrix too and are never stored
+    int64_t ks;
+    __device__ __forceinline__ void init(const uint32_t* base, int64_t row0, int64_t limit, int64_t rs, int64_t kstride, int tid) {
+        row = KC ? tid >> 3 : tid & 127;
+        kofs = KC ? (tid & 7) * 4 : (tid >> 7) * 8;
+        p0 = base + (row0 + row < limit ? (row0 + row) * rs : 0);
+        p1 = base + (KC && row0 + row + 64 < limit ? (row0 + row + 64) * rs : 0);
+        ks = KC ? 1 : kstride;
+    }
+    template <bool TAIL>
+    __device__ __forceinline__ void load(int64_t k0, int64_t K, uint32_t (&r)[8]) const {
+        if (!TAIL || k0 + kI8BK <= K) {
+            if constexpr (KC) {
+                typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+                const u32x4v v0 = *reinterpret_cast<const u32x4v*>(p0 + k0 + kofs), v1 = *reinterpret_cast<const u32x4v*>(p1 + k0 + kofs);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    r[e] = v0[e];
+                    r[4 + e] = v1[e];
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) r[e] = p0[(k0 + kofs + e) * ks];
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                const int64_t k = k0 + kofs + (KC ? (e & 3) : e);
+                const uint32_t* p = (KC && e >= 4) ? p1 : p0;
+                const uint32_t v = p[(k < K ? k : K - 1) * ks];
+                r[e] = k < K ? v : 0u;
+            }
+        }
+    }
+    __device__ __forceinline__ void store(const uint32_t (&r)[8], unsigned char (*tile)[BM][kI8Row]) const {
+        uint32_t w0[4] = {r[0], r[1], r[2], r[3]}, w1[4] = {r[4], r[5], r[6], r[7]}, q0[4], q1[4];
+        cut4_i8(w0, q0);
+        cut4_i8(w1, q1);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            if constexpr (KC) {
+                *reinterpret_cast<uint32_t*>(&tile[s][row][kofs]) = q0[s];
+                *reinterpret_cast<uint32_t*>(&tile[s][row + 64][kofs]) = q1[s];
+            } else {
+                typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+                *reinterpret_cast<u32x2*>(&tile[s][row][kofs]) = u32x2{q0[s], q1[s]};
+            }
+        }
+    }
+};
+
+template <bool TAIL, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kI8Threads) void gemm_i32_i8parts_kernel(uint32_t* c, const uint32_t* a, const uint32_t* b, GemmArgs g) {
+    extern __shared__ __align__(16) unsigned char i8_lds[];
+    typedef unsigned char (*Tiles)[4][BM][kI8Row];                 // [buffer][plane][row][k]
+    Tiles As = reinterpret_cast<Tiles>(i8_lds);
+    Tiles Bs = reinterpret_cast<Tiles>(i8_lds + kI8LdsBytes / 2);
+
+    uint32_t bid = blockIdx.x;
+    if (g.xcd_chunk) bid = (bid % 8u) * g.xcd_chunk + bid / 8u;
+    const uint32_t tn = bid % g.tiles_n;
+    bid /= g.tiles_n;
+    const uint32_t tm = bid % g.tiles_m;
+    bid /= g.tiles_m;
+    int64_t oa = 0, ob = 0, oc = 0;
+    for (int d = g.nbatch - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
+        const uint32_t i = bid - q * g.bshape[d];
+        bid = q;
+        oa += (int64_t)i * g.bsa[d];
+        ob += (int64_t)i * g.bsb[d];
+        oc += (int64_t)i * g.bsc[d];
+    }
+    const int64_t K = g.K;
+    const int64_t m0 = (int64_t)tm * BM, n0 = (int64_t)tn * BN;
+    a += oa;
+    b += ob;
+    c += oc;
+    const int tid = threadIdx.x;
+
+    I8Stage<A_KC> sa;
+    I8Stage<B_KC> sb;
+    sa.init(a, m0, g.M, g.sam, g.sak, tid);
+    sb.init(b, n0, g.N, g.sbn, g.sbk, tid);
+    uint32_t ra[8], rb[8];
+
+    // operand lane l supplies 16 consecutive k (16 (l / 32) ...) of row l % 32; accumulator register r of lane l holds row
+    // 8 (r / 4) + 4 (l / 32) + r % 4, column l % 32 of its 32 x 32 tile (as the other 32 x 32 matrix instructions)
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 2) * 64, wn = (wave & 3) * 32;
+    const int lm = lane & 31, lk = lane >> 5;
+    i32x16v acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int s = 0; s < 4; s++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][s][r] = 0;
+
+    int cur = 0;
+    auto compute = [&]() {
+        i32x4v av[2][4], bv[4];
+#pragma unroll
+        for (int s = 0; s < 4; s++) bv[s] = *reinterpret_cast<const i32x4v*>(&Bs[cur][s][wn + lm][lk * 16]);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int s = 0; s < 4; s++) av[i][s] = *reinterpret_cast<const i32x4v*>(&As[cur][s][wm + i * 32 + lm][lk * 16]);
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int sh = 0; sh < 4; sh++)
+#pragma unroll
+                for (int pa = 0; pa <= sh; pa++)
+                    acc[i][sh] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i][pa], bv[sh - pa], acc[i][sh], 0, 0, 0);
+    };
+
+    const int64_t nsteps = (K + kI8BK - 1) / kI8BK;
+    sa.template load<TAIL>(0, K, ra);
+    sb.template load<TAIL>(0, K, rb);
+    sa.store(ra, As[0]);
+    sb.store(rb, Bs[0]);
+    __syncthreads();
+    for (int64_t s = 0; s + 1 < nsteps; s++) {
+        sa.template load<TAIL>((s + 1) * kI8BK, K, ra);
+        sb.template load<TAIL>((s + 1) * kI8BK, K, rb);
+        __builtin_amdgcn_sched_barrier(0);   // the fetches stay in front of the matrix instructions
+        compute();
+        sa.store(ra, As[cur ^ 1]);
+        sb.store(rb, Bs[cur ^ 1]);
+        __syncthreads();
+        cur ^= 1;
+    }
+    compute();
+
+    const bool full_mn = m0 + BM <= g.M && n0 + BN <= g.N;
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int64_t m = m0 + wm + i * 32 + (r >> 2) * 8 + lk * 4 + (r & 3);
+            const int64_t n = n0 + wn + lm;
+            const uint32_t v = (uint32_t)acc[i][0][r] + ((uint32_t)acc[i][1][r] << 8) + ((uint32_t)acc[i][2][r] << 16) + ((uint32_t)acc[i][3][r] << 24);
+            if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = v;
+        }
+}
+
+bool use_int_mfma() {
+    static const bool on = [] { const char* e = getenv("DNH_DOT_INT_MFMA"); return !e || e[0] != '0'; }();   // 0: every integer product on gemm_int_kernel
+    return on;
+}
+
 template <class T>
 int32_t launch_gemm_int(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hipStream_t stream) {
+    if constexpr (sizeof(T) == 4) {
+        // each operand either k-contiguous with 16-byte aligned rows, or contiguous along its other dimension
+        bool a_kc = g.sak == 1 && (g.sam % 4) == 0 && aligned_to(a, 16);
+        bool b_kc = g.sbk == 1 && (g.sbn % 4) == 0 && aligned_to(b, 16);
+        for (int d = 0; d < g.nbatch; d++) {
+            a_kc = a_kc && (g.bsa[d] % 4) == 0;
+            b_kc = b_kc && (g.bsb[d] % 4) == 0;
+        }
+        if (g.K >= kI8BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && use_int_mfma()) {
+            g.tiles_m = (uint32_t)cdiv(g.M, (int64_t)BM);
+            g.tiles_n = (uint32_t)cdiv(g.N, (int64_t)BN);
+            const int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
+            if (blocks > 0x7FFFFFFF) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: too many output tiles");
+            g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
+#define DNH_I8_LAUNCH(TL, AK, BK_) do { \
+                static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_i32_i8parts_kernel<TL, AK, BK_>), \
+                                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kI8LdsBytes); \
+                if (attr != hipSuccess) return fail(DNH_ERR_HIP, "dnh_dot: %s", hipGetErrorString(attr)); \
+                hipLaunchKernelGGL((gemm_i32_i8parts_kernel<TL, AK, BK_>), dim3((unsigned)blocks), dim3(kI8Threads), kI8LdsBytes, stream, \
+                                   (uint32_t*)c, (const uint32_t*)a, (const uint32_t*)b, g); } while (0)
+#define DNH_I8_AB(TL) do { if (a_kc) { if (b_kc) DNH_I8_LAUNCH(TL, true, true); else DNH_I8_LAUNCH(TL, true, false); } \
+                           else { if (b_kc) DNH_I8_LAUNCH(TL, false, true); else DNH_I8_LAUNCH(TL, false, false); } } while (0)
+            if (g.K % kI8BK) DNH_I8_AB(true); else DNH_I8_AB(false);
+#undef DNH_I8_AB
+#undef DNH_I8_LAUNCH
+            DNH_LAUNCH_CHECK();
+            return DNH_OK;
+        }
+    }
+
     g.tiles_m = cdiv(g.M, 64);
     g.tiles_n = cdiv(g.N, 64);
     const int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * batch;

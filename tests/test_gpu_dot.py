@@ -471,3 +471,40 @@ def test_double_precision_stagings(H, G, rng, ta, tb, m, k, n):
     b2 = np.where(np.isfinite(b), b, 0.0)
     got = G.toNumpy(G.ofNumpy(wide)[:, :, 0] @ G.ofNumpy(b2))
     check_dot(wide[:, :, 0] @ b2, got, wide[:, :, 0], b2)
+
+
+@pytest.mark.parametrize("dt", [np.int32, np.uint32])
+@pytest.mark.parametrize("ta,tb", STAGINGS)
+@pytest.mark.parametrize("m,k,n", [(128, 32, 128), (130, 70, 50), (257, 1000, 300), (64, 4099, 33)])
+def test_32_bit_integer_dot_on_the_int8_matrix_instruction(G, rng, dt, ta, tb, m, k, n):
+    """int32 / uint32 products with K >= 32 are formed from signed byte planes on the int8 matrix instruction (ten byte products, one
+    accumulator per shift): bit-identical to wrapping multiply + sum for every value, including the extremes, for both stagings of
+    either operand, partial K steps and edge tiles; NumPy's integer matmul wraps the same way."""
+    info = np.iinfo(dt)
+    a = rng.integers(info.min, info.max, size=(m, k), dtype=dt, endpoint=True)
+    b = rng.integers(info.min, info.max, size=(k, n), dtype=dt, endpoint=True)
+    special = np.array([info.min, info.max, 0, 1, 127, 128, 255, 256, 0x7F7F7F7F, 0x80808080 & info.max, info.max - 127], dtype=np.int64).astype(dt)
+    a[0, :special.size] = special
+    a[1, :] = info.min
+    b[:special.size, 0] = special[::-1]
+    b[:, 1] = info.max
+    if info.min < 0:
+        a[2, :] = -1
+        b[:, 2] = -1
+        b[:, 3] = -128
+    x, y = _views(G, a, b, ta, tb)
+    got = G.toNumpy(x @ y)
+    with np.errstate(over="ignore"):
+        want = np.matmul(a, b)
+    assert got.dtype == np.dtype(dt) and np.array_equal(got, want)
+
+
+def test_32_bit_integer_dot_batched_and_large(G, rng):
+    a = rng.integers(-2 ** 31, 2 ** 31 - 1, size=(3, 2, 200, 96), dtype=np.int32)
+    b = rng.integers(-2 ** 31, 2 ** 31 - 1, size=(1, 2, 96, 150), dtype=np.int32)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b)), np.matmul(a, b))
+    a = rng.integers(0, 2 ** 32 - 1, size=(1024, 2048), dtype=np.uint32)
+    b = rng.integers(0, 2 ** 32 - 1, size=(2048, 1000), dtype=np.uint32)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b)), np.matmul(a, b))
