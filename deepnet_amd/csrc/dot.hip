@@ -1758,6 +1758,192 @@ __global__ __launch_bounds__(kI8Threads) void gemm_i32_i8parts_kernel(uint32_t* 
         }
 }
 
+// 64-bit integers the same way: eight signed byte planes per operand, the 36 byte products with i + j <= 7, one int32 accumulator
+// per shift.  Modulo 2^64 the accumulators of the low shifts must not wrap (shift s needs its sum modulo 2^(64 - 8 s)): 8 (s + 1)
+// byte products of at most 2^14 per K step of 32 stay below 2^31 for 256 steps, so every 256 steps (and at the end) the accumulators are
+// added into the 64-bit result, each shifted by its 8 s, and cleared.  64 x 128 tile, 512 threads = 8 wavefronts 2 x 4, 32 x 32 each.
+constexpr int kI64BM = 64, kI64BN = 128, kI64FoldSteps = 256;
+constexpr size_t kI64LdsBytes = (size_t)2 * 8 * (kI64BM + kI64BN) * kI8Row;
+
+// four elements (consecutive k) -> one dword of each of the eight byte planes
+__device__ __forceinline__ void cut4_i8x8(const uint64_t (&w)[4], uint32_t (&plane)[8]) {
+    uint32_t lo[4], hi[4], q[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const uint64_t d = (w[e] + 0x8080808080808080ull) ^ 0x8080808080808080ull;
+        lo[e] = (uint32_t)d;
+        hi[e] = (uint32_t)(d >> 32);
+    }
+    // (the byte transposition of cut4_i8, without its digit step)
+    auto transpose = [](const uint32_t (&d)[4], uint32_t (&out)[4]) {
+        const uint32_t lo01 = __builtin_amdgcn_perm(d[1], d[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(d[1], d[0], 0x07030602u);
+        const uint32_t lo23 = __builtin_amdgcn_perm(d[3], d[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(d[3], d[2], 0x07030602u);
+        out[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+        out[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+        out[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+        out[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+    };
+    transpose(lo, q);
+#pragma unroll
+    for (int s = 0; s < 4; s++) plane[s] = q[s];
+    transpose(hi, q);
+#pragma unroll
+    for (int s = 0; s < 4; s++) plane[4 + s] = q[s];
+}
+
+// Staging of one operand tile (ROWS rows x 32 k of 64-bit elements) by 512 threads: NG = ROWS / 64 groups of four consecutive k per thread.
+//   KC (k contiguous, 16-byte aligned rows): eight lanes cover the 32 k of a row, 32 bytes each; group i is row r + 64 i.
+//   otherwise (rows contiguous): a thread takes one row and 4 NG consecutive k with element loads.
+template <bool KC, int ROWS>
+struct I64Stage {
+    static constexpr int NG = ROWS / 64;
+    int row, kofs;
+    const uint64_t* p[NG];   // KC: the rows of the groups (a row beyond the matrix reads row 0: its products are never stored)
+    int64_t ks;
+    __device__ __forceinline__ void init(const uint64_t* base, int64_t row0, int64_t limit, int64_t rs, int64_t kstride, int tid) {
+        row = KC ? tid >> 3 : tid & (ROWS - 1);
+        kofs = KC ? (tid & 7) * 4 : (tid / ROWS) * 4 * NG;
+#pragma unroll
+        for (int i = 0; i < NG; i++) {
+            const int64_t rr = row0 + row + (KC ? 64 * i : 0);
+            p[i] = base + (rr < limit ? rr * rs : 0);
+        }
+        ks = KC ? 1 : kstride;
+    }
+    template <bool TAIL>
+    __device__ __forceinline__ void load(int64_t k0, int64_t K, uint64_t (&r)[4 * NG]) const {
+#pragma unroll
+        for (int i = 0; i < NG; i++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int64_t k = k0 + kofs + (KC ? e : 4 * i + e);
+                if (!TAIL || k0 + kI8BK <= K) {
+                    r[4 * i + e] = p[i][k * ks];   // (KC: the four loads of a group are 32 contiguous bytes: two 16-byte loads)
+                } else {
+                    const uint64_t v = p[i][(k < K ? k : K - 1) * ks];
+                    r[4 * i + e] = k < K ? v : 0ull;
+                }
+            }
+    }
+    __device__ __forceinline__ void store(const uint64_t (&r)[4 * NG], unsigned char (*tile)[ROWS][kI8Row]) const {
+        uint32_t q[NG][8];
+#pragma unroll
+        for (int i = 0; i < NG; i++) {
+            const uint64_t w[4] = {r[4 * i], r[4 * i + 1], r[4 * i + 2], r[4 * i + 3]};
+            cut4_i8x8(w, q[i]);
+        }
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int i = 0; i < NG; i++) {
+                if constexpr (KC) *reinterpret_cast<uint32_t*>(&tile[s][row + 64 * i][kofs]) = q[i][s];
+                else *reinterpret_cast<uint32_t*>(&tile[s][row][kofs + 4 * i]) = q[i][s];
+            }
+    }
+};
+
+template <bool TAIL, bool A_KC, bool B_KC>
+__global__ __launch_bounds__(kI8Threads) void gemm_i64_i8parts_kernel(uint64_t* c, const uint64_t* a, const uint64_t* b, GemmArgs g) {
+    extern __shared__ __align__(16) unsigned char i8_lds[];
+    typedef unsigned char (*TilesA)[8][kI64BM][kI8Row];            // [buffer][plane][row][k]
+    typedef unsigned char (*TilesB)[8][kI64BN][kI8Row];
+    TilesA As = reinterpret_cast<TilesA>(i8_lds);
+    TilesB Bs = reinterpret_cast<TilesB>(i8_lds + (size_t)2 * 8 * kI64BM * kI8Row);
+
+    uint32_t bid = blockIdx.x;
+    if (g.xcd_chunk) bid = (bid % 8u) * g.xcd_chunk + bid / 8u;
+    const uint32_t tn = bid % g.tiles_n;
+    bid /= g.tiles_n;
+    const uint32_t tm = bid % g.tiles_m;
+    bid /= g.tiles_m;
+    int64_t oa = 0, ob = 0, oc = 0;
+    for (int d = g.nbatch - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bid / g.bshape[d];
+        const uint32_t i = bid - q * g.bshape[d];
+        bid = q;
+        oa += (int64_t)i * g.bsa[d];
+        ob += (int64_t)i * g.bsb[d];
+        oc += (int64_t)i * g.bsc[d];
+    }
+    const int64_t K = g.K;
+    const int64_t m0 = (int64_t)tm * kI64BM, n0 = (int64_t)tn * kI64BN;
+    a += oa;
+    b += ob;
+    c += oc;
+    const int tid = threadIdx.x;
+
+    I64Stage<A_KC, kI64BM> sa;
+    I64Stage<B_KC, kI64BN> sb;
+    sa.init(a, m0, g.M, g.sam, g.sak, tid);
+    sb.init(b, n0, g.N, g.sbn, g.sbk, tid);
+    uint64_t ra[4], rb[8];
+
+    const int wave = tid >> 6, lane = tid & 63;
+    const int wm = (wave >> 2) * 32, wn = (wave & 3) * 32;
+    const int lm = lane & 31, lk = lane >> 5;
+    i32x16v acc[8];
+    uint64_t tot[16];
+#pragma unroll
+    for (int r = 0; r < 16; r++) tot[r] = 0;
+    auto clear = [&]() {
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[s][r] = 0;
+    };
+    auto fold = [&]() {
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) tot[r] += (uint64_t)(int64_t)acc[s][r] << (8 * s);
+    };
+    clear();
+
+    int cur = 0;
+    auto compute = [&]() {
+        i32x4v bv[8];
+#pragma unroll
+        for (int s = 0; s < 8; s++) bv[s] = *reinterpret_cast<const i32x4v*>(&Bs[cur][s][wn + lm][lk * 16]);
+#pragma unroll
+        for (int pa = 0; pa < 8; pa++) {
+            const i32x4v av = *reinterpret_cast<const i32x4v*>(&As[cur][pa][wm + lm][lk * 16]);
+#pragma unroll
+            for (int pb = 0; pa + pb < 8; pb++) acc[pa + pb] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av, bv[pb], acc[pa + pb], 0, 0, 0);
+        }
+    };
+
+    const int64_t nsteps = (K + kI8BK - 1) / kI8BK;
+    sa.template load<TAIL>(0, K, ra);
+    sb.template load<TAIL>(0, K, rb);
+    sa.store(ra, As[0]);
+    sb.store(rb, Bs[0]);
+    __syncthreads();
+    for (int64_t s = 0; s + 1 < nsteps; s++) {
+        sa.template load<TAIL>((s + 1) * kI8BK, K, ra);
+        sb.template load<TAIL>((s + 1) * kI8BK, K, rb);
+        __builtin_amdgcn_sched_barrier(0);   // the fetches stay in front of the matrix instructions
+        compute();
+        if ((s + 1) % kI64FoldSteps == 0) {
+            fold();
+            clear();
+        }
+        sa.store(ra, As[cur ^ 1]);
+        sb.store(rb, Bs[cur ^ 1]);
+        __syncthreads();
+        cur ^= 1;
+    }
+    compute();
+    fold();
+
+    const bool full_mn = m0 + kI64BM <= g.M && n0 + kI64BN <= g.N;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int64_t m = m0 + wm + (r >> 2) * 8 + lk * 4 + (r & 3);
+        const int64_t n = n0 + wn + lm;
+        if (full_mn || (m < g.M && n < g.N)) c[m * g.scm + n * g.scn] = tot[r];
+    }
+}
+
 bool use_int_mfma() {
     static const bool on = [] { const char* e = getenv("DNH_DOT_INT_MFMA"); return !e || e[0] != '0'; }();   // 0: every integer product on gemm_int_kernel
     return on;
@@ -1790,6 +1976,34 @@ int32_t launch_gemm_int(GemmArgs g, T* c, const T* a, const T* b, int64_t batch,
             if (g.K % kI8BK) DNH_I8_AB(true); else DNH_I8_AB(false);
 #undef DNH_I8_AB
 #undef DNH_I8_LAUNCH
+            DNH_LAUNCH_CHECK();
+            return DNH_OK;
+        }
+    }
+    if constexpr (sizeof(T) == 8) {
+        bool a_kc = g.sak == 1 && (g.sam % 2) == 0 && aligned_to(a, 16);
+        bool b_kc = g.sbk == 1 && (g.sbn % 2) == 0 && aligned_to(b, 16);
+        for (int d = 0; d < g.nbatch; d++) {
+            a_kc = a_kc && (g.bsa[d] % 2) == 0;
+            b_kc = b_kc && (g.bsb[d] % 2) == 0;
+        }
+        if (g.K >= kI8BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && use_int_mfma()) {
+            g.tiles_m = (uint32_t)cdiv(g.M, (int64_t)kI64BM);
+            g.tiles_n = (uint32_t)cdiv(g.N, (int64_t)kI64BN);
+            const int64_t blocks = (int64_t)g.tiles_m * g.tiles_n * batch;
+            if (blocks > 0x7FFFFFFF) return fail(DNH_ERR_NOT_SUPPORTED, "dnh_dot: too many output tiles");
+            g.xcd_chunk = (blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
+#define DNH_I64_LAUNCH(TL, AK, BK_) do { \
+                static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&gemm_i64_i8parts_kernel<TL, AK, BK_>), \
+                                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)kI64LdsBytes); \
+                if (attr != hipSuccess) return fail(DNH_ERR_HIP, "dnh_dot: %s", hipGetErrorString(attr)); \
+                hipLaunchKernelGGL((gemm_i64_i8parts_kernel<TL, AK, BK_>), dim3((unsigned)blocks), dim3(kI8Threads), kI64LdsBytes, stream, \
+                                   (uint64_t*)c, (const uint64_t*)a, (const uint64_t*)b, g); } while (0)
+#define DNH_I64_AB(TL) do { if (a_kc) { if (b_kc) DNH_I64_LAUNCH(TL, true, true); else DNH_I64_LAUNCH(TL, true, false); } \
+                            else { if (b_kc) DNH_I64_LAUNCH(TL, false, true); else DNH_I64_LAUNCH(TL, false, false); } } while (0)
+            if (g.K % kI8BK) DNH_I64_AB(true); else DNH_I64_AB(false);
+#undef DNH_I64_AB
+#undef DNH_I64_LAUNCH
             DNH_LAUNCH_CHECK();
             return DNH_OK;
         }

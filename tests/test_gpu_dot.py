@@ -473,17 +473,19 @@ def test_double_precision_stagings(H, G, rng, ta, tb, m, k, n):
     check_dot(wide[:, :, 0] @ b2, got, wide[:, :, 0], b2)
 
 
-@pytest.mark.parametrize("dt", [np.int32, np.uint32])
+@pytest.mark.parametrize("dt", [np.int32, np.uint32, np.int64, np.uint64])
 @pytest.mark.parametrize("ta,tb", STAGINGS)
 @pytest.mark.parametrize("m,k,n", [(128, 32, 128), (130, 70, 50), (257, 1000, 300), (64, 4099, 33)])
-def test_32_bit_integer_dot_on_the_int8_matrix_instruction(G, rng, dt, ta, tb, m, k, n):
-    """int32 / uint32 products with K >= 32 are formed from signed byte planes on the int8 matrix instruction (ten byte products, one
-    accumulator per shift): bit-identical to wrapping multiply + sum for every value, including the extremes, for both stagings of
-    either operand, partial K steps and edge tiles; NumPy's integer matmul wraps the same way."""
+def test_wide_integer_dot_on_the_int8_matrix_instruction(G, rng, dt, ta, tb, m, k, n):
+    """32- and 64-bit integer products with K >= 32 are formed from signed byte planes on the int8 matrix instruction (the byte
+    products that survive the modulus, one accumulator per shift): bit-identical to wrapping multiply + sum for every value,
+    including the extremes, for both stagings of either operand, partial K steps and edge tiles; NumPy's integer matmul wraps
+    the same way."""
     info = np.iinfo(dt)
     a = rng.integers(info.min, info.max, size=(m, k), dtype=dt, endpoint=True)
     b = rng.integers(info.min, info.max, size=(k, n), dtype=dt, endpoint=True)
-    special = np.array([info.min, info.max, 0, 1, 127, 128, 255, 256, 0x7F7F7F7F, 0x80808080 & info.max, info.max - 127], dtype=np.int64).astype(dt)
+    special = np.array([int(info.min), int(info.max), 0, 1, 127, 128, 255, 256, 0x7F7F7F7F, 0x80808080 & int(info.max), int(info.max) - 127,
+                        0x7F7F7F7F7F7F7F7F & int(info.max), 0x8080808080808080 & int(info.max)], dtype=object).astype(dt)
     a[0, :special.size] = special
     a[1, :] = info.min
     b[:special.size, 0] = special[::-1]
@@ -497,6 +499,23 @@ def test_32_bit_integer_dot_on_the_int8_matrix_instruction(G, rng, dt, ta, tb, m
     with np.errstate(over="ignore"):
         want = np.matmul(a, b)
     assert got.dtype == np.dtype(dt) and np.array_equal(got, want)
+
+
+def test_64_bit_integer_dot_long_inner_dimension(G, rng):
+    """More than 256 K steps: the int32 accumulators of the byte products are added into the 64-bit result before they can wrap.
+    All-extreme operands make every byte product as large as it gets."""
+    k = 20000
+    for fill_a, fill_b in ((-2 ** 63, -2 ** 63), (2 ** 63 - 1, -2 ** 63), (-1, 2 ** 63 - 1), (0x7F7F7F7F7F7F7F7F, 0x7F7F7F7F7F7F7F7F)):
+        a = np.full((40, k), fill_a, dtype=np.int64)
+        b = np.full((k, 70), fill_b, dtype=np.int64)
+        a[:, ::7] = rng.integers(-2 ** 63, 2 ** 63 - 1, size=a[:, ::7].shape, dtype=np.int64)
+        with np.errstate(over="ignore"):
+            want = np.matmul(a, b)
+        assert np.array_equal(G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b)), want)
+    u = rng.integers(0, 2 ** 64 - 1, size=(33, 9000), dtype=np.uint64)
+    v = rng.integers(0, 2 ** 64 - 1, size=(9000, 65), dtype=np.uint64)
+    with np.errstate(over="ignore"):
+        assert np.array_equal(G.toNumpy(G.ofNumpy(u) @ G.ofNumpy(v)), np.matmul(u, v))
 
 
 def test_32_bit_integer_dot_batched_and_large(G, rng):
