@@ -527,3 +527,47 @@ def test_32_bit_integer_dot_batched_and_large(G, rng):
     b = rng.integers(0, 2 ** 32 - 1, size=(2048, 1000), dtype=np.uint32)
     with np.errstate(over="ignore"):
         assert np.array_equal(G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b)), np.matmul(a, b))
+
+
+import os as _os
+
+_DOT_FUZZ = int(_os.environ.get("DNH_FUZZ_SEEDS_FACTOR", "1"))
+
+
+@pytest.mark.parametrize("seed", range(24 * _DOT_FUZZ))
+def test_dot_random_shapes_types_and_views(G, seed):
+    """Random extents (tile edges, K tails, chunk counts and tile forms as the library chooses them), element types, transposed
+    views and broadcast batch dimensions against NumPy: integers bit for bit (wrapping), floats within 16 u S of the fp64 product."""
+    rng = np.random.default_rng(7000 + seed)
+    for case in range(6):
+        dt = [np.float32, np.float64, np.int32, np.int64, np.uint32, np.float32][int(rng.integers(0, 6))]
+        big = rng.random() < 0.25
+        m = int(rng.integers(1, 1500 if big else 300))
+        n = int(rng.integers(1, 1500 if big else 300))
+        k = int(rng.integers(1, 400 if big else 2500))
+        batch = () if big or rng.random() < 0.5 else tuple(int(x) for x in rng.integers(1, 4, size=int(rng.integers(1, 3))))
+        ta, tb = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        bcast = len(batch) > 0 and rng.random() < 0.3
+        sa = batch + (m, k)
+        sb = ((1,) * len(batch) if bcast else batch) + (k, n)
+        if np.dtype(dt).kind == "f":
+            a = rng.standard_normal(sa).astype(dt)
+            b = rng.standard_normal(sb).astype(dt)
+        else:
+            info = np.iinfo(dt)
+            a = rng.integers(info.min, info.max, size=sa, dtype=dt, endpoint=True)
+            b = rng.integers(info.min, info.max, size=sb, dtype=dt, endpoint=True)
+        x, y = _views(G, a, b, ta, tb)
+        got = G.toNumpy(x @ y)
+        what = (seed, case, np.dtype(dt).name, sa, sb, ta, tb)
+        if np.dtype(dt).kind == "f":
+            u = np.finfo(dt).eps / 2
+            exact = np.matmul(a.astype(np.float64), b.astype(np.float64))
+            S = np.matmul(np.abs(a).astype(np.float64), np.abs(b).astype(np.float64))
+            # fp64 results are compared with an fp64 product: leave room for its own rounding
+            bound = (16 if dt == np.float32 else 2 * k + 64) * u * S + np.finfo(dt).tiny
+            assert got.shape == exact.shape and np.all(np.abs(got - exact) <= bound), what
+        else:
+            with np.errstate(over="ignore"):
+                want = np.matmul(a, b)
+            assert got.dtype == np.dtype(dt) and np.array_equal(got, want), what
