@@ -548,12 +548,15 @@ __global__ __launch_bounds__(kBlock) void compact_move_kernel(MaskArgs m, W* ful
 constexpr int kFastJ = 4;
 
 template <int VEC>
-__device__ __forceinline__ uint32_t mask_flags(const uint8_t* m) {
-    const Pack<uint8_t, VEC> v = load_pack<uint8_t, VEC>(m);
+__device__ __forceinline__ uint32_t flags_of(const Pack<uint8_t, VEC>& v) {
     uint32_t f = 0;
 #pragma unroll
     for (int e = 0; e < VEC; e++) f |= (uint32_t)(v.v[e] != 0) << e;
     return f;
+}
+template <int VEC>
+__device__ __forceinline__ uint32_t mask_flags(const uint8_t* m) {
+    return flags_of<VEC>(load_pack<uint8_t, VEC>(m));
 }
 
 __device__ __forceinline__ uint64_t block_exclusive_scan64(uint64_t c, uint64_t* total) {
@@ -611,7 +614,23 @@ __global__ __launch_bounds__(kBlock) void compact_count_fast_kernel(const uint8_
 __device__ __forceinline__ uint32_t block_sum_before(const uint32_t* counts, uint32_t n) {
     __shared__ uint32_t part[kBlock / 64];
     uint32_t s = 0;
-    for (uint32_t i = threadIdx.x; i < n; i += kBlock) s += counts[i];
+    // eight loads in flight per thread (one after the other they cost a trip to L2 each: up to 32 in a row for 8192 blocks)
+    constexpr uint32_t U = 8;
+    uint32_t i = threadIdx.x;
+    for (; i + (U - 1) * kBlock < n; i += U * kBlock) {
+        uint32_t v[U];
+#pragma unroll
+        for (uint32_t u = 0; u < U; u++) v[u] = counts[i + u * kBlock];
+#pragma unroll
+        for (uint32_t u = 0; u < U; u++) s += v[u];
+    }
+    {
+        uint32_t v[U];   // the rest: clamped loads, masked sums (no branch between the loads)
+#pragma unroll
+        for (uint32_t u = 0; u < U; u++) v[u] = counts[i + u * kBlock < n ? i + u * kBlock : 0];
+#pragma unroll
+        for (uint32_t u = 0; u < U; u++) s += i + u * kBlock < n ? v[u] : 0u;
+    }
 #pragma unroll
     for (int m = 32; m >= 1; m >>= 1) s += (uint32_t)__shfl_xor((int)s, m, 64);
     if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = s;
@@ -629,19 +648,30 @@ __global__ __launch_bounds__(kBlock) void compact_move_fast_kernel(const uint8_t
     uint32_t flags[kFastJ];
     Pack<W, VEC> data[kFastJ];
     uint64_t packed = 0;
+    uint32_t seg_base;
+    {
+        // every load of the thread is issued before the first one is used, without a branch in between (a vector beyond the end reads
+        // vector 0 and counts nothing): with `if (v < nvec) { load; use }` per segment each segment waited for its own mask bytes
+        // before the next segment's loads went out
+        Pack<uint8_t, VEC> mk[kFastJ];
 #pragma unroll
-    for (int j = 0; j < kFastJ; j++) {
-        const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
-        flags[j] = 0;
-        if (v < nvec) {
-            flags[j] = mask_flags<VEC>(mask + (size_t)v * VEC);
-            if constexpr (!SET || sizeof(W) >= 4) data[j] = load_pack<W, VEC>(full + (size_t)v * VEC);
+        for (int j = 0; j < kFastJ; j++) {
+            const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+            const size_t vc = v < nvec ? (size_t)v : 0;
+            mk[j] = load_pack<uint8_t, VEC>(mask + vc * VEC);
+            if constexpr (!SET || sizeof(W) >= 4) data[j] = load_pack<W, VEC>(full + vc * VEC);
         }
-        packed |= (uint64_t)__popc(flags[j]) << (16 * j);
+        // (the counts of the blocks before this one are fetched while the loads above are on their way)
+        seg_base = PREFIXED ? block_base[blockIdx.x] : block_sum_before(block_base, blockIdx.x);
+#pragma unroll
+        for (int j = 0; j < kFastJ; j++) {
+            const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+            flags[j] = v < nvec ? flags_of<VEC>(mk[j]) : 0u;
+            packed |= (uint64_t)__popc(flags[j]) << (16 * j);
+        }
     }
     uint64_t total;
     const uint64_t pre = block_exclusive_scan64(packed, &total);
-    uint32_t seg_base = PREFIXED ? block_base[blockIdx.x] : block_sum_before(block_base, blockIdx.x);
     if constexpr (!SET && sizeof(W) >= 4) {
         // masked get: the block's selected elements are gathered in LDS at their rank inside the block and leave as one
         // contiguous run, so every store instruction of a wavefront writes 64 consecutive elements
@@ -668,8 +698,23 @@ __global__ __launch_bounds__(kBlock) void compact_move_fast_kernel(const uint8_t
         uint32_t btotal = 0;
 #pragma unroll
         for (int j = 0; j < kFastJ; j++) btotal += (uint32_t)((total >> (16 * j)) & 0xFFFF);
-        for (uint32_t i = threadIdx.x; i < btotal; i += kBlock)
-            if (seg_base + i < nout) stage[i] = out[seg_base + i];
+        {
+            // the block's run of values: at most kFastJ * VEC fetches per thread, all issued before the first is written to LDS
+            // (positions beyond the run fetch its first value again and write nothing)
+            constexpr int NI = kFastJ * VEC;
+            const uint32_t limit = btotal < nout - (seg_base < nout ? seg_base : nout) ? btotal : nout - (seg_base < nout ? seg_base : nout);
+            W val[NI];
+#pragma unroll
+            for (int q = 0; q < NI; q++) {
+                const uint32_t i = threadIdx.x + q * kBlock;
+                val[q] = out[(seg_base < nout ? seg_base : 0) + (i < limit ? i : 0)];
+            }
+#pragma unroll
+            for (int q = 0; q < NI; q++) {
+                const uint32_t i = threadIdx.x + q * kBlock;
+                if (i < limit) stage[i] = val[q];
+            }
+        }
         __syncthreads();
         uint32_t lbase = 0;
 #pragma unroll
@@ -719,15 +764,24 @@ __global__ __launch_bounds__(kBlock) void true_indices_fast_kernel(const uint8_t
     __shared__ uint16_t stage[kFastJ * kBlock * VEC];
     uint32_t flags[kFastJ];
     uint64_t packed = 0;
+    uint32_t seg_base;
+    {
+        Pack<uint8_t, VEC> mk[kFastJ];   // all loads first, as in compact_move_fast_kernel
 #pragma unroll
-    for (int j = 0; j < kFastJ; j++) {
-        const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
-        flags[j] = v < nvec ? mask_flags<VEC>(mask + (size_t)v * VEC) : 0u;
-        packed |= (uint64_t)__popc(flags[j]) << (16 * j);
+        for (int j = 0; j < kFastJ; j++) {
+            const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+            mk[j] = load_pack<uint8_t, VEC>(mask + (v < nvec ? (size_t)v : 0) * VEC);
+        }
+        seg_base = PREFIXED ? block_base[blockIdx.x] : block_sum_before(block_base, blockIdx.x);
+#pragma unroll
+        for (int j = 0; j < kFastJ; j++) {
+            const uint32_t v = (blockIdx.x * kFastJ + j) * kBlock + threadIdx.x;
+            flags[j] = v < nvec ? flags_of<VEC>(mk[j]) : 0u;
+            packed |= (uint64_t)__popc(flags[j]) << (16 * j);
+        }
     }
     uint64_t total;
     const uint64_t pre = block_exclusive_scan64(packed, &total);
-    const uint32_t seg_base = PREFIXED ? block_base[blockIdx.x] : block_sum_before(block_base, blockIdx.x);
     uint32_t lbase = 0;
 #pragma unroll
     for (int j = 0; j < kFastJ; j++) {
