@@ -962,12 +962,12 @@ struct F64Stage {
     __device__ __forceinline__ void load(int64_t k0, int64_t K, double (&r)[4]) const {
         if (!TAIL || k0 + kF64BK <= K) {
             if constexpr (KC) {
-                typedef double f64x2v __attribute__((ext_vector_type(2)));   // plain loads, as in X3Stage
-                const f64x2v v0 = *reinterpret_cast<const f64x2v*>(p0 + k0 + kofs), v1 = *reinterpret_cast<const f64x2v*>(p1 + k0 + kofs);
-                r[0] = v0[0];
-                r[1] = v0[1];
-                r[2] = v1[0];
-                r[3] = v1[1];
+                // (non-temporal loads; plain ones measured the same here)
+                const Pack<double, 2> v0 = load_pack<double, 2>(p0 + k0 + kofs), v1 = load_pack<double, 2>(p1 + k0 + kofs);
+                r[0] = v0.v[0];
+                r[1] = v0.v[1];
+                r[2] = v1.v[0];
+                r[3] = v1.v[1];
             } else {
 #pragma unroll
                 for (int e = 0; e < 4; e++) r[e] = p0[(k0 + kofs + e) * ks];
