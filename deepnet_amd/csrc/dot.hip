@@ -1645,6 +1645,18 @@ struct I8Stage {
             }
         }
     }
+    // half of store(): elements 4 H .. 4 H + 3
+    template <int H>
+    __device__ __forceinline__ void piece(const uint32_t (&r)[8], unsigned char (*tile)[BM][kI8Row]) const {
+        const uint32_t w[4] = {r[4 * H], r[4 * H + 1], r[4 * H + 2], r[4 * H + 3]};
+        uint32_t q[4];
+        cut4_i8(w, q);
+#pragma unroll
+        for (int s = 0; s < 4; s++) {
+            if constexpr (KC) *reinterpret_cast<uint32_t*>(&tile[s][row + 64 * H][kofs]) = q[s];
+            else *reinterpret_cast<uint32_t*>(&tile[s][row][kofs + 4 * H]) = q[s];
+        }
+    }
     __device__ __forceinline__ void store(const uint32_t (&r)[8], unsigned char (*tile)[BM][kI8Row]) const {
         uint32_t w0[4] = {r[0], r[1], r[2], r[3]}, w1[4] = {r[4], r[5], r[6], r[7]}, q0[4], q1[4];
         cut4_i8(w0, q0);
@@ -1710,22 +1722,38 @@ __global__ __launch_bounds__(kI8Threads) void gemm_i32_i8parts_kernel(uint32_t* 
 #pragma unroll
             for (int r = 0; r < 16; r++) acc[i][s][r] = 0;
 
+    // One K step, the instruction order pinned as in the bf16-parts kernels: the fetch of the next step (NEXT), the LDS reads of B and of
+    // the first 32 rows of A, then the 20 matrix instructions with the remaining LDS reads behind the first four and the four pieces of
+    // the cutting (one cut4_i8 each with its LDS writes) behind numbers 8, 11, 14 and 17.
     int cur = 0;
-    auto compute = [&]() {
+    auto k_step = [&](auto next_tag, auto tail_tag, int64_t k_next) {
+        constexpr bool NEXT = decltype(next_tag)::value, TL = decltype(tail_tag)::value;
+        if constexpr (NEXT) {
+            sa.template load<TL>(k_next, K, ra);
+            sb.template load<TL>(k_next, K, rb);
+        }
+        __builtin_amdgcn_sched_barrier(0);
         i32x4v av[2][4], bv[4];
 #pragma unroll
         for (int s = 0; s < 4; s++) bv[s] = *reinterpret_cast<const i32x4v*>(&Bs[cur][s][wn + lm][lk * 16]);
 #pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int s = 0; s < 4; s++) av[i][s] = *reinterpret_cast<const i32x4v*>(&As[cur][s][wm + i * 32 + lm][lk * 16]);
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int sh = 0; sh < 4; sh++)
-#pragma unroll
-                for (int pa = 0; pa <= sh; pa++)
-                    acc[i][sh] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i][pa], bv[sh - pa], acc[i][sh], 0, 0, 0);
+        for (int s = 0; s < 4; s++) av[0][s] = *reinterpret_cast<const i32x4v*>(&As[cur][s][wm + lm][lk * 16]);
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<20>([&](auto tt) {
+            // products in the order (sub-tile i, shift sh, plane pa of A): 1 + 2 + 3 + 4 per sub-tile
+            constexpr int t = decltype(tt)::value, i = t / 10, u = t % 10;
+            constexpr int sh = u < 1 ? 0 : u < 3 ? 1 : u < 6 ? 2 : 3;
+            constexpr int pa = u - (sh == 0 ? 0 : sh == 1 ? 1 : sh == 2 ? 3 : 6);
+            acc[i][sh] = __builtin_amdgcn_mfma_i32_32x32x32_i8(av[i][pa], bv[sh - pa], acc[i][sh], 0, 0, 0);
+            if constexpr (t < 4) av[1][t] = *reinterpret_cast<const i32x4v*>(&As[cur][t][wm + 32 + lm][lk * 16]);
+            if constexpr (NEXT && (t == 8 || t == 11)) sa.template piece<(t - 8) / 3>(ra, As[cur ^ 1]);
+            if constexpr (NEXT && (t == 14 || t == 17)) sb.template piece<(t - 14) / 3>(rb, Bs[cur ^ 1]);
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        if constexpr (NEXT) {
+            __syncthreads();
+            cur ^= 1;
+        }
     };
 
     const int64_t nsteps = (K + kI8BK - 1) / kI8BK;
@@ -1734,17 +1762,9 @@ __global__ __launch_bounds__(kI8Threads) void gemm_i32_i8parts_kernel(uint32_t* 
     sa.store(ra, As[0]);
     sb.store(rb, Bs[0]);
     __syncthreads();
-    for (int64_t s = 0; s + 1 < nsteps; s++) {
-        sa.template load<TAIL>((s + 1) * kI8BK, K, ra);
-        sb.template load<TAIL>((s + 1) * kI8BK, K, rb);
-        __builtin_amdgcn_sched_barrier(0);   // the fetches stay in front of the matrix instructions
-        compute();
-        sa.store(ra, As[cur ^ 1]);
-        sb.store(rb, Bs[cur ^ 1]);
-        __syncthreads();
-        cur ^= 1;
-    }
-    compute();
+    for (int64_t s = 0; s + 2 < nsteps; s++) k_step(std::true_type(), std::false_type(), (s + 1) * kI8BK);
+    if (nsteps >= 2) k_step(std::true_type(), std::integral_constant<bool, TAIL>(), (nsteps - 1) * kI8BK);
+    k_step(std::false_type(), std::false_type(), 0);
 
     const bool full_mn = m0 + BM <= g.M && n0 + BN <= g.N;
 #pragma unroll
