@@ -2,7 +2,8 @@
 // ITensorBackend SumLastAxis..CountTrueLastAxis, ArgMin/ArgMaxLastAxis, FindLastAxis (Tensor/Tensor/TensorBackend.fs:125-135).
 // Fold semantics follow Tensor/Tensor/Host/ScalarOps.fs:606-665: sum from zero, product from one, max from minValue<T>
 // with `if res > v then res else v`, min from maxValue<T>, all from true, any from false, countTrue into int64; an empty
-// axis yields the initial value.  Float sums and products are re-associated (tree order); everything else is order-independent.
+// axis yields the initial value.  Float sums and products are re-associated (tree order); Max / Min of floats follow the sequential
+// rule for NaNs as well (RMax); everything else is order-independent.
 #include "reduce_kernels.h"
 #include "ops.h"
 
@@ -26,19 +27,44 @@ template <class X> struct RProd {
     __device__ X combine(X a, X b) const { return OpMul<X>{}(a, b); }
     __device__ X extract(X s) const { return s; }
 };
+// Max / Min follow the reference's sequential rule `if res > v then res else v` from minValue (Host/ScalarOps.fs:620-628).  Without
+// NaNs any order gives the same value.  With a NaN the rule depends on the order: the NaN replaces the running value, and the next
+// element replaces the NaN, so the result is the fold of what follows the last NaN (NaN if it comes last).  The tree therefore carries
+// a NaN through every step and combination (a result that met one is a NaN), and the thread that stores a NaN result recomputes it in
+// order (kSeqFix, finish_value): faithful for every input, at one extra comparison per element for NaN-free data.
 template <class X> struct RMax {
     using In = X; using State = X; using Out = X;
+    static constexpr bool kSeqFix = std::is_floating_point<X>::value;
     __device__ X init() const { return std::numeric_limits<X>::lowest(); }
-    __device__ X step(X s, X v, int64_t) const { return s > v ? s : v; }
-    __device__ X combine(X a, X b) const { return a > b ? a : b; }
+    __device__ X step(X s, X v, int64_t) const { return (s > v || s != s) ? s : v; }
+    __device__ X combine(X a, X b) const { return (a > b || a != a) ? a : b; }
     __device__ X extract(X s) const { return s; }
+    __device__ bool needs_fix(X s) const { return s != s; }
+    __device__ X sequential(const X* p, int64_t n, int64_t stride) const {
+        X s = std::numeric_limits<X>::lowest();
+        for (int64_t i = 0; i < n; i++) {
+            const X v = p[i * stride];
+            s = s > v ? s : v;
+        }
+        return s;
+    }
 };
 template <class X> struct RMin {
     using In = X; using State = X; using Out = X;
+    static constexpr bool kSeqFix = std::is_floating_point<X>::value;
     __device__ X init() const { return std::numeric_limits<X>::max(); }
-    __device__ X step(X s, X v, int64_t) const { return s < v ? s : v; }
-    __device__ X combine(X a, X b) const { return a < b ? a : b; }
+    __device__ X step(X s, X v, int64_t) const { return (s < v || s != s) ? s : v; }
+    __device__ X combine(X a, X b) const { return (a < b || a != a) ? a : b; }
     __device__ X extract(X s) const { return s; }
+    __device__ bool needs_fix(X s) const { return s != s; }
+    __device__ X sequential(const X* p, int64_t n, int64_t stride) const {
+        X s = std::numeric_limits<X>::max();
+        for (int64_t i = 0; i < n; i++) {
+            const X v = p[i * stride];
+            s = s < v ? s : v;
+        }
+        return s;
+    }
 };
 struct RAll {
     using In = uint8_t; using State = uint8_t; using Out = uint8_t;

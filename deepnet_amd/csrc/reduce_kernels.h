@@ -56,9 +56,24 @@ __device__ __forceinline__ typename R::State group_reduce(const R& r, typename R
     return s;
 }
 
+// A fold may name results that the tree cannot produce faithfully (kSeqFix: Max / Min of floats that met a NaN, whose value under
+// the reference's sequential rule depends on where the NaN stood): the thread that stores such a result recomputes it by walking the
+// reduced axis in order (elements p[0], p[stride], ... p[(n - 1) stride]).  Rare by construction; every other result is extract(state).
+template <class R, class = void> struct NeedsSeqFix : std::false_type {};
+template <class R> struct NeedsSeqFix<R, std::void_t<decltype(R::kSeqFix)>> : std::integral_constant<bool, R::kSeqFix> {};
+template <class R>
+__device__ __forceinline__ typename R::Out finish_value(const R& r, const typename R::State& s, const typename R::In* p, int64_t n, int64_t stride) {
+    if constexpr (NeedsSeqFix<R>::value) {
+        if (r.needs_fix(s)) return r.sequential(p, n, stride);
+    }
+    return r.extract(s);
+}
+
+// fix_src / fix_n / fix_sr (FROM_STATE only): the fold's source, the length and the stride of its reduced axis, for finish_value.
 template <class R, int VEC, int TPR, bool FROM_STATE>
 __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(R r, const void* src_, typename R::Out* out, typename R::State* partial,
-                                                             OuterArgs o, uint32_t rows, int64_t n, int64_t sr, int64_t chunk, uint32_t splits) {
+                                                             OuterArgs o, uint32_t rows, int64_t n, int64_t sr, int64_t chunk, uint32_t splits,
+                                                             const typename R::In* fix_src, int64_t fix_n, int64_t fix_sr) {
     using State = typename R::State;
     using In = typename std::conditional<FROM_STATE, State, typename R::In>::type;
     constexpr int RPB = kBlock / TPR;
@@ -68,8 +83,10 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(R r, const void* sr
     const uint32_t lane = threadIdx.x % TPR;
     const bool active = row < rows;
     int64_t toff = 0, soff = 0;
+    [[maybe_unused]] int64_t soff0 = 0;   // offset of the row in the fold's source
     if (active) {
         outer_offsets(o, row, toff, soff);
+        soff0 = soff;
         if constexpr (FROM_STATE) soff = (int64_t)row * n;
     }
     const int64_t c0 = (int64_t)blockIdx.y * chunk;
@@ -121,8 +138,10 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(R r, const void* sr
         }
     }
     if (active && lane == 0) {
-        if (splits == 1) out[toff] = r.extract(s);
-        else partial[(int64_t)row * splits + blockIdx.y] = s;
+        if (splits == 1) {
+            if constexpr (FROM_STATE) out[toff] = finish_value(r, s, fix_src + soff0, fix_n, fix_sr);
+            else out[toff] = finish_value(r, s, (const typename R::In*)src_ + soff0, n, sr);
+        } else partial[(int64_t)row * splits + blockIdx.y] = s;
     }
 }
 
@@ -189,7 +208,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(R r, const typename
     if (y == 0 && active) {
         if (splits == 1) {
 #pragma unroll
-            for (int e = 0; e < VEC; e++) out[toff + (int64_t)(col0 + e) * tc_stride] = r.extract(st[e]);
+            for (int e = 0; e < VEC; e++) out[toff + (int64_t)(col0 + e) * tc_stride] = finish_value(r, st[e], src + soff + col0 + e, n, sr);
         } else {
             State* q = partial + ((int64_t)other * splits + split) * nc + col0;
             if constexpr (VEC > 1 && sizeof(State) * VEC == 16) {
@@ -209,7 +228,8 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(R r, const typename
 // of State), kBlock / WX groups share the splits and are combined through LDS in a fixed order.
 template <class R, int WX>
 __global__ __launch_bounds__(kBlock) void reduce_cols_finish_kernel(R r, const typename R::State* partial, typename R::Out* out, OuterArgs o,
-                                                                    uint32_t col_tiles, uint32_t nc, int64_t tc_stride, uint32_t splits) {
+                                                                    uint32_t col_tiles, uint32_t nc, int64_t tc_stride, uint32_t splits,
+                                                                    const typename R::In* fix_src, int64_t fix_n, int64_t fix_sr) {
     using State = typename R::State;
     constexpr int NY = kBlock / WX;
     const uint32_t x = threadIdx.x % WX, y = threadIdx.x / WX;
@@ -236,7 +256,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_finish_kernel(R r, const t
         for (int w = 1; w < NY; w++) st = r.combine(st, sh[w][x]);
         int64_t toff, soff;
         outer_offsets(o, other, toff, soff);
-        out[toff + (int64_t)col * tc_stride] = r.extract(st);
+        out[toff + (int64_t)col * tc_stride] = finish_value(r, st, fix_src + soff + col, fix_n, fix_sr);
     }
 }
 
@@ -250,7 +270,7 @@ __global__ __launch_bounds__(kBlock) void reduce_generic_kernel(R r, const typen
     typename R::State s = r.init();
     const typename R::In* p = src + soff;
     for (int64_t i = 0; i < n; i++) s = r.step(s, p[i * sr], i);
-    out[toff] = r.extract(s);
+    out[toff] = finish_value(r, s, p, n, sr);
 }
 
 // ---- host-side strategy --------------------------------------------------------------------------------------------------
@@ -258,10 +278,10 @@ __global__ __launch_bounds__(kBlock) void reduce_generic_kernel(R r, const typen
 // Finishing pass of the two-pass tree: `nout` rows of `splits` State partials each.
 template <class R>
 int32_t launch_finish(const R& r, typename R::State* partial, typename R::Out* out, const OuterArgs& o, uint32_t nout, uint32_t splits,
-                      hipStream_t stream) {
+                      const typename R::In* fix_src, int64_t fix_n, int64_t fix_sr, hipStream_t stream) {
     using State = typename R::State;
 #define DNH_FIN(TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, 1, TPR, true>), dim3(cdiv(nout, kBlock / TPR)), dim3(kBlock), 0, stream, r, \
-                                        (const void*)partial, out, (State*)nullptr, o, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u)
+                                        (const void*)partial, out, (State*)nullptr, o, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u, fix_src, fix_n, fix_sr)
     if (splits > 512) DNH_FIN(256);
     else if (splits > 32) DNH_FIN(64);
     else DNH_FIN(16);
@@ -367,7 +387,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         WorkspaceLease lease;
         if (splits > 1) DNH_TRY(partial_buffer(ps, stream, sizeof(State) * (size_t)nout * splits, (void**)&partial, lease, what));
         const dim3 grid((unsigned)row_blocks, splits);
-#define DNH_ROWS(V, TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, V, TPR, false>), grid, dim3(kBlock), 0, stream, r, (const void*)src, out, partial, o, nout, n, sr, chunk, splits)
+#define DNH_ROWS(V, TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, V, TPR, false>), grid, dim3(kBlock), 0, stream, r, (const void*)src, out, partial, o, nout, n, sr, chunk, splits, src, n, sr)
         if (vec) {
             if (tpr == 256) DNH_ROWS(VEC, 256); else if (tpr == 64) DNH_ROWS(VEC, 64); else DNH_ROWS(VEC, 16);
         } else {
@@ -377,7 +397,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         DNH_LAUNCH_CHECK();
         if (splits > 1) {
             // finishing pass: rows of `splits` State partials
-            DNH_TRY(launch_finish(r, partial, out, o, nout, splits, stream));
+            DNH_TRY(launch_finish(r, partial, out, o, nout, splits, src, n, sr, stream));
         }
         return DNH_OK;
     }
@@ -442,7 +462,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
                 constexpr int FW = 32;   // (16 and 64 columns per finishing workgroup measured 1-2 % slower on 8192 x 8192)
                 const uint32_t ftiles = cdiv(nc, FW);
                 hipLaunchKernelGGL((reduce_cols_finish_kernel<R, FW>), dim3(ftiles * others), dim3(kBlock), 0, stream, r, (const State*)partial, out,
-                                   oo, ftiles, nc, tc_stride, splits);
+                                   oo, ftiles, nc, tc_stride, splits, src, n, sr);
                 DNH_LAUNCH_CHECK();
             }
             return DNH_OK;

@@ -121,11 +121,12 @@ typedef enum DnhCompareOp {
 
 /* Last-axis folds: ITensorBackend SumLastAxis..CountTrueLastAxis (TensorBackend.fs:125-131);
  * Host/ScalarOps.fs:299-361 (ApplyAxisFold), :606-636.
- * NaN in Min / Max (and in the element-wise MaxElemwise / MinElemwise): the reference's fold is the sequential
- * `if res > v then res else v` (ScalarOps.fs:620-628), whose result with NaNs depends on their positions (a NaN replaces the
- * running value and is itself replaced by the next element), and its SIMD path (Host/VectorOps.fs:234-240) behaves differently
- * again.  Here the folds combine in tree order with the same comparison, so a NaN among the folded elements gives an unspecified
- * element of the axis or NaN; results are identical to the reference's on NaN-free data.  ArgMin / ArgMax never select a NaN, as
+ * NaN in Min / Max: the reference's fold is the sequential `if res > v then res else v` from minValue (ScalarOps.fs:620-628), whose
+ * result with NaNs depends on their positions: a NaN replaces the running value and is itself replaced by the next element, so the
+ * result is the fold of what follows the last NaN, or NaN when it comes last.  The folds here give exactly that for every input (a
+ * result that met a NaN is recomputed in the reference's order by the thread that stores it).  The element-wise MaxElemwise /
+ * MinElemwise are the same comparison, `a > b ? a : b` (ScalarOps.fs:525-533; the reference's SIMD path for contiguous single and
+ * double data, Host/VectorOps.fs:234-240, leaves the NaN case to the platform).  ArgMin / ArgMax never select a NaN, as
  * in the reference.  Sum / Product are re-associated: |result - reference| <= (n + 64) u sum|x_i| (u = unit roundoff). */
 typedef enum DnhReduceOp {
     DNH_SUM = 0, DNH_PRODUCT, DNH_MIN, DNH_MAX, DNH_ALL, DNH_ANY, DNH_COUNT_TRUE, DNH_REDUCE_COUNT

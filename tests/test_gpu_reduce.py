@@ -157,3 +157,55 @@ def test_strided_reduce_axis(H, G, rng):
     # a single strided column reduced to a scalar
     ref, got = both(H, G, lambda t: t[:, 7, 9].maxAxis(0), x)
     assert_exact(ref, got)
+
+
+def _seq_fold(x, is_max):
+    """The reference's sequential Max / Min fold (Host/ScalarOps.fs:620-628) over the last axis, element by element."""
+    dt = x.dtype
+    init = np.finfo(dt).min if is_max else np.finfo(dt).max
+    out = np.empty(x.shape[:-1], dt)
+    for idx in np.ndindex(*x.shape[:-1]):
+        r = dt.type(init)
+        for v in x[idx]:
+            r = r if (r > v if is_max else r < v) else v
+        out[idx] = r
+    return out
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("shape", [(37, 300), (3, 70000), (600, 40), (1, 5), (2000, 16), (40, 2, 513)])
+def test_max_min_follow_the_sequential_rule_with_nans(H, G, rng, dt, shape):
+    """With NaNs among the elements the reference's `if res > v then res else v` gives the fold of what follows the last NaN (NaN if
+    it comes last).  Rows without a NaN, with one in front, in the middle, at the end, several, all NaN, NaN followed only by -inf;
+    along the last axis and (through a transposed view) along the first; row, split-row and column forms of the kernels.  Bit for bit
+    against the oracle, and against the rule spelled out in Python on the smaller shapes."""
+    x = rng.standard_normal(shape).astype(dt)
+    flat = x.reshape(-1, shape[-1])
+    n = shape[-1]
+    for i in range(flat.shape[0]):
+        kind = i % 8
+        if kind == 1: flat[i, 0] = np.nan
+        elif kind == 2: flat[i, n // 2] = np.nan
+        elif kind == 3: flat[i, n - 1] = np.nan
+        elif kind == 4: flat[i, rng.integers(0, n, size=min(n, 5))] = np.nan
+        elif kind == 5: flat[i, :] = np.nan
+        elif kind == 6:
+            flat[i, : n // 2 + 1] = np.nan
+            flat[i, n // 2 + 1:] = -np.inf if i % 16 == 6 else np.inf
+        elif kind == 7: flat[i, rng.integers(0, n)] = np.nan
+    for name in ("maxAxis", "minAxis"):
+        for axis_last in (True, False):
+            def f(t):
+                v = t if axis_last else t.permuteAxes(list(range(1, len(shape))) + [0])   # the reduced axis first, as a view
+                return getattr(v, name)(len(shape) - 1 if axis_last else 0)
+            ref, got = both(H, G, f, x)
+            assert ref.dtype == got.dtype == np.dtype(dt)
+            assert np.array_equal(ref, got, equal_nan=True), (name, axis_last)
+            if x.size <= 40000 and axis_last:
+                want = _seq_fold(x, name == "maxAxis")
+                assert np.array_equal(want, got, equal_nan=True), name
+    # the whole tensor as one row (the split-row form for the long shapes)
+    ref, got = both(H, G, lambda t: t.max(), x)
+    assert np.array_equal(ref, got, equal_nan=True)
+    ref, got = both(H, G, lambda t: t.min(), x)
+    assert np.array_equal(ref, got, equal_nan=True)

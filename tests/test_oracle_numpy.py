@@ -241,3 +241,19 @@ def test_convert_of_floats_outside_the_integer_range(H):
     r = np.random.default_rng(2).uniform(-100, 100, 1000)
     for dst in (np.int32, np.int64, np.int8, np.int16):
         assert np.array_equal(H.toNumpy(H.ofNumpy(r).convert(dst)), np.trunc(r).astype(dst))
+
+
+def test_max_min_folds_with_nans_follow_the_sequential_rule(H):
+    """`if res > v then res else v` from minValue (Host/ScalarOps.fs:620-628), spelled out element by element: a NaN replaces the
+    running value and is replaced by the next element, so the result is the fold of what follows the last NaN."""
+    nan, inf = np.nan, np.inf
+    x = np.array([[1, 5, 2, 4], [nan, 5, 2, 4], [1, nan, 2, 4], [1, 5, 2, nan], [nan, nan, nan, nan], [9, nan, -inf, -inf],
+                  [nan, 3, nan, 3], [-inf, -inf, -inf, -inf]], dtype=np.float32)
+    fmin, fmax = np.finfo(np.float32).min, np.finfo(np.float32).max
+    want_max = np.array([5, 5, 4, nan, nan, -inf, 3, fmin], dtype=np.float32)
+    want_min = np.array([1, 2, 2, nan, nan, -inf, 3, -inf], dtype=np.float32)
+    got_max = run_on(H, lambda t: t.maxAxis(1), [x])
+    got_min = run_on(H, lambda t: t.minAxis(1), [x])
+    assert np.array_equal(got_max, want_max, equal_nan=True), got_max
+    assert np.array_equal(got_min, want_min, equal_nan=True), got_min
+    assert fmax > 0 and run_on(H, lambda t: t.minAxis(1), [np.array([[inf, inf]], np.float64)]).tolist() == [np.finfo(np.float64).max]
