@@ -459,6 +459,134 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
     }
 }
 
+// The transposing kernel for 4-byte staged elements and whole tiles, with both LDS phases free of bank conflicts and on 16-byte
+// LDS instructions.  map_tr_kernel's [b][a + 1] tile is written with one 4-byte store per element at a lane stride of four words
+// (8 of the 32 banks) and read element by element (16 banks).  Here a staging thread fetches the same vector of four a's from
+// four consecutive rows b, so that it holds a 4 x 4 block, and writes its four columns: LDS is [a][b] in 16-byte groups of four
+// b's, group g of row a stored at g ^ ((a / 4) % 8); consecutive lanes (a four apart) then fall into different groups, and a storing
+// thread fetches its four b's of row a with one 16-byte read, consecutive lanes again in different groups.
+// One staged source (MASK 1 or 2); for two-operand ops the other source is read in the store pattern, MODE 1 (broadcast along B:
+// one value per stored row, fetched ahead of the barrier) or MODE 2 (broadcast or in aligned vectors along B).
+template <class Op, int TA, int TB, int MASK>
+__global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* t, const typename Op::A* a, const typename Op::B* b,
+                                                         TrArgs p, uint32_t xcd_chunk) {
+    using T = typename Op::T;
+    using A = typename Op::A;
+    using B = typename Op::B;
+    using C = typename Op::C;
+    static_assert(Op::NSRC >= 1 && Op::NSRC <= 2 && (MASK == 1 || MASK == 2) && MASK <= Op::NSRC, "one staged source of one or two");
+    constexpr int VEC = 4;
+    constexpr bool S1 = MASK == 1;
+    using S = std::conditional_t<S1, A, B>;   // the staged source
+    using D = std::conditional_t<S1, B, A>;   // the other one (two-operand ops only)
+    static_assert(sizeof(S) == 4, "staged elements of four bytes");
+    constexpr int KS = S1 ? 1 : 2, KD = S1 ? 2 : 1;
+    constexpr bool HAS_D = Op::NSRC == 2;
+    constexpr int TVA = TA / VEC, RS = kBlock / TVA, JT = TB / (4 * RS);     // staging: threads along A, thread rows, passes of 4 * RS rows
+    constexpr int TVB = TB / VEC, RT = kBlock / TVB, ITER_T = TA / RT;       // storing: threads along B, rows per pass, passes
+    static_assert(TA % VEC == 0 && TB % 32 == 0 && kBlock % TVA == 0 && kBlock % TVB == 0 && TB % (4 * RS) == 0 && TA % RT == 0 && TVA % 8 == 0,
+                  "tile shape");
+    typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    extern __shared__ __align__(16) unsigned char tr_lds[];
+    u32x4* l = (u32x4*)tr_lds;                // [TA][TVB] groups
+    [[maybe_unused]] D* lv = (D*)(tr_lds + (size_t)TA * TB * 4);   // [TA] values of a source that has one per stored row
+    constexpr int NDV = (TA + kBlock - 1) / kBlock;
+    const S* sp = S1 ? (const S*)a : (const S*)b;
+    const D* dp = S1 ? (const D*)b : (const D*)a;
+
+    uint32_t bid = blockIdx.x;
+    if (xcd_chunk) bid = (bid % 8u) * xcd_chunk + bid / 8u;
+    const uint32_t tb = bid % p.tiles_b;
+    bid /= p.tiles_b;
+    const uint32_t ta = bid % p.tiles_a;
+    bid /= p.tiles_a;
+    const int64_t a0 = (int64_t)ta * TA, b0 = (int64_t)tb * TB;
+    int64_t ot = a0 * p.sa[0] + b0 * p.sb[0], os = a0 * p.sa[KS] + b0 * p.sb[KS], od = a0 * p.sa[KD] + b0 * p.sb[KD];
+    for (int d = p.nouter - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : bid / p.oshape[d];
+        const int64_t idx = bid - q * p.oshape[d];
+        bid = q;
+        ot += idx * p.ostride[0][d];
+        os += idx * p.ostride[KS][d];
+        od += idx * p.ostride[KD][d];
+    }
+    t += ot;
+    sp += os;
+    dp += od;
+
+    const uint32_t gl = threadIdx.x % TVB, tx = gl * VEC, ty = threadIdx.x / TVB;
+    const bool rows_only = p.dmode == 1;
+    {
+        const uint32_t lx = threadIdx.x % TVA, sy = threadIdx.x / TVA;    // a = 4 lx .. 4 lx + 3
+        Pack<S, VEC> g[JT][4];
+#pragma unroll
+        for (int jt = 0; jt < JT; jt++)
+#pragma unroll
+            for (int k = 0; k < 4; k++) g[jt][k] = load_pack<S, VEC>(sp + (int64_t)(4 * (RS * jt + sy) + k) * p.sb[KS] + 4 * lx);
+        // a source with one value per stored row: the tile's TA values go through LDS (one load per thread here, behind the staging
+        // loads and ahead of the wait for them; fetched by every storing thread for its own rows they cost as many load
+        // instructions as the tile itself)
+        [[maybe_unused]] D dv[NDV];
+        if constexpr (HAS_D) {
+            if (rows_only) {
+#pragma unroll
+                for (int q = 0; q < NDV; q++) dv[q] = dp[(int64_t)((threadIdx.x + q * kBlock) % TA) * p.sa[KD]];
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int jt = 0; jt < JT; jt++) {
+            const uint32_t grp = (RS * jt + sy) ^ (lx % 8u);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                u32x4 w;
+#pragma unroll
+                for (int k = 0; k < 4; k++) w[k] = __builtin_bit_cast(uint32_t, g[jt][k].v[e]);
+                l[(4 * lx + e) * TVB + grp] = w;
+            }
+        }
+        if constexpr (HAS_D) {
+            if (rows_only) {
+#pragma unroll
+                for (int q = 0; q < NDV; q++) lv[(threadIdx.x + q * kBlock) % TA] = dv[q];
+            }
+        }
+    }
+    __syncthreads();
+    [[maybe_unused]] D pd[ITER_T];
+    if constexpr (HAS_D) {
+        if (rows_only) {
+#pragma unroll
+            for (int it = 0; it < ITER_T; it++) pd[it] = lv[ty + it * RT];
+        }
+    }
+    auto store_tile = [&](auto mode_tag) {
+        constexpr int MODE = decltype(mode_tag)::value;
+        [[maybe_unused]] Pack<D, VEC> dd[ITER_T];
+        if constexpr (HAS_D && MODE == 2) {
+#pragma unroll
+            for (int i = 0; i < ITER_T; i++) dd[i] = tr_direct_fast<D, VEC>(dp, ty + i * RT, tx, p.sa[KD], p.sb[KD]);
+        }
+#pragma unroll
+        for (int i = 0; i < ITER_T; i++) {
+            const uint32_t r = ty + i * RT;
+            const u32x4 w = l[r * TVB + (gl ^ ((r / 4u) % 8u))];
+            Pack<T, VEC> res;
+#pragma unroll
+            for (int e = 0; e < VEC; e++) {
+                const S xs = __builtin_bit_cast(S, (uint32_t)w[e]);
+                D xd = D();
+                if constexpr (HAS_D) xd = MODE == 1 ? pd[i] : dd[i].v[e];
+                if constexpr (S1) res.v[e] = apply_op(op, xs, xd, C());
+                else res.v[e] = apply_op(op, xd, xs, C());
+            }
+            store_pack<T, VEC>(t + (int64_t)r * p.sa[0] + tx, res);
+        }
+    };
+    if (!HAS_D || rows_only) store_tile(std::integral_constant<int, 1>{});
+    else store_tile(std::integral_constant<int, 2>{});
+}
+
 // ---- launcher -------------------------------------------------------------------------------------------------------------
 
 template <class Op>
@@ -589,12 +717,26 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 for (int d = 0; d < q.nouter && ok; d++) ok = (q.ostride[k][d] % VEC) == 0;
                 if (!ok) q.dmode = 0;
             }
-            bool big = false;
+            // Large tiles (128 KB of LDS, one workgroup per CU) for 4-byte elements in whole tiles with one staged source:
+            //   256 x 128 when the target's rows are short (at most 256 elements);
+            //   128 x 256 (map_tr4_kernel only) for longer rows whose pitch in the target stays below 256 KB: 512 MiB copies of
+            //   8192 x 16384 250 -> 180 us, 16384 x 8192 207 -> 196, 1024 x 131072 207 -> 175, 64 x [2048 x 1024] 188 -> 167;
+            //   with a target pitch of 512 KB (131072 x 1024, or 256 x 512 x 1024 permuted to 1024 x 256 x 512) every large
+            //   tile shape and tile order measured 186 us or more, the 128 x 64 tiles' time, so those keep them.
+            bool big = false, tall = false, tr4 = false;
+            constexpr int TALL_TA = 128, TALL_TB = 256;
             if constexpr (!WIDE && VEC == 4 && Op::NSRC >= 1 && Op::NSRC <= 2) {
-                big = vec && nstaged == 1 && staged_esize == 4 && q.nb <= 256 && (q.na % BIG_TA) == 0 && (q.nb % BIG_TB) == 0 &&
+                static const bool tr4_on = [] { const char* e = getenv("DNH_TR4"); return !e || e[0] != '0'; }();
+                const bool tr4_ok = tr4_on && (Op::NSRC == 1 || q.dmode != 0);
+                const bool one4 = vec && nstaged == 1 && staged_esize == 4;
+                big = one4 && q.nb <= 256 && (q.na % BIG_TA) == 0 && (q.nb % BIG_TB) == 0 &&
                       (int64_t)(q.na / BIG_TA) * (q.nb / BIG_TB) * outer >= (int64_t)device_cus() * 8;
+                tall = !big && tr4_ok && one4 && q.nb > 256 && (q.na % TALL_TA) == 0 && (q.nb % TALL_TB) == 0 &&
+                       q.sa[0] * (int64_t)es[0] < 256 * 1024 &&
+                       (int64_t)(q.na / TALL_TA) * (q.nb / TALL_TB) * outer >= (int64_t)device_cus() * 8;
+                tr4 = tr4_ok && (big || tall);
             }
-            const int ta_n = big ? BIG_TA : TA, tb_n = big ? BIG_TB : TB;
+            const int ta_n = big ? BIG_TA : tall ? TALL_TA : TA, tb_n = big ? BIG_TB : tall ? TALL_TB : TB;
             q.tiles_a = cdiv(q.na, ta_n);
             q.tiles_b = cdiv(q.nb, tb_n);
             uint32_t lds_bytes = 0;
@@ -605,7 +747,7 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
             }
             const int64_t blocks = (int64_t)q.tiles_a * q.tiles_b * outer;
             if (blocks <= 0x7FFFFFFF) {
-                const uint32_t xcd_chunk = (!big && blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
+                const uint32_t xcd_chunk = (!big && !tall && blocks % 8 == 0 && blocks >= 64) ? (uint32_t)(blocks / 8) : 0u;
                 const int mask = (q.staged[1] ? 1 : 0) | (q.staged[2] ? 2 : 0) | (q.staged[3] ? 4 : 0);
                 int32_t st = DNH_ERR_NOT_SUPPORTED;
                 // launches map_tr_kernel<Op, TA_, TB_, V_, M_>; more than 64 KB of LDS (two or three staged sources, or the large tile)
@@ -639,7 +781,30 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
             }                                                                                            \
         }                                                                                                \
     } while (0)
-                if (big) {
+#define DNH_TR4_LAUNCH(TA_, TB_, M_)                                                                                                      \
+    do {                                                                                                                                  \
+        auto kern = map_tr4_kernel<Op, TA_, TB_, M_>;                                                                                     \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, TA_ * TB_ * 4 + TA_ * 4); \
+        if (attr != hipSuccess) { st = fail(DNH_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(attr)); break; }                    \
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBlock), (size_t)TA_ * TB_ * 4 + TA_ * 4, stream, op, t, a, b, q, xcd_chunk);                    \
+        st = DNH_OK;                                                                                                                      \
+    } while (0)
+                if (tr4) {
+                    if constexpr (!WIDE && VEC == 4 && Op::NSRC >= 1 && Op::NSRC <= 2) {
+                        // (the staged source is the one of four bytes: `staged_esize` above)
+#define DNH_TR4_PICK(TA_, TB_)                                                                           \
+    do {                                                                                                 \
+        if (mask == 1) {                                                                                 \
+            if constexpr (sizeof(A) == 4) DNH_TR4_LAUNCH(TA_, TB_, 1);                                   \
+        } else if constexpr (Op::NSRC == 2) {                                                            \
+            if constexpr (sizeof(B) == 4) DNH_TR4_LAUNCH(TA_, TB_, 2);                                   \
+        }                                                                                                \
+    } while (0)
+                        if (big) DNH_TR4_PICK(BIG_TA, BIG_TB);
+                        else DNH_TR4_PICK(TALL_TA, TALL_TB);
+#undef DNH_TR4_PICK
+                    }
+                } else if (big) {
                     if constexpr (!WIDE && VEC == 4 && Op::NSRC >= 1 && Op::NSRC <= 2) {
                         if constexpr (Op::NSRC == 1) DNH_TR_LAUNCH(BIG_TA, BIG_TB, 4, 1);
                         else if (mask == 1) DNH_TR_LAUNCH(BIG_TA, BIG_TB, 4, 1);
@@ -650,6 +815,7 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 } else {
                     DNH_TR_MASKS(TA, TB, 1);
                 }
+#undef DNH_TR4_LAUNCH
 #undef DNH_TR_MASKS
 #undef DNH_TR_LAUNCH
                 DNH_TRY(st);

@@ -43,6 +43,45 @@ def test_config2_permuted_broadcast_add_and_copy(G):
     assert_exact(np.transpose(x, (2, 0, 1)) + v[:, None, None], G.toNumpy(xq + tv[:, None, None]))
 
 
+def test_large_transposing_tiles_operand_order_types_and_modes(G):
+    """The large-tile transposing kernel (taken from 2048 tiles of 256 x 128 on) with the permuted operand first and second, a full
+    second operand, a row-wise and an element-wise broadcast one, a bool result and a converting copy; NumPy is the checker."""
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((256, 256, 1024), dtype=np.float32)
+    w = rng.standard_normal((256, 1024, 256), dtype=np.float32)
+    tx, tw = G.ofNumpy(x), G.ofNumpy(w)
+    xp = tx.permuteAxes([2, 0, 1])                               # shape [256, 1024, 256], strides [1024, 1, 262144]
+    assert xp.Shape == [256, 1024, 256] and xp.Stride == [1024, 1, 262144]
+    xt = np.transpose(x, (1, 2, 0))
+    assert_exact(xt - w, G.toNumpy(xp - tw))
+    assert_exact(w - xt, G.toNumpy(tw - xp))
+    assert_exact(xt > w, G.toNumpy(xp > tw))
+    r = rng.random(256, dtype=np.float32)
+    assert_exact(r[None, None, :] - xt, G.toNumpy(G.ofNumpy(r)[None, None, :] - xp))
+    v = rng.random(1024, dtype=np.float32)
+    assert_exact(v[None, :, None] - xt, G.toNumpy(G.ofNumpy(v)[None, :, None] - xp))
+    del w, tw
+    i = rng.integers(-2 ** 24, 2 ** 24, (256, 256, 1024), dtype=np.int32)
+    ip = G.ofNumpy(i).permuteAxes([2, 0, 1])
+    assert_exact(np.ascontiguousarray(np.transpose(i, (1, 2, 0))).astype(np.float32), G.toNumpy(ip.convert(np.float32)))
+
+
+def test_large_transposing_tiles_long_rows(G):
+    """The 128 x 256 tiles that transposes with long target rows take from 2048 tiles on: a plain 2-D transpose, both operand
+    orders, a row-wise operand and a bool result."""
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((8192, 8192), dtype=np.float32)
+    w = rng.standard_normal((8192, 8192), dtype=np.float32)
+    tx, tw = G.ofNumpy(x), G.ofNumpy(w)
+    assert_exact(np.ascontiguousarray(x.T), G.toNumpy(tx.T.Copy()))
+    assert_exact(x.T - w, G.toNumpy(tx.T - tw))
+    assert_exact(w - x.T, G.toNumpy(tw - tx.T))
+    assert_exact(x.T < w, G.toNumpy(tx.T < tw))
+    v = rng.random(8192, dtype=np.float32)
+    assert_exact(v[:, None] - x.T, G.toNumpy(G.ofNumpy(v)[:, None] - tx.T))
+    assert_exact(x.T - v[None, :], G.toNumpy(tx.T - G.ofNumpy(v)[None, :]))
+
+
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_config3_reductions_8192(G, dt):
     rng = np.random.default_rng(123)
