@@ -236,6 +236,70 @@ __global__ __launch_bounds__(kBlock) void map_nd_kernel(Op op, typename Op::T* t
     }
 }
 
+// The n-d kernel for calls whose target runs along the last dimension but that the vector form above cannot take: an operand that
+// is misaligned (a view that starts at an odd element: x[:, 1:] - x[:, :-1]), has row pitches that are not whole vectors, or is
+// strided along the last dimension, and rows whose length is not a multiple of VEC.  Every thread still handles VEC consecutive
+// elements of a row; per operand, `mode` says how it gets them: 0 one element for all (stride 0), 1 one aligned vector, 2 one
+// element at a time at `estride`.  The last item of a row may hold fewer than VEC elements (`lastlen` is the row length): that
+// item is moved element by element, with guards.  All of a thread's loads are issued before the first use.
+struct NdMixArgs {
+    int mode[kMaxOperands];          // [0] is the target: 1 vector stores, 2 element stores
+    int64_t estride[kMaxOperands];   // element stride along the last dimension
+    uint32_t lastlen;                // elements per row
+};
+
+template <class Op, int VEC>
+__global__ __launch_bounds__(kBlock) void map_nd_mix_kernel(Op op, typename Op::T* t, const typename Op::A* a, const typename Op::B* b,
+                                                            const typename Op::C* c, NdArgs p, NdMixArgs m, uint32_t nitems) {
+    using T = typename Op::T;
+    using A = typename Op::A;
+    using B = typename Op::B;
+    using C = typename Op::C;
+    const uint32_t item = blockIdx.x * (uint32_t)kBlock + threadIdx.x;
+    if (item >= nitems) return;
+    int64_t ot = 0, oa = 0, ob = 0, oc = 0;
+    uint32_t rem = item, ilast = 0;
+    for (int d = p.nd - 1; d >= 0; d--) {
+        const uint32_t q = (d == 0) ? 0u : fast_div(rem, p.div[d]);
+        const uint32_t idx = rem - q * p.shape[d];
+        rem = q;
+        if (d == p.nd - 1) ilast = idx;
+        ot += (int64_t)idx * p.stride[0][d];
+        if constexpr (Op::NSRC >= 1) oa += (int64_t)idx * p.stride[1][d];
+        if constexpr (Op::NSRC >= 2) ob += (int64_t)idx * p.stride[2][d];
+        if constexpr (Op::NSRC >= 3) oc += (int64_t)idx * p.stride[3][d];
+    }
+    const uint32_t left = m.lastlen - ilast * (uint32_t)VEC;     // elements of the row from this item on
+    const bool whole = left >= (uint32_t)VEC;
+    // element e of a partial item beyond the row's end reads element 0 of the item instead (and is not stored)
+    auto fetch = [&](auto* src, int64_t off, int mode, int64_t es) {
+        using X = std::remove_cv_t<std::remove_pointer_t<decltype(src)>>;
+        Pack<X, VEC> v;
+        if (mode == 1 && whole) return load_pack<X, VEC>(src + off);
+        if (mode == 0) return splat_pack<X, VEC>(src[off]);
+        const int64_t step = mode == 1 ? 1 : es;
+#pragma unroll
+        for (int e = 0; e < VEC; e++) v.v[e] = src[off + ((uint32_t)e < left ? e * step : 0)];
+        return v;
+    };
+    Pack<A, VEC> va;
+    Pack<B, VEC> vb;
+    Pack<C, VEC> vc;
+    if constexpr (Op::NSRC >= 1) va = fetch(a, oa, m.mode[1], m.estride[1]);
+    if constexpr (Op::NSRC >= 2) vb = fetch(b, ob, m.mode[2], m.estride[2]);
+    if constexpr (Op::NSRC >= 3) vc = fetch(c, oc, m.mode[3], m.estride[3]);
+    Pack<T, VEC> r;
+#pragma unroll
+    for (int e = 0; e < VEC; e++) r.v[e] = apply_op(op, va.v[e], vb.v[e], vc.v[e]);
+    if (m.mode[0] == 1 && whole) {
+        store_pack<T, VEC>(t + ot, r);
+    } else {
+#pragma unroll
+        for (int e = 0; e < VEC; e++)
+            if ((uint32_t)e < left) t[ot + e] = r.v[e];
+    }
+}
+
 // ---- LDS-staged transpose -------------------------------------------------------------------------------------------------
 
 struct TrArgs {
@@ -841,6 +905,33 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
     for (int d = 0; d < last && vec; d++)
         for (int k = 0; k < NOPS; k++)
             if (p.stride[k][last] == 1) vec = vec && (p.stride[k][d] % VEC) == 0;
+    // the target runs along the last dimension but something else keeps the vector form away: per-operand access modes
+    if constexpr (VEC > 1) {
+        if (!vec && nd >= 1 && p.stride[0][last] == 1 && p.shape[last] >= 4 * VEC) {
+            NdMixArgs mx;
+            memset(&mx, 0, sizeof(mx));
+            const int64_t L = p.shape[last];
+            for (int k = 0; k < NOPS; k++) {
+                bool whole_vectors = p.stride[k][last] == 1 && aligned_to(p.ptr[k], VEC * es[k]);
+                for (int d = 0; d < last && whole_vectors; d++) whole_vectors = (p.stride[k][d] % VEC) == 0;
+                mx.mode[k] = (k > 0 && p.stride[k][last] == 0) ? 0 : whole_vectors ? 1 : 2;
+                mx.estride[k] = p.stride[k][last];
+                q.stride[k][last] = p.stride[k][last] * VEC;
+            }
+            mx.lastlen = (uint32_t)L;
+            q.shape[last] = (uint32_t)((L + VEC - 1) / VEC);
+            for (int d = 0; d < q.nd; d++) q.div[d] = make_fast_div(q.shape[d]);
+            const int64_t nitems64 = (p.total / L) * q.shape[last];
+            if (nitems64 <= (int64_t)kMaxItems) {
+                const uint32_t nitems = (uint32_t)nitems64;
+                hipLaunchKernelGGL((map_nd_mix_kernel<Op, VEC>), dim3(cdiv(nitems, kBlock)), dim3(kBlock), 0, stream, op, t, a, b, c, q, mx, nitems);
+                DNH_LAUNCH_CHECK();
+                return DNH_OK;
+            }
+            q.shape[last] = (uint32_t)p.shape[last];
+            for (int k = 0; k < NOPS; k++) q.stride[k][last] = p.stride[k][last];
+        }
+    }
     constexpr int UNROLL = 1;
     if (vec) q.shape[last] = (uint32_t)(p.shape[last] / VEC);
     for (int d = 0; d < q.nd; d++) q.div[d] = make_fast_div(q.shape[d]);

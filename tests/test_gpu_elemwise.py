@@ -183,6 +183,42 @@ def test_strided_and_broadcast_views(H, G, rng, dt):
     assert_exact(ref, got)
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64, np.int32, np.uint8, np.int16, np.int64])
+def test_misaligned_ragged_and_strided_rows(H, G, rng, dt):
+    """Row-wise calls that the aligned vector kernels cannot take: differences of shifted views (every operand starts at another
+    element), odd row lengths, a target that is itself a shifted view, a source strided along the rows, a row-broadcast and a
+    column-broadcast operand beside them; NumPy is the checker, the oracle device the second one."""
+    x = rand(rng, dt, (37, 1031))
+    y = rand(rng, dt, (37, 1031))
+    v = rand(rng, dt, (1031,))
+    tx, ty, tv = G.ofNumpy(x), G.ofNumpy(y), G.ofNumpy(v)
+    assert_exact(x[:, 1:] - x[:, :-1], G.toNumpy(tx[:, 1:] - tx[:, :1030]))               # row length 1030, one operand misaligned
+    assert_exact(x[:, 3:1027] - y[:, 5:1029], G.toNumpy(tx[:, 3:1027] - ty[:, 5:1029]))  # whole vectors per row, both misaligned
+    assert_exact(x[:, 2:] - v[None, 2:], G.toNumpy(tx[:, 2:] - tv[None, 2:]))
+    assert_exact(x[:, 7:900] - y[:, 0:1][:, :].repeat(893, axis=1), G.toNumpy(tx[:, 7:900] - ty[:, 0:1].broadcastTo([37, 893])))
+    assert_exact(x[1:, 1:] > y[:-1, :-1], G.toNumpy(tx[1:, 1:] > ty[:36, :1030]))
+    # 1-d: the finite difference of a long vector
+    z = rand(rng, dt, (100003,))
+    tz = G.ofNumpy(z)
+    assert_exact(z[1:] - z[:-1], G.toNumpy(tz[1:] - tz[:100002]))
+    # a target that starts at an odd element and whose rows are not whole vectors
+    out = G.zeros([37, 1031], dt)
+    out[:, 1:].FillSubtract(tx[:, 1:], ty[:, :1030])
+    want = np.zeros_like(x)
+    want[:, 1:] = x[:, 1:] - y[:, :-1]
+    assert_exact(want, G.toNumpy(out))
+    # a source strided along the rows (a plane of a 3-d tensor) against a contiguous one
+    c = rand(rng, dt, (29, 515, 3))
+    d = rand(rng, dt, (29, 515))
+    tc, td = G.ofNumpy(c), G.ofNumpy(d)
+    assert_exact(c[:, :, 1] - d, G.toNumpy(tc[:, :, 1] - td))
+    assert_exact(d[:, ::-1] - c[:, :, 2], G.toNumpy(td.reverseAxis(1) - tc[:, :, 2]))
+    # the oracle device on the same views
+    ref, got = both(H, G, lambda a, b: (a[:, 1:] - b[:, :1030], a[2:, 5:] + b[:35, :1026]), x, y)
+    assert_exact(ref[0], got[0])
+    assert_exact(ref[1], got[1])
+
+
 def test_large_transpose_copy_and_add(H, G, rng):
     x = rng.standard_normal((16, 96, 200)).astype(np.float32)
     v = rng.random(200).astype(np.float32)
