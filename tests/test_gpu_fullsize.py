@@ -82,6 +82,34 @@ def test_large_transposing_tiles_long_rows(G):
     assert_exact(x.T - v[None, :], G.toNumpy(tx.T - G.ofNumpy(v)[None, :]))
 
 
+def test_transposing_calls_on_ragged_shapes(G):
+    """Transposing calls at full size on extents that are not multiples of the tiles: target rows that are not whole vectors
+    (250 elements), a second operand of the target's shape, a row-wise one, a bool result; NumPy is the checker."""
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((250, 500, 1000), dtype=np.float32)
+    tx = G.ofNumpy(x)
+    xp = tx.permuteAxes([2, 0, 1])                               # shape [500, 1000, 250], strides [1000, 1, 500000]
+    assert xp.Shape == [500, 1000, 250]
+    xt = np.transpose(x, (1, 2, 0))
+    assert_exact(np.ascontiguousarray(xt), G.toNumpy(xp.Copy()))
+    v = rng.random(1000, dtype=np.float32)
+    assert_exact(xt - v[None, :, None], G.toNumpy(xp - G.ofNumpy(v)[None, :, None]))
+    w = rng.standard_normal((500, 1000, 250), dtype=np.float32)
+    tw = G.ofNumpy(w)
+    assert_exact(w - xt, G.toNumpy(tw - xp))
+    assert_exact(xt <= w, G.toNumpy(xp <= tw))
+    del w, tw, x, tx, xp, xt
+    # 2-d, long rows: 9000 x 7000 -> 7000 x 9000 (edge tiles on both sides, whole vectors)
+    y = rng.standard_normal((9000, 7000), dtype=np.float32)
+    z = rng.standard_normal((7000, 9000), dtype=np.float32)
+    ty, tz = G.ofNumpy(y), G.ofNumpy(z)
+    assert_exact(np.ascontiguousarray(y.T), G.toNumpy(ty.T.Copy()))
+    assert_exact(y.T - z, G.toNumpy(ty.T - tz))
+    # ... and rows of 9001 elements in the target (element stores), the source's rows still whole vectors
+    y2 = rng.standard_normal((9001, 7000), dtype=np.float32)
+    assert_exact(np.ascontiguousarray(y2.T), G.toNumpy(G.ofNumpy(y2).T.Copy()))
+
+
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 def test_config3_reductions_8192(G, dt):
     rng = np.random.default_rng(123)
