@@ -44,10 +44,7 @@ extern "C" int32_t dnh_binary(int32_t op, const DnhTensor* t, const DnhTensor* a
         case DNH_ADD: return run_numeric<OpAdd>(dt, p, s);
         case DNH_SUBTRACT: return run_numeric<OpSub>(dt, p, s);
         case DNH_MULTIPLY: return run_numeric<OpMul>(dt, p, s);
-        case DNH_DIVIDE: return run_numeric<OpDiv>(dt, p, s);
-        case DNH_MODULO: return run_numeric<OpMod>(dt, p, s);
-        case DNH_MAX_ELEMWISE: return run_numeric<OpMax>(dt, p, s);
-        case DNH_MIN_ELEMWISE: return run_numeric<OpMin>(dt, p, s);
+        case DNH_DIVIDE: case DNH_MODULO: case DNH_MAX_ELEMWISE: case DNH_MIN_ELEMWISE: return binary_second_unit(op, dt, p, s);
         case DNH_POWER:
             if (dt == DNH_F32) return launch_map(OpPow<float>{}, p, s);
             if (dt == DNH_F64) return launch_map(OpPow<double>{}, p, s);

@@ -37,9 +37,7 @@ extern "C" int32_t dnh_compare(int32_t op, const DnhTensor* t, const DnhTensor* 
         case DNH_EQUAL: return run_cmp<OpEq>(a->dtype, p, s);
         case DNH_NOT_EQUAL: return run_cmp<OpNe>(a->dtype, p, s);
         case DNH_LESS: return run_cmp<OpLt>(a->dtype, p, s);
-        case DNH_LESS_OR_EQUAL: return run_cmp<OpLe>(a->dtype, p, s);
-        case DNH_GREATER: return run_cmp<OpGt>(a->dtype, p, s);
-        case DNH_GREATER_OR_EQUAL: return run_cmp<OpGe>(a->dtype, p, s);
+        case DNH_LESS_OR_EQUAL: case DNH_GREATER: case DNH_GREATER_OR_EQUAL: return compare_second_unit(op, a->dtype, p, s);
     }
     return fail(DNH_ERR_INVALID_ARG, "dnh_compare: unknown op %d", op);
 }
