@@ -523,8 +523,8 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
     }
 }
 
-// The transposing kernel for 4-byte staged elements and whole tiles, with both LDS phases free of bank conflicts and on 16-byte
-// LDS instructions.  map_tr_kernel's [b][a + 1] tile is written with one 4-byte store per element at a lane stride of four words
+// The transposing kernel for 4- and 8-byte staged elements and whole tiles, with both LDS phases free of bank conflicts and on
+// 16-byte LDS instructions (described for 4-byte elements, VEC = 4; 8-byte elements have VEC = 2, blocks of 2 x 2 and groups of two b's).  map_tr_kernel's [b][a + 1] tile is written with one 4-byte store per element at a lane stride of four words
 // (8 of the 32 banks) and read element by element (16 banks).  Here a staging thread fetches the same vector of four a's from
 // four consecutive rows b, so that it holds a 4 x 4 block, and writes its four columns: LDS is [a][b] in 16-byte groups of four
 // b's, group g of row a stored at g ^ ((a / 4) % 8); consecutive lanes (a four apart) then fall into different groups, and a storing
@@ -539,21 +539,23 @@ __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* 
     using B = typename Op::B;
     using C = typename Op::C;
     static_assert(Op::NSRC >= 1 && Op::NSRC <= 2 && (MASK == 1 || MASK == 2) && MASK <= Op::NSRC, "one staged source of one or two");
-    constexpr int VEC = 4;
+    using S0 = std::conditional_t<MASK == 1, A, B>;
+    static_assert(sizeof(S0) == 4 || sizeof(S0) == 8, "staged elements of four or eight bytes");
+    constexpr int VEC = 16 / (int)sizeof(S0);   // elements per 16-byte group: the blocks a staging thread holds are VEC x VEC
     constexpr bool S1 = MASK == 1;
     using S = std::conditional_t<S1, A, B>;   // the staged source
     using D = std::conditional_t<S1, B, A>;   // the other one (two-operand ops only)
-    static_assert(sizeof(S) == 4, "staged elements of four bytes");
     constexpr int KS = S1 ? 1 : 2, KD = S1 ? 2 : 1;
     constexpr bool HAS_D = Op::NSRC == 2;
-    constexpr int TVA = TA / VEC, RS = kBlock / TVA, JT = TB / (4 * RS);     // staging: threads along A, thread rows, passes of 4 * RS rows
+    constexpr int TVA = TA / VEC, RS = kBlock / TVA, JT = TB / (VEC * RS);     // staging: threads along A, thread rows, passes of VEC * RS rows
     constexpr int TVB = TB / VEC, RT = kBlock / TVB, ITER_T = TA / RT;       // storing: threads along B, rows per pass, passes
-    static_assert(TA % VEC == 0 && TB % 32 == 0 && kBlock % TVA == 0 && kBlock % TVB == 0 && TB % (4 * RS) == 0 && TA % RT == 0 && TVA % 8 == 0,
+    static_assert(TA % VEC == 0 && TB % 32 == 0 && kBlock % TVA == 0 && kBlock % TVB == 0 && TB % (VEC * RS) == 0 && TA % RT == 0 && TVA % 8 == 0,
                   "tile shape");
     typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+    struct Group { S v[VEC]; };               // VEC consecutive b's of one a: 16 bytes
     extern __shared__ __align__(16) unsigned char tr_lds[];
     u32x4* l = (u32x4*)tr_lds;                // [TA][TVB] groups
-    [[maybe_unused]] D* lv = (D*)(tr_lds + (size_t)TA * TB * 4);   // [TA] values of a source that has one per stored row
+    [[maybe_unused]] D* lv = (D*)(tr_lds + (size_t)TA * TB * sizeof(S));   // [TA] values of a source that has one per stored row
     constexpr int NDV = (TA + kBlock - 1) / kBlock;
     const S* sp = S1 ? (const S*)a : (const S*)b;
     const D* dp = S1 ? (const D*)b : (const D*)a;
@@ -581,12 +583,12 @@ __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* 
     const uint32_t gl = threadIdx.x % TVB, tx = gl * VEC, ty = threadIdx.x / TVB;
     const bool rows_only = p.dmode == 1;
     {
-        const uint32_t lx = threadIdx.x % TVA, sy = threadIdx.x / TVA;    // a = 4 lx .. 4 lx + 3
-        Pack<S, VEC> g[JT][4];
+        const uint32_t lx = threadIdx.x % TVA, sy = threadIdx.x / TVA;    // a = VEC lx .. VEC lx + VEC - 1
+        Pack<S, VEC> g[JT][VEC];
 #pragma unroll
         for (int jt = 0; jt < JT; jt++)
 #pragma unroll
-            for (int k = 0; k < 4; k++) g[jt][k] = load_pack<S, VEC>(sp + (int64_t)(4 * (RS * jt + sy) + k) * p.sb[KS] + 4 * lx);
+            for (int k = 0; k < VEC; k++) g[jt][k] = load_pack<S, VEC>(sp + (int64_t)(VEC * (RS * jt + sy) + k) * p.sb[KS] + VEC * lx);
         // a source with one value per stored row: the tile's TA values go through LDS (one load per thread here, behind the staging
         // loads and ahead of the wait for them; fetched by every storing thread for its own rows they cost as many load
         // instructions as the tile itself)
@@ -602,11 +604,11 @@ __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* 
         for (int jt = 0; jt < JT; jt++) {
             const uint32_t grp = (RS * jt + sy) ^ (lx % 8u);
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                u32x4 w;
+            for (int e = 0; e < VEC; e++) {
+                Group w;
 #pragma unroll
-                for (int k = 0; k < 4; k++) w[k] = __builtin_bit_cast(uint32_t, g[jt][k].v[e]);
-                l[(4 * lx + e) * TVB + grp] = w;
+                for (int k = 0; k < VEC; k++) w.v[k] = g[jt][k].v[e];
+                l[(VEC * lx + e) * TVB + grp] = __builtin_bit_cast(u32x4, w);
             }
         }
         if constexpr (HAS_D) {
@@ -634,11 +636,11 @@ __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* 
 #pragma unroll
         for (int i = 0; i < ITER_T; i++) {
             const uint32_t r = ty + i * RT;
-            const u32x4 w = l[r * TVB + (gl ^ ((r / 4u) % 8u))];
+            const Group w = __builtin_bit_cast(Group, l[r * TVB + (gl ^ ((r / (uint32_t)VEC) % 8u))]);
             Pack<T, VEC> res;
 #pragma unroll
             for (int e = 0; e < VEC; e++) {
-                const S xs = __builtin_bit_cast(S, (uint32_t)w[e]);
+                const S xs = w.v[e];
                 D xd = D();
                 if constexpr (HAS_D) xd = MODE == 1 ? pd[i] : dd[i].v[e];
                 if constexpr (S1) res.v[e] = apply_op(op, xs, xd, C());
@@ -665,6 +667,7 @@ constexpr int op_vec() {
 inline bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
 
 constexpr uint32_t kMaxItems = 0xFFFF0000u;
+
 
 template <class Op>
 int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
@@ -741,7 +744,8 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
             constexpr bool WIDE = sizeof(T) > 4 || (Op::NSRC >= 1 && sizeof(A) > 4) || (Op::NSRC >= 2 && sizeof(B) > 4) ||
                                   (Op::NSRC >= 3 && sizeof(C) > 4);
             constexpr int TA = WIDE ? 64 : 128, TB = WIDE ? 32 : 64;
-            constexpr int BIG_TA = 256, BIG_TB = 128;
+            constexpr int ESZ = WIDE ? 8 : 4;                       // element size of the large tiles' staged source
+            constexpr int BIG_TA = WIDE ? 128 : 256, BIG_TB = 128;
             TrArgs q;
             memset(&q, 0, sizeof(q));
             q.na = (uint32_t)p.shape[dA];
@@ -781,19 +785,22 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 for (int d = 0; d < q.nouter && ok; d++) ok = (q.ostride[k][d] % VEC) == 0;
                 if (!ok) q.dmode = 0;
             }
-            // Large tiles (128 KB of LDS, one workgroup per CU) for 4-byte elements in whole tiles with one staged source:
-            //   256 x 128 when the target's rows are short (at most 256 elements);
-            //   128 x 256 (map_tr4_kernel only) for longer rows whose pitch in the target stays below 256 KB: 512 MiB copies of
+            // Large tiles (128 KB of LDS, one workgroup per CU) for 4- and 8-byte elements in whole tiles with one staged source:
+            //   256 x 128 (8-byte elements: 128 x 128) when the target's rows are short (at most 256 elements);
+            //   128 x 256 (8-byte: 128 x 128; map_tr4_kernel only) for longer rows whose pitch in the target stays below 256 KB: 512 MiB copies of
             //   8192 x 16384 250 -> 180 us, 16384 x 8192 207 -> 196, 1024 x 131072 207 -> 175, 64 x [2048 x 1024] 188 -> 167;
             //   with a target pitch of 512 KB (131072 x 1024, or 256 x 512 x 1024 permuted to 1024 x 256 x 512) every large
             //   tile shape and tile order measured 186 us or more, the 128 x 64 tiles' time, so those keep them.
+            //   8-byte elements (512 MiB copies, 64 x 32 tiles of map_tr_kernel before): 8192 x 8192 244 -> 181 us, 4096 x 16384 245 -> 182,
+            //   16384 x 4096 216 -> 195, 1024 x 65536 198 -> 174, 64 x [1024 x 1024] 197 -> 164, [256, 512, 512] permuted to [512, 512, 256]
+            //   185 -> 173; 64 x 256, 256 x 64 and 32 x 512 tiles measured no better than 128 x 128 over these layouts.
             bool big = false, tall = false, tr4 = false;
-            constexpr int TALL_TA = 128, TALL_TB = 256;
-            if constexpr (!WIDE && VEC == 4 && Op::NSRC >= 1 && Op::NSRC <= 2) {
+            constexpr int TALL_TA = 128, TALL_TB = WIDE ? 128 : 256;
+            if constexpr (VEC == 16 / ESZ && Op::NSRC >= 1 && Op::NSRC <= 2) {
                 static const bool tr4_on = [] { const char* e = getenv("DNH_TR4"); return !e || e[0] != '0'; }();
                 const bool tr4_ok = tr4_on && (Op::NSRC == 1 || q.dmode != 0);
-                const bool one4 = vec && nstaged == 1 && staged_esize == 4;
-                big = one4 && q.nb <= 256 && (q.na % BIG_TA) == 0 && (q.nb % BIG_TB) == 0 &&
+                const bool one4 = vec && nstaged == 1 && staged_esize == ESZ;
+                big = (tr4_ok || !WIDE) && one4 && q.nb <= 256 && (q.na % BIG_TA) == 0 && (q.nb % BIG_TB) == 0 &&
                       (int64_t)(q.na / BIG_TA) * (q.nb / BIG_TB) * outer >= (int64_t)device_cus() * 8;
                 tall = !big && tr4_ok && one4 && q.nb > 256 && (q.na % TALL_TA) == 0 && (q.nb % TALL_TB) == 0 &&
                        q.sa[0] * (int64_t)es[0] < 256 * 1024 &&
@@ -848,20 +855,20 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
 #define DNH_TR4_LAUNCH(TA_, TB_, M_)                                                                                                      \
     do {                                                                                                                                  \
         auto kern = map_tr4_kernel<Op, TA_, TB_, M_>;                                                                                     \
-        static const hipError_t attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, TA_ * TB_ * 4 + TA_ * 4); \
+        static const hipError_t attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, TA_ * TB_ * ESZ + TA_ * 8); \
         if (attr != hipSuccess) { st = fail(DNH_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(attr)); break; }                    \
-        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBlock), (size_t)TA_ * TB_ * 4 + TA_ * 4, stream, op, t, a, b, q, xcd_chunk);                    \
+        hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBlock), (size_t)TA_ * TB_ * ESZ + TA_ * 8, stream, op, t, a, b, q, xcd_chunk);                    \
         st = DNH_OK;                                                                                                                      \
     } while (0)
                 if (tr4) {
-                    if constexpr (!WIDE && VEC == 4 && Op::NSRC >= 1 && Op::NSRC <= 2) {
+                    if constexpr (VEC == 16 / ESZ && Op::NSRC >= 1 && Op::NSRC <= 2) {
                         // (the staged source is the one of four bytes: `staged_esize` above)
 #define DNH_TR4_PICK(TA_, TB_)                                                                           \
     do {                                                                                                 \
         if (mask == 1) {                                                                                 \
-            if constexpr (sizeof(A) == 4) DNH_TR4_LAUNCH(TA_, TB_, 1);                                   \
+            if constexpr (sizeof(A) == ESZ) DNH_TR4_LAUNCH(TA_, TB_, 1);                                   \
         } else if constexpr (Op::NSRC == 2) {                                                            \
-            if constexpr (sizeof(B) == 4) DNH_TR4_LAUNCH(TA_, TB_, 2);                                   \
+            if constexpr (sizeof(B) == ESZ) DNH_TR4_LAUNCH(TA_, TB_, 2);                                   \
         }                                                                                                \
     } while (0)
                         if (big) DNH_TR4_PICK(BIG_TA, BIG_TB);

@@ -82,6 +82,30 @@ def test_large_transposing_tiles_long_rows(G):
     assert_exact(x.T - v[None, :], G.toNumpy(tx.T - G.ofNumpy(v)[None, :]))
 
 
+def test_large_transposing_tiles_double_precision(G):
+    """The same kernel on 8-byte elements (two elements per 16-byte group, 128 x 128 tiles): short target rows with a row-wise
+    operand, long rows with a second operand in either position, a bool result."""
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((256, 128, 1024))
+    tx = G.ofNumpy(x)
+    xp = tx.permuteAxes([2, 0, 1])                               # shape [128, 1024, 256]
+    assert xp.Shape == [128, 1024, 256]
+    xt = np.transpose(x, (1, 2, 0))
+    assert_exact(np.ascontiguousarray(xt), G.toNumpy(xp.Copy()))
+    v = rng.random(1024)
+    assert_exact(xt - v[None, :, None], G.toNumpy(xp - G.ofNumpy(v)[None, :, None]))
+    del x, tx, xp, xt
+    y = rng.standard_normal((4096, 8192))
+    z = rng.standard_normal((8192, 4096))
+    ty, tz = G.ofNumpy(y), G.ofNumpy(z)
+    assert_exact(np.ascontiguousarray(y.T), G.toNumpy(ty.T.Copy()))
+    assert_exact(y.T - z, G.toNumpy(ty.T - tz))
+    assert_exact(z - y.T, G.toNumpy(tz - ty.T))
+    assert_exact(y.T >= z, G.toNumpy(ty.T >= tz))
+    i = rng.integers(-2 ** 62, 2 ** 62, (4096, 8192), dtype=np.int64)
+    assert_exact(np.ascontiguousarray(i.T), G.toNumpy(G.ofNumpy(i).T.Copy()))
+
+
 def test_transposing_calls_on_ragged_shapes(G):
     """Transposing calls at full size on extents that are not multiples of the tiles: target rows that are not whole vectors
     (250 elements), a second operand of the target's shape, a row-wise one, a bool result; NumPy is the checker."""
