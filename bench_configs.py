@@ -48,6 +48,22 @@ def nsets_for(nbytes):
     return max(1, min(40, math.ceil(600e6 / max(nbytes, 1))))
 
 
+def profiled_call_traffic(tag):
+    """HBM bytes one call moves according to the committed hardware-counter summary (`traffic_bytes_per_call <tag> <bytes>` lines of
+    profiles/configs_1_to_6_all_kernels.txt), or None.  Used for the calls whose traffic is far from their algorithmic bytes."""
+    import os
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "configs_1_to_6_all_kernels.txt")
+    try:
+        with open(path) as f:
+            for line in f:
+                parts = line.split()
+                if len(parts) == 3 and parts[0] == "traffic_bytes_per_call" and parts[1] == tag:
+                    return int(parts[2])
+    except OSError:
+        pass
+    return None
+
+
 def report(log, cfg, name, ms, nbytes=None, flops=None, fp64=False):
     """One line of the per-configuration table: `frac` is the fraction of the roofline that bounds the call (8 TB/s of HBM for
     algorithmic bytes, or the fp32 / fp64 matrix peak for a product's FLOPs)."""
@@ -58,7 +74,16 @@ def report(log, cfg, name, ms, nbytes=None, flops=None, fp64=False):
         return {"cfg": cfg, "op": name, "us": round(ms * 1e3, 2), "flops": int(flops), "TFLOPs": round(tf, 2), "bound": "mfma", "frac": round(tf / peak, 4)}
     gb = nbytes / (ms * 1e-3) / 1e9
     log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {gb:8.1f} GB/s  {100 * gb / HBM_PEAK_GBS:5.1f}% of HBM peak  ({nbytes / 1e6:.1f} MB)")
-    return {"cfg": cfg, "op": name, "us": round(ms * 1e3, 2), "bytes": int(nbytes), "GBps": round(gb, 1), "bound": "hbm", "frac": round(gb / HBM_PEAK_GBS, 4)}
+    row = {"cfg": cfg, "op": name, "us": round(ms * 1e3, 2), "bytes": int(nbytes), "GBps": round(gb, 1), "bound": "hbm", "frac": round(gb / HBM_PEAK_GBS, 4)}
+    # gather / scatter move far more than their algorithmic bytes (a cache line per random 4-byte access): the counter-measured
+    # traffic of the call and the rate it stands for are reported beside the algorithmic figures
+    tag = "Gather" if name.startswith("Gather") else "Scatter" if "Scatter" in name else None
+    traffic = profiled_call_traffic(tag) if tag else None
+    if traffic:
+        row.update({"traffic_bytes": traffic, "traffic_GBps": round(traffic / (ms * 1e-3) / 1e9, 1),
+                    "traffic_frac": round(traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic_source": "profiles/configs_1_to_6_all_kernels.txt"})
+        log(f"       (counter-measured traffic of this call {traffic / 1e6:.1f} MB = {traffic / (ms * 1e-3) / 1e9:.0f} GB/s = {100 * traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS:.1f}% of HBM peak)")
+    return row
 
 
 def summarise(results):
