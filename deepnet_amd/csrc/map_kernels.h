@@ -69,6 +69,31 @@ __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& r) {
     }
 }
 
+// 16-byte accesses at addresses that are only aligned to the element (4 or 8 bytes): the hardware serves them (measured on a
+// 256 MiB copy with every combination of source and target offsets: 5.8-6.05 TB/s and every element right, against 3.5 TB/s for the
+// same copy with 4-byte accesses), and the compiler emits one instruction for an access declared with the element's alignment.
+template <class T, int N>
+struct __attribute__((packed, aligned(alignof(T)))) UnalignedPack {
+    T v[N];
+};
+template <class T, int N>
+__device__ __forceinline__ Pack<T, N> load_pack_unaligned(const T* p) {
+    static_assert(sizeof(T) >= 4 && sizeof(T) * N == 16, "elements of 4 or 8 bytes, one 16-byte access");
+    const UnalignedPack<T, N> u = *reinterpret_cast<const UnalignedPack<T, N>*>(p);
+    Pack<T, N> r;
+#pragma unroll
+    for (int i = 0; i < N; i++) r.v[i] = u.v[i];
+    return r;
+}
+template <class T, int N>
+__device__ __forceinline__ void store_pack_unaligned(T* p, const Pack<T, N>& r) {
+    static_assert(sizeof(T) >= 4 && sizeof(T) * N == 16, "elements of 4 or 8 bytes, one 16-byte access");
+    UnalignedPack<T, N> u;
+#pragma unroll
+    for (int i = 0; i < N; i++) u.v[i] = r.v[i];
+    *reinterpret_cast<UnalignedPack<T, N>*>(p) = u;
+}
+
 template <class T, int N>
 __device__ __forceinline__ Pack<T, N> splat_pack(T x) {
     Pack<T, N> r;
@@ -240,10 +265,11 @@ __global__ __launch_bounds__(kBlock) void map_nd_kernel(Op op, typename Op::T* t
 // is misaligned (a view that starts at an odd element: x[:, 1:] - x[:, :-1]), has row pitches that are not whole vectors, or is
 // strided along the last dimension, and rows whose length is not a multiple of VEC.  Every thread still handles VEC consecutive
 // elements of a row; per operand, `mode` says how it gets them: 0 one element for all (stride 0), 1 one aligned vector, 2 one
-// element at a time at `estride`.  The last item of a row may hold fewer than VEC elements (`lastlen` is the row length): that
+// element at a time at `estride`, 3 one 16-byte access at an address aligned to the element only (unit stride, elements of 4 or
+// 8 bytes).  The last item of a row may hold fewer than VEC elements (`lastlen` is the row length): that
 // item is moved element by element, with guards.  All of a thread's loads are issued before the first use.
 struct NdMixArgs {
-    int mode[kMaxOperands];          // [0] is the target: 1 vector stores, 2 element stores
+    int mode[kMaxOperands];          // [0] is the target: 1 vector stores, 2 element stores, 3 vector stores at element alignment
     int64_t estride[kMaxOperands];   // element stride along the last dimension
     uint32_t lastlen;                // elements per row
 };
@@ -277,7 +303,10 @@ __global__ __launch_bounds__(kBlock) void map_nd_mix_kernel(Op op, typename Op::
         Pack<X, VEC> v;
         if (mode == 1 && whole) return load_pack<X, VEC>(src + off);
         if (mode == 0) return splat_pack<X, VEC>(src[off]);
-        const int64_t step = mode == 1 ? 1 : es;
+        if constexpr (sizeof(X) >= 4 && sizeof(X) * VEC == 16) {
+            if (mode == 3 && whole) return load_pack_unaligned<X, VEC>(src + off);
+        }
+        const int64_t step = mode == 2 ? es : 1;
 #pragma unroll
         for (int e = 0; e < VEC; e++) v.v[e] = src[off + ((uint32_t)e < left ? e * step : 0)];
         return v;
@@ -293,6 +322,8 @@ __global__ __launch_bounds__(kBlock) void map_nd_mix_kernel(Op op, typename Op::
     for (int e = 0; e < VEC; e++) r.v[e] = apply_op(op, va.v[e], vb.v[e], vc.v[e]);
     if (m.mode[0] == 1 && whole) {
         store_pack<T, VEC>(t + ot, r);
+    } else if (sizeof(T) >= 4 && sizeof(T) * VEC == 16 && m.mode[0] == 3 && whole) {
+        if constexpr (sizeof(T) >= 4 && sizeof(T) * VEC == 16) store_pack_unaligned<T, VEC>(t + ot, r);
     } else {
 #pragma unroll
         for (int e = 0; e < VEC; e++)
@@ -921,7 +952,7 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
             for (int k = 0; k < NOPS; k++) {
                 bool whole_vectors = p.stride[k][last] == 1 && aligned_to(p.ptr[k], VEC * es[k]);
                 for (int d = 0; d < last && whole_vectors; d++) whole_vectors = (p.stride[k][d] % VEC) == 0;
-                mx.mode[k] = (k > 0 && p.stride[k][last] == 0) ? 0 : whole_vectors ? 1 : 2;
+                mx.mode[k] = (k > 0 && p.stride[k][last] == 0) ? 0 : whole_vectors ? 1 : (p.stride[k][last] == 1 && es[k] >= 4 && es[k] * VEC == 16) ? 3 : 2;
                 mx.estride[k] = p.stride[k][last];
                 q.stride[k][last] = p.stride[k][last] * VEC;
             }
