@@ -33,16 +33,25 @@ struct Pack {
     T v[N];
 };
 
+// The word type a pack of N elements of T moves as.  Elements of 4 bytes and more: declared with the element's alignment only.
+// The hardware serves 8- and 16-byte accesses at any dword address (measured on a 256 MiB copy with every combination of source
+// and target offsets: 5.8-6.05 TB/s and every element right, against 3.5 TB/s with 4-byte accesses), the compiler emits the same
+// single instruction, and views that start at an odd element or have odd row pitches keep the vector kernels.  Narrower
+// elements keep the natural alignment of the word (their launchers check it).
+template <class T, int BYTES, bool ELEM_ALIGNED = (sizeof(T) >= 4)> struct PackWord { using type = typename RawWord<BYTES>::type; };
+template <class T> struct PackWord<T, 8, true> { typedef uint32_t type __attribute__((ext_vector_type(2), aligned(4))); };
+template <class T> struct PackWord<T, 16, true> { typedef uint32_t type __attribute__((ext_vector_type(4), aligned(4))); };
+
 // packs wider than 16 bytes move as consecutive 16-byte words
 template <class T, int N>
 __device__ __forceinline__ Pack<T, N> load_pack(const T* p) {
     Pack<T, N> r;
     if constexpr (sizeof(T) * N <= 16) {
-        using W = typename RawWord<sizeof(T) * N>::type;
+        using W = typename PackWord<T, sizeof(T) * N>::type;
         W w = __builtin_nontemporal_load((const W*)p);
         __builtin_memcpy(&r, &w, sizeof(w));
     } else {
-        using W = typename RawWord<16>::type;
+        using W = typename PackWord<T, 16>::type;
         constexpr int NW = (int)(sizeof(T) * N / 16);
         W w[NW];
 #pragma unroll
@@ -55,43 +64,18 @@ __device__ __forceinline__ Pack<T, N> load_pack(const T* p) {
 template <class T, int N>
 __device__ __forceinline__ void store_pack(T* p, const Pack<T, N>& r) {
     if constexpr (sizeof(T) * N <= 16) {
-        using W = typename RawWord<sizeof(T) * N>::type;
+        using W = typename PackWord<T, sizeof(T) * N>::type;
         W w;
         __builtin_memcpy(&w, &r, sizeof(w));
         __builtin_nontemporal_store(w, (W*)p);
     } else {
-        using W = typename RawWord<16>::type;
+        using W = typename PackWord<T, 16>::type;
         constexpr int NW = (int)(sizeof(T) * N / 16);
         W w[NW];
         __builtin_memcpy(w, &r, sizeof(w));
 #pragma unroll
         for (int i = 0; i < NW; i++) __builtin_nontemporal_store(w[i], (W*)p + i);
     }
-}
-
-// 16-byte accesses at addresses that are only aligned to the element (4 or 8 bytes): the hardware serves them (measured on a
-// 256 MiB copy with every combination of source and target offsets: 5.8-6.05 TB/s and every element right, against 3.5 TB/s for the
-// same copy with 4-byte accesses), and the compiler emits one instruction for an access declared with the element's alignment.
-template <class T, int N>
-struct __attribute__((packed, aligned(alignof(T)))) UnalignedPack {
-    T v[N];
-};
-template <class T, int N>
-__device__ __forceinline__ Pack<T, N> load_pack_unaligned(const T* p) {
-    static_assert(sizeof(T) >= 4 && sizeof(T) * N == 16, "elements of 4 or 8 bytes, one 16-byte access");
-    const UnalignedPack<T, N> u = *reinterpret_cast<const UnalignedPack<T, N>*>(p);
-    Pack<T, N> r;
-#pragma unroll
-    for (int i = 0; i < N; i++) r.v[i] = u.v[i];
-    return r;
-}
-template <class T, int N>
-__device__ __forceinline__ void store_pack_unaligned(T* p, const Pack<T, N>& r) {
-    static_assert(sizeof(T) >= 4 && sizeof(T) * N == 16, "elements of 4 or 8 bytes, one 16-byte access");
-    UnalignedPack<T, N> u;
-#pragma unroll
-    for (int i = 0; i < N; i++) u.v[i] = r.v[i];
-    *reinterpret_cast<UnalignedPack<T, N>*>(p) = u;
 }
 
 template <class T, int N>
@@ -265,11 +249,10 @@ __global__ __launch_bounds__(kBlock) void map_nd_kernel(Op op, typename Op::T* t
 // is misaligned (a view that starts at an odd element: x[:, 1:] - x[:, :-1]), has row pitches that are not whole vectors, or is
 // strided along the last dimension, and rows whose length is not a multiple of VEC.  Every thread still handles VEC consecutive
 // elements of a row; per operand, `mode` says how it gets them: 0 one element for all (stride 0), 1 one aligned vector, 2 one
-// element at a time at `estride`, 3 one 16-byte access at an address aligned to the element only (unit stride, elements of 4 or
-// 8 bytes).  The last item of a row may hold fewer than VEC elements (`lastlen` is the row length): that
+// element at a time at `estride`.  The last item of a row may hold fewer than VEC elements (`lastlen` is the row length): that
 // item is moved element by element, with guards.  All of a thread's loads are issued before the first use.
 struct NdMixArgs {
-    int mode[kMaxOperands];          // [0] is the target: 1 vector stores, 2 element stores, 3 vector stores at element alignment
+    int mode[kMaxOperands];          // [0] is the target: 1 vector stores, 2 element stores
     int64_t estride[kMaxOperands];   // element stride along the last dimension
     uint32_t lastlen;                // elements per row
 };
@@ -303,9 +286,6 @@ __global__ __launch_bounds__(kBlock) void map_nd_mix_kernel(Op op, typename Op::
         Pack<X, VEC> v;
         if (mode == 1 && whole) return load_pack<X, VEC>(src + off);
         if (mode == 0) return splat_pack<X, VEC>(src[off]);
-        if constexpr (sizeof(X) >= 4 && sizeof(X) * VEC == 16) {
-            if (mode == 3 && whole) return load_pack_unaligned<X, VEC>(src + off);
-        }
         const int64_t step = mode == 2 ? es : 1;
 #pragma unroll
         for (int e = 0; e < VEC; e++) v.v[e] = src[off + ((uint32_t)e < left ? e * step : 0)];
@@ -322,8 +302,6 @@ __global__ __launch_bounds__(kBlock) void map_nd_mix_kernel(Op op, typename Op::
     for (int e = 0; e < VEC; e++) r.v[e] = apply_op(op, va.v[e], vb.v[e], vc.v[e]);
     if (m.mode[0] == 1 && whole) {
         store_pack<T, VEC>(t + ot, r);
-    } else if (sizeof(T) >= 4 && sizeof(T) * VEC == 16 && m.mode[0] == 3 && whole) {
-        if constexpr (sizeof(T) >= 4 && sizeof(T) * VEC == 16) store_pack_unaligned<T, VEC>(t + ot, r);
     } else {
 #pragma unroll
         for (int e = 0; e < VEC; e++)
@@ -696,6 +674,11 @@ constexpr int op_vec() {
 }
 
 inline bool aligned_to(const void* p, size_t a) { return ((uintptr_t)p % a) == 0; }
+// an operand of `esize`-byte elements can be moved in vectors of `vec` elements from `p` on: any address for elements of 4 bytes
+// and more (PackWord), the vector's own alignment for narrower ones
+inline bool vector_address(const void* p, int vec, size_t esize) { return esize >= 4 || aligned_to(p, vec * esize); }
+// ... and a row pitch or outer stride of `stride` elements keeps every row's vectors addressable
+inline bool vector_stride(int64_t stride, int vec, size_t esize) { return esize >= 4 || (stride % vec) == 0; }
 
 constexpr uint32_t kMaxItems = 0xFFFF0000u;
 
@@ -724,9 +707,9 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
         for (int k = 1; k < NOPS; k++) flat = flat && (p.stride[k][0] == 1 || p.stride[k][0] == 0);
     }
     if (flat && nd == 1) {
-        bool al = aligned_to(t, VEC * es[0]);
+        bool al = vector_address(t, VEC, es[0]);
         for (int k = 1; k < NOPS; k++)
-            if (p.stride[k][0] == 1) al = al && aligned_to(p.ptr[k], VEC * es[k]);
+            if (p.stride[k][0] == 1) al = al && vector_address(p.ptr[k], VEC, es[k]);
         if (al) {
             // one 16-byte vector per thread: measured fastest on MI355X (more per-thread unrolling lowers achieved bandwidth; for
             // narrowing ops such as int32 -> bool compares, four consecutive loads per thread to reach a 16-byte store measured
@@ -798,12 +781,12 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 if (q.staged[k]) { nstaged++; staged_esize = es[k]; }
             }
             // vector path: every tile row a whole number of aligned vectors for the target and every staged source
-            bool vec = VEC > 1 && (q.na % VEC) == 0 && (q.nb % VEC) == 0 && aligned_to(t, VEC * es[0]) && (q.sa[0] % VEC) == 0;
-            for (int d = 0; d < q.nouter && vec; d++) vec = (q.ostride[0][d] % VEC) == 0;
+            bool vec = VEC > 1 && (q.na % VEC) == 0 && (q.nb % VEC) == 0 && vector_address(t, VEC, es[0]) && vector_stride(q.sa[0], VEC, es[0]);
+            for (int d = 0; d < q.nouter && vec; d++) vec = vector_stride(q.ostride[0][d], VEC, es[0]);
             for (int k = 1; k < NOPS && vec; k++) {
                 if (!q.staged[k]) continue;
-                vec = aligned_to(p.ptr[k], VEC * es[k]) && (q.sb[k] % VEC) == 0;
-                for (int d = 0; d < q.nouter && vec; d++) vec = (q.ostride[k][d] % VEC) == 0;
+                vec = vector_address(p.ptr[k], VEC, es[k]) && vector_stride(q.sb[k], VEC, es[k]);
+                for (int d = 0; d < q.nouter && vec; d++) vec = vector_stride(q.ostride[k][d], VEC, es[k]);
             }
             // sources that are not staged: all broadcast along B, or each broadcast or in aligned vectors along B, lets the kernel fetch
             // them without branches
@@ -812,8 +795,8 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 if (q.staged[k] || q.sb[k] == 0) continue;
                 if (q.dmode == 1) q.dmode = 2;
                 if (!vec) continue;   // the element-wise kernel fetches single elements either way
-                bool ok = q.sb[k] == 1 && aligned_to(p.ptr[k], VEC * es[k]) && (q.sa[k] % VEC) == 0;
-                for (int d = 0; d < q.nouter && ok; d++) ok = (q.ostride[k][d] % VEC) == 0;
+                bool ok = q.sb[k] == 1 && vector_address(p.ptr[k], VEC, es[k]) && vector_stride(q.sa[k], VEC, es[k]);
+                for (int d = 0; d < q.nouter && ok; d++) ok = vector_stride(q.ostride[k][d], VEC, es[k]);
                 if (!ok) q.dmode = 0;
             }
             // Large tiles (128 KB of LDS, one workgroup per CU) for 4- and 8-byte elements in whole tiles with one staged source:
@@ -935,14 +918,14 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
         q.shape[d] = (uint32_t)p.shape[d];
         for (int k = 0; k < NOPS; k++) q.stride[k][d] = p.stride[k][d];
     }
-    bool vec = VEC > 1 && nd >= 1 && p.stride[0][last] == 1 && (p.shape[last] % VEC) == 0 && aligned_to(t, VEC * es[0]);
+    bool vec = VEC > 1 && nd >= 1 && p.stride[0][last] == 1 && (p.shape[last] % VEC) == 0 && vector_address(t, VEC, es[0]);
     for (int k = 1; k < NOPS && vec; k++) {
         vec = vec && (p.stride[k][last] == 0 || p.stride[k][last] == 1);
-        if (p.stride[k][last] == 1) vec = vec && aligned_to(p.ptr[k], VEC * es[k]);
+        if (p.stride[k][last] == 1) vec = vec && vector_address(p.ptr[k], VEC, es[k]);
     }
     for (int d = 0; d < last && vec; d++)
         for (int k = 0; k < NOPS; k++)
-            if (p.stride[k][last] == 1) vec = vec && (p.stride[k][d] % VEC) == 0;
+            if (p.stride[k][last] == 1) vec = vec && vector_stride(p.stride[k][d], VEC, es[k]);
     // the target runs along the last dimension but something else keeps the vector form away: per-operand access modes
     if constexpr (VEC > 1) {
         if (!vec && nd >= 1 && p.stride[0][last] == 1 && p.shape[last] >= 4 * VEC) {
@@ -950,9 +933,9 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
             memset(&mx, 0, sizeof(mx));
             const int64_t L = p.shape[last];
             for (int k = 0; k < NOPS; k++) {
-                bool whole_vectors = p.stride[k][last] == 1 && aligned_to(p.ptr[k], VEC * es[k]);
-                for (int d = 0; d < last && whole_vectors; d++) whole_vectors = (p.stride[k][d] % VEC) == 0;
-                mx.mode[k] = (k > 0 && p.stride[k][last] == 0) ? 0 : whole_vectors ? 1 : (p.stride[k][last] == 1 && es[k] >= 4 && es[k] * VEC == 16) ? 3 : 2;
+                bool whole_vectors = p.stride[k][last] == 1 && vector_address(p.ptr[k], VEC, es[k]);
+                for (int d = 0; d < last && whole_vectors; d++) whole_vectors = vector_stride(p.stride[k][d], VEC, es[k]);
+                mx.mode[k] = (k > 0 && p.stride[k][last] == 0) ? 0 : whole_vectors ? 1 : 2;
                 mx.estride[k] = p.stride[k][last];
                 q.stride[k][last] = p.stride[k][last] * VEC;
             }

@@ -213,6 +213,19 @@ def test_misaligned_ragged_and_strided_rows(H, G, rng, dt):
     tc, td = G.ofNumpy(c), G.ofNumpy(d)
     assert_exact(c[:, :, 1] - d, G.toNumpy(tc[:, :, 1] - td))
     assert_exact(d[:, ::-1] - c[:, :, 2], G.toNumpy(td.reverseAxis(1) - tc[:, :, 2]))
+    # transposing calls on views that start at odd elements and have odd row pitches (whole vectors per row all the same)
+    m = rand(rng, dt, (200, 301))
+    n = rand(rng, dt, (260, 131))
+    tm, tn = G.ofNumpy(m), G.ofNumpy(n)
+    sm, sn = m[1:129, 3:259], n[2:258, 1:129]
+    assert_exact(np.ascontiguousarray(sm.T), G.toNumpy(tm[1:129, 3:259].T.Copy()))
+    assert_exact(sm.T - sn, G.toNumpy(tm[1:129, 3:259].T - tn[2:258, 1:129]))
+    assert_exact(sn - sm.T, G.toNumpy(tn[2:258, 1:129] - tm[1:129, 3:259].T))
+    outv = G.zeros([260, 131], dt)
+    outv[2:258, 1:129].FillSubtract(tm[1:129, 3:259].T, tn[2:258, 1:129])
+    wantv = np.zeros_like(n)
+    wantv[2:258, 1:129] = sm.T - sn
+    assert_exact(wantv, G.toNumpy(outv))
     # the oracle device on the same views
     ref, got = both(H, G, lambda a, b: (a[:, 1:] - b[:, :1030], a[2:, 5:] + b[:35, :1026]), x, y)
     assert_exact(ref[0], got[0])
