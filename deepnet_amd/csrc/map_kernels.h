@@ -414,20 +414,44 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
     // outside an edge tile fetch element (0, 0) of the tile instead, and what they put into LDS is never read).
     {
         const uint32_t sx = (threadIdx.x % TVA) * VEC, sy = threadIdx.x / TVA;
-        const uint32_t sxc = sx < la_n ? sx : 0u;
+        const uint32_t sxc = sx + VEC <= la_n ? sx : 0u;
+        // (a row of the tensor that is not a whole number of vectors ends inside one thread column's vector: those threads fetch
+        // column 0 with the others and then their own elements one by one)
+        const bool part_a = VEC > 1 && sx < la_n && sx + VEC > la_n;
         Pack<A, VEC> ga[ITER_S];
         Pack<B, VEC> gb[ITER_S];
         Pack<C, VEC> gc[ITER_S];
+        if (la_n >= (uint32_t)VEC) {   // (a tile narrower than one vector has no whole vector to fetch: elements only, below)
 #pragma unroll
-        for (int it = 0; it < ITER_S; it++) {
-            const uint32_t r = sy + it * ROWS_S;
-            const int64_t rc = r < lb_n ? (int64_t)r : 0;
-            if constexpr (Op::NSRC >= 1)
-                if constexpr (S1) ga[it] = load_pack<A, VEC>(a + rc * p.sb[1] + sxc);
-            if constexpr (Op::NSRC >= 2)
-                if constexpr (S2) gb[it] = load_pack<B, VEC>(b + rc * p.sb[2] + sxc);
-            if constexpr (Op::NSRC >= 3)
-                if constexpr (S3) gc[it] = load_pack<C, VEC>(c + rc * p.sb[3] + sxc);
+            for (int it = 0; it < ITER_S; it++) {
+                const uint32_t r = sy + it * ROWS_S;
+                const int64_t rc = r < lb_n ? (int64_t)r : 0;
+                if constexpr (Op::NSRC >= 1)
+                    if constexpr (S1) ga[it] = load_pack<A, VEC>(a + rc * p.sb[1] + sxc);
+                if constexpr (Op::NSRC >= 2)
+                    if constexpr (S2) gb[it] = load_pack<B, VEC>(b + rc * p.sb[2] + sxc);
+                if constexpr (Op::NSRC >= 3)
+                    if constexpr (S3) gc[it] = load_pack<C, VEC>(c + rc * p.sb[3] + sxc);
+            }
+        }
+        if constexpr (VEC > 1) {
+            if (part_a) {
+#pragma unroll
+                for (int it = 0; it < ITER_S; it++) {
+                    const uint32_t r = sy + it * ROWS_S;
+                    const int64_t rc = r < lb_n ? (int64_t)r : 0;
+#pragma unroll
+                    for (int e = 0; e < VEC - 1; e++) {
+                        const uint32_t col = sx + e < la_n ? sx + e : 0u;
+                        if constexpr (Op::NSRC >= 1)
+                            if constexpr (S1) ga[it].v[e] = a[rc * p.sb[1] + col];
+                        if constexpr (Op::NSRC >= 2)
+                            if constexpr (S2) gb[it].v[e] = b[rc * p.sb[2] + col];
+                        if constexpr (Op::NSRC >= 3)
+                            if constexpr (S3) gc[it].v[e] = c[rc * p.sb[3] + col];
+                    }
+                }
+            }
         }
 #pragma unroll
         for (int it = 0; it < ITER_S; it++) {
@@ -475,6 +499,13 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
     auto store_phase = [&](auto mode_tag, auto full_tag) {
         constexpr int MODE = decltype(mode_tag)::value;    // as TrArgs::dmode
         constexpr bool FULL = decltype(full_tag)::value;
+        [[maybe_unused]] const bool whole_b = tx + VEC <= lb_n;   // this thread's vector lies inside the row
+        // Rows beyond an edge tile's extent repeat its last row: they fetch what that row fetches and store what it stores (the same
+        // values to the same addresses), so that no store of the loop sits behind a test.
+        auto row_of = [&](int i) {
+            const uint32_t r0 = ty + (uint32_t)i * ROWS_T;
+            return FULL ? r0 : (r0 < la_n ? r0 : la_n - 1u);
+        };
 #pragma unroll 1
         for (int g0 = 0; g0 < ITER_T; g0 += G) {
             Pack<A, VEC> da[G];
@@ -483,23 +514,38 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
             if constexpr (MODE != 1) {
 #pragma unroll
                 for (int i = 0; i < G; i++) {
-                    const uint32_t r = ty + (g0 + i) * ROWS_T;
+                    const uint32_t r = row_of(g0 + i);
                     if constexpr (MODE == 2) {
-                        const uint32_t rc = (FULL || r < la_n) ? r : 0u;   // rows outside an edge tile fetch row 0, nothing of them is stored
-                        if constexpr (Op::NSRC >= 1 && !S1) da[i] = tr_direct_fast<A, VEC>(a, rc, tx, p.sa[1], p.sb[1]);
-                        if constexpr (Op::NSRC >= 2 && !S2) db[i] = tr_direct_fast<B, VEC>(b, rc, tx, p.sa[2], p.sb[2]);
-                        if constexpr (Op::NSRC >= 3 && !S3) dc[i] = tr_direct_fast<C, VEC>(c, rc, tx, p.sa[3], p.sb[3]);
-                    } else if (r < la_n) {
+                        const uint32_t rc = r;
+                        const uint32_t txc = (FULL || whole_b) ? tx : 0u;  // a vector that would cross the row's end fetches column 0
+                        if (FULL || lb_n >= (uint32_t)VEC) {   // (as in the staging: no whole vector in a tile narrower than one)
+                            if constexpr (Op::NSRC >= 1 && !S1) da[i] = tr_direct_fast<A, VEC>(a, rc, txc, p.sa[1], p.sb[1]);
+                            if constexpr (Op::NSRC >= 2 && !S2) db[i] = tr_direct_fast<B, VEC>(b, rc, txc, p.sa[2], p.sb[2]);
+                            if constexpr (Op::NSRC >= 3 && !S3) dc[i] = tr_direct_fast<C, VEC>(c, rc, txc, p.sa[3], p.sb[3]);
+                        }
+                    } else if (FULL || whole_b) {
                         if constexpr (Op::NSRC >= 1 && !S1) da[i] = tr_direct<A, VEC>(a, r, tx, p.sa[1], p.sb[1]);
                         if constexpr (Op::NSRC >= 2 && !S2) db[i] = tr_direct<B, VEC>(b, r, tx, p.sa[2], p.sb[2]);
                         if constexpr (Op::NSRC >= 3 && !S3) dc[i] = tr_direct<C, VEC>(c, r, tx, p.sa[3], p.sb[3]);
+                    }
+                    if constexpr (!FULL && VEC > 1) {
+                        // the elements of a vector that crosses the row's end, one by one
+                        if (!whole_b) {
+#pragma unroll
+                            for (int e = 0; e < VEC - 1; e++) {
+                                const uint32_t col = tx + e < lb_n ? tx + e : tx;
+                                if constexpr (Op::NSRC >= 1 && !S1) da[i].v[e] = a[(int64_t)r * p.sa[1] + (int64_t)col * p.sb[1]];
+                                if constexpr (Op::NSRC >= 2 && !S2) db[i].v[e] = b[(int64_t)r * p.sa[2] + (int64_t)col * p.sb[2]];
+                                if constexpr (Op::NSRC >= 3 && !S3) dc[i].v[e] = c[(int64_t)r * p.sa[3] + (int64_t)col * p.sb[3]];
+                            }
+                        }
                     }
                 }
             }
 #pragma unroll
             for (int i = 0; i < G; i++) {
-                const uint32_t r = ty + (g0 + i) * ROWS_T;
-                if (FULL || r < la_n) {
+                const uint32_t r = row_of(g0 + i);
+                {
                     Pack<T, VEC> res;
 #pragma unroll
                     for (int e = 0; e < VEC; e++) {
@@ -511,7 +557,13 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
                         if constexpr (Op::NSRC >= 3) xc = S3 ? lc[tx + e][r] : (MODE == 1 ? pc[g0 + i] : dc[i].v[e]);
                         res.v[e] = apply_op(op, xa, xb, xc);
                     }
-                    store_pack<T, VEC>(t + (int64_t)r * p.sa[0] + tx, res);
+                    if (FULL || whole_b) {
+                        store_pack<T, VEC>(t + (int64_t)r * p.sa[0] + tx, res);
+                    } else {
+#pragma unroll
+                        for (int e = 0; e < VEC - 1; e++)
+                            if (tx + e < lb_n) t[(int64_t)r * p.sa[0] + tx + e] = res.v[e];
+                    }
                 }
             }
         }
@@ -528,7 +580,10 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
     } else {
         if (full && p.dmode == 1) store_phase(M1{}, std::true_type{});
         else if (full && p.dmode == 2) store_phase(M2{}, std::true_type{});
-        else if (tx < lb_n) store_phase(M0{}, std::false_type{});
+        else if (tx < lb_n) {
+            if (p.dmode == 2) store_phase(M2{}, std::false_type{});
+            else store_phase(M0{}, std::false_type{});
+        }
     }
 }
 
@@ -539,8 +594,12 @@ __global__ __launch_bounds__(kBlock) void map_tr_kernel(Op op, typename Op::T* t
 // b's, group g of row a stored at g ^ ((a / 4) % 8); consecutive lanes (a four apart) then fall into different groups, and a storing
 // thread fetches its four b's of row a with one 16-byte read, consecutive lanes again in different groups.
 // One staged source (MASK 1 or 2); for two-operand ops the other source is read in the store pattern, MODE 1 (broadcast along B:
-// one value per stored row, fetched ahead of the barrier) or MODE 2 (broadcast or in aligned vectors along B).
-template <class Op, int TA, int TB, int MASK>
+// one value per stored row, fetched ahead of the barrier) or MODE 2 (broadcast or in vectors along B).
+// GEN = false: whole tiles.  GEN = true: tiles on the tensor's edge, target rows that are not whole vectors, a second operand with
+// any strides (the staged source's rows still are whole vectors).  What it is for: short target rows of any length (250 elements,
+// say) that follow one another in memory, where one workgroup writes its 256 rows as one contiguous run; cut into the 128 x 64
+// tiles of map_tr_kernel the same rows are written as 256-byte pieces that start and end inside cache lines, at half the speed.
+template <class Op, int TA, int TB, int MASK, bool GEN>
 __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* t, const typename Op::A* a, const typename Op::B* b,
                                                          TrArgs p, uint32_t xcd_chunk) {
     using T = typename Op::T;
@@ -588,6 +647,10 @@ __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* 
     t += ot;
     sp += os;
     dp += od;
+    // GEN: valid extent of this tile along A and B.  Positions outside it fetch what a position inside fetches, and what they put
+    // into LDS is never stored.  (The staged source's rows are whole vectors, so la_n is a multiple of VEC.)
+    const uint32_t la_n = GEN ? (uint32_t)min((int64_t)TA, (int64_t)p.na - a0) : (uint32_t)TA;
+    const uint32_t lb_n = GEN ? (uint32_t)min((int64_t)TB, (int64_t)p.nb - b0) : (uint32_t)TB;
 
     const uint32_t gl = threadIdx.x % TVB, tx = gl * VEC, ty = threadIdx.x / TVB;
     const bool rows_only = p.dmode == 1;
@@ -597,7 +660,11 @@ __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* 
 #pragma unroll
         for (int jt = 0; jt < JT; jt++)
 #pragma unroll
-            for (int k = 0; k < VEC; k++) g[jt][k] = load_pack<S, VEC>(sp + (int64_t)(VEC * (RS * jt + sy) + k) * p.sb[KS] + VEC * lx);
+            for (int k = 0; k < VEC; k++) {
+                const uint32_t rb = VEC * (RS * jt + sy) + k;
+                const uint32_t rbc = (!GEN || rb < lb_n) ? rb : 0u, ac = (!GEN || VEC * lx < la_n) ? VEC * lx : 0u;
+                g[jt][k] = load_pack<S, VEC>(sp + (int64_t)rbc * p.sb[KS] + ac);
+            }
         // a source with one value per stored row: the tile's TA values go through LDS (one load per thread here, behind the staging
         // loads and ahead of the wait for them; fetched by every storing thread for its own rows they cost as many load
         // instructions as the tile itself)
@@ -605,7 +672,10 @@ __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* 
         if constexpr (HAS_D) {
             if (rows_only) {
 #pragma unroll
-                for (int q = 0; q < NDV; q++) dv[q] = dp[(int64_t)((threadIdx.x + q * kBlock) % TA) * p.sa[KD]];
+                for (int q = 0; q < NDV; q++) {
+                    const uint32_t ia = (threadIdx.x + q * kBlock) % TA;
+                    dv[q] = dp[(int64_t)((!GEN || ia < la_n) ? ia : 0u) * p.sa[KD]];
+                }
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -628,23 +698,45 @@ __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* 
         }
     }
     __syncthreads();
+    // the row of this thread's i-th pass; GEN: rows beyond the tile's extent repeat its last row
+    auto row_of = [&](int i) {
+        const uint32_t r0 = ty + (uint32_t)i * RT;
+        return !GEN ? r0 : (r0 < la_n ? r0 : la_n - 1u);
+    };
     [[maybe_unused]] D pd[ITER_T];
     if constexpr (HAS_D) {
         if (rows_only) {
 #pragma unroll
-            for (int it = 0; it < ITER_T; it++) pd[it] = lv[ty + it * RT];
+            for (int it = 0; it < ITER_T; it++) pd[it] = lv[row_of(it)];
         }
     }
+    // MODE 1: the other source has one value per stored row (or there is none); MODE 2: it is broadcast or runs in vectors along B;
+    // MODE 0 (GEN only): any strides, fetched element by element.  GEN: rows beyond the tile's extent repeat its last row (the same
+    // values to the same addresses, so that no store sits behind a test); a vector that crosses the end of the target's row is
+    // moved element by element, vectors beyond it are skipped.
     auto store_tile = [&](auto mode_tag) {
         constexpr int MODE = decltype(mode_tag)::value;
+        const uint32_t cnt = !GEN ? (uint32_t)VEC : lb_n > tx ? min((uint32_t)VEC, lb_n - tx) : 0u;   // elements of this thread's vector inside the tile
+        if (GEN && cnt == 0u) return;
+        const bool whole = !GEN || cnt == (uint32_t)VEC;
         [[maybe_unused]] Pack<D, VEC> dd[ITER_T];
         if constexpr (HAS_D && MODE == 2) {
 #pragma unroll
-            for (int i = 0; i < ITER_T; i++) dd[i] = tr_direct_fast<D, VEC>(dp, ty + i * RT, tx, p.sa[KD], p.sb[KD]);
+            for (int i = 0; i < ITER_T; i++) dd[i] = tr_direct_fast<D, VEC>(dp, row_of(i), whole ? tx : 0u, p.sa[KD], p.sb[KD]);
+        }
+        if constexpr (HAS_D && GEN && MODE != 1) {
+            if (MODE == 0 || !whole) {
+#pragma unroll
+                for (int i = 0; i < ITER_T; i++) {
+                    const int64_t ro = (int64_t)row_of(i) * p.sa[KD];
+#pragma unroll
+                    for (int e = 0; e < VEC; e++) dd[i].v[e] = dp[ro + (int64_t)((uint32_t)e < cnt ? tx + e : tx) * p.sb[KD]];
+                }
+            }
         }
 #pragma unroll
         for (int i = 0; i < ITER_T; i++) {
-            const uint32_t r = ty + i * RT;
+            const uint32_t r = row_of(i);
             const Group w = __builtin_bit_cast(Group, l[r * TVB + (gl ^ ((r / (uint32_t)VEC) % 8u))]);
             Pack<T, VEC> res;
 #pragma unroll
@@ -655,9 +747,21 @@ __global__ __launch_bounds__(kBlock) void map_tr4_kernel(Op op, typename Op::T* 
                 if constexpr (S1) res.v[e] = apply_op(op, xs, xd, C());
                 else res.v[e] = apply_op(op, xd, xs, C());
             }
-            store_pack<T, VEC>(t + (int64_t)r * p.sa[0] + tx, res);
+            if (whole) {
+                store_pack<T, VEC>(t + (int64_t)r * p.sa[0] + tx, res);
+            } else {
+#pragma unroll
+                for (int e = 0; e < VEC - 1; e++)
+                    if ((uint32_t)e < cnt) t[(int64_t)r * p.sa[0] + tx + e] = res.v[e];
+            }
         }
     };
+    if constexpr (GEN && HAS_D) {
+        if (p.dmode == 0) {
+            store_tile(std::integral_constant<int, 0>{});
+            return;
+        }
+    }
     if (!HAS_D || rows_only) store_tile(std::integral_constant<int, 1>{});
     else store_tile(std::integral_constant<int, 2>{});
 }
@@ -781,7 +885,8 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 if (q.staged[k]) { nstaged++; staged_esize = es[k]; }
             }
             // vector path: every tile row a whole number of aligned vectors for the target and every staged source
-            bool vec = VEC > 1 && (q.na % VEC) == 0 && (q.nb % VEC) == 0 && vector_address(t, VEC, es[0]) && vector_stride(q.sa[0], VEC, es[0]);
+            // (rows that are not whole vectors end inside one vector of an edge tile: the kernel moves that one element by element)
+            bool vec = VEC > 1 && vector_address(t, VEC, es[0]) && vector_stride(q.sa[0], VEC, es[0]);
             for (int d = 0; d < q.nouter && vec; d++) vec = vector_stride(q.ostride[0][d], VEC, es[0]);
             for (int k = 1; k < NOPS && vec; k++) {
                 if (!q.staged[k]) continue;
@@ -808,7 +913,7 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
             //   8-byte elements (512 MiB copies, 64 x 32 tiles of map_tr_kernel before): 8192 x 8192 244 -> 181 us, 4096 x 16384 245 -> 182,
             //   16384 x 4096 216 -> 195, 1024 x 65536 198 -> 174, 64 x [1024 x 1024] 197 -> 164, [256, 512, 512] permuted to [512, 512, 256]
             //   185 -> 173; 64 x 256, 256 x 64 and 32 x 512 tiles measured no better than 128 x 128 over these layouts.
-            bool big = false, tall = false, tr4 = false;
+            bool big = false, tall = false, tr4 = false, tr4_gen = false;
             constexpr int TALL_TA = 128, TALL_TB = WIDE ? 128 : 256;
             if constexpr (VEC == 16 / ESZ && Op::NSRC >= 1 && Op::NSRC <= 2) {
                 static const bool tr4_on = [] { const char* e = getenv("DNH_TR4"); return !e || e[0] != '0'; }();
@@ -820,6 +925,14 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                        q.sa[0] * (int64_t)es[0] < 256 * 1024 &&
                        (int64_t)(q.na / TALL_TA) * (q.nb / TALL_TB) * outer >= (int64_t)device_cus() * 8;
                 tr4 = tr4_ok && (big || tall);
+                // short rows that are ragged in any way (extents that are not multiples of the tile, rows that are not whole vectors,
+                // a second operand with other strides): the kernel's general form on the 256-row tiles, whose rows follow one another
+                // in a contiguous target ([250, 500, 1000] permuted to [500, 1000, 250]: 128 x 64 tiles 337 us)
+                if (!tr4 && tr4_on && one4 && q.nb <= 256 && (q.na % VEC) == 0 &&
+                    (int64_t)cdiv(q.na, BIG_TA) * cdiv(q.nb, BIG_TB) * outer >= (int64_t)device_cus() * 8) {
+                    tr4 = tr4_gen = big = true;
+                    tall = false;
+                }
             }
             const int ta_n = big ? BIG_TA : tall ? TALL_TA : TA, tb_n = big ? BIG_TB : tall ? TALL_TB : TB;
             q.tiles_a = cdiv(q.na, ta_n);
@@ -866,9 +979,9 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
             }                                                                                            \
         }                                                                                                \
     } while (0)
-#define DNH_TR4_LAUNCH(TA_, TB_, M_)                                                                                                      \
+#define DNH_TR4_LAUNCH(TA_, TB_, M_, G_)                                                                                                  \
     do {                                                                                                                                  \
-        auto kern = map_tr4_kernel<Op, TA_, TB_, M_>;                                                                                     \
+        auto kern = map_tr4_kernel<Op, TA_, TB_, M_, G_>;                                                                                   \
         static const hipError_t attr = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, TA_ * TB_ * ESZ + TA_ * 8); \
         if (attr != hipSuccess) { st = fail(DNH_ERR_HIP, "hipFuncSetAttribute: %s", hipGetErrorString(attr)); break; }                    \
         hipLaunchKernelGGL(kern, dim3((unsigned)blocks), dim3(kBlock), (size_t)TA_ * TB_ * ESZ + TA_ * 8, stream, op, t, a, b, q, xcd_chunk);                    \
@@ -877,16 +990,17 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
                 if (tr4) {
                     if constexpr (VEC == 16 / ESZ && Op::NSRC >= 1 && Op::NSRC <= 2) {
                         // (the staged source is the one of four bytes: `staged_esize` above)
-#define DNH_TR4_PICK(TA_, TB_)                                                                           \
+#define DNH_TR4_PICK(TA_, TB_, G_)                                                                       \
     do {                                                                                                 \
         if (mask == 1) {                                                                                 \
-            if constexpr (sizeof(A) == ESZ) DNH_TR4_LAUNCH(TA_, TB_, 1);                                   \
+            if constexpr (sizeof(A) == ESZ) DNH_TR4_LAUNCH(TA_, TB_, 1, G_);                             \
         } else if constexpr (Op::NSRC == 2) {                                                            \
-            if constexpr (sizeof(B) == ESZ) DNH_TR4_LAUNCH(TA_, TB_, 2);                                   \
+            if constexpr (sizeof(B) == ESZ) DNH_TR4_LAUNCH(TA_, TB_, 2, G_);                             \
         }                                                                                                \
     } while (0)
-                        if (big) DNH_TR4_PICK(BIG_TA, BIG_TB);
-                        else DNH_TR4_PICK(TALL_TA, TALL_TB);
+                        if (tr4_gen) DNH_TR4_PICK(BIG_TA, BIG_TB, true);
+                        else if (big) DNH_TR4_PICK(BIG_TA, BIG_TB, false);
+                        else DNH_TR4_PICK(TALL_TA, TALL_TB, false);
 #undef DNH_TR4_PICK
                     }
                 } else if (big) {
