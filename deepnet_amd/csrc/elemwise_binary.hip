@@ -43,12 +43,9 @@ extern "C" int32_t dnh_binary(int32_t op, const DnhTensor* t, const DnhTensor* a
     switch (op) {
         case DNH_ADD: return run_numeric<OpAdd>(dt, p, s);
         case DNH_SUBTRACT: return run_numeric<OpSub>(dt, p, s);
-        case DNH_MULTIPLY: return run_numeric<OpMul>(dt, p, s);
-        case DNH_DIVIDE: case DNH_MODULO: case DNH_MAX_ELEMWISE: case DNH_MIN_ELEMWISE: return binary_second_unit(op, dt, p, s);
-        case DNH_POWER:
-            if (dt == DNH_F32) return launch_map(OpPow<float>{}, p, s);
-            if (dt == DNH_F64) return launch_map(OpPow<double>{}, p, s);
-            return fail(DNH_ERR_NOT_SUPPORTED, "Power is defined for single and double only, not %s", dtype_name(dt));
+        case DNH_MULTIPLY: case DNH_POWER: return binary_fourth_unit(op, dt, p, s);
+        case DNH_DIVIDE: case DNH_MODULO: return binary_second_unit(op, dt, p, s);
+        case DNH_MAX_ELEMWISE: case DNH_MIN_ELEMWISE: return binary_third_unit(op, dt, p, s);
     }
     return fail(DNH_ERR_INVALID_ARG, "dnh_binary: unknown op %d", op);
 }

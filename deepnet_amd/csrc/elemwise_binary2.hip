@@ -1,4 +1,4 @@
-// The second half of dnh_binary's ops: ITensorBackend Divide, Modulo, MaxElemwise, MinElemwise (Tensor/Tensor/TensorBackend.fs:100-104).
+// More of dnh_binary's ops: ITensorBackend Divide, Modulo (Tensor/Tensor/TensorBackend.fs:100-101).
 #include "map_kernels.h"
 #include "ops.h"
 
@@ -29,8 +29,6 @@ int32_t dnh::binary_second_unit(int32_t op, int dt, const MapPlan& p, hipStream_
     switch (op) {
         case DNH_DIVIDE: return run_numeric<OpDiv>(dt, p, s);
         case DNH_MODULO: return run_numeric<OpMod>(dt, p, s);
-        case DNH_MAX_ELEMWISE: return run_numeric<OpMax>(dt, p, s);
-        case DNH_MIN_ELEMWISE: return run_numeric<OpMin>(dt, p, s);
     }
     return fail(DNH_ERR_INVALID_ARG, "dnh_binary: unknown op %d", op);
 }

@@ -1086,9 +1086,11 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
     return DNH_OK;
 }
 
-// The arithmetic and comparison entry points are spread over two translation units each (the element-wise instantiations dominate
+// The arithmetic and comparison entry points are spread over four and two translation units (the element-wise instantiations dominate
 // the library's build time, and the units compile side by side); these take the ops of the second unit.
-int32_t binary_second_unit(int32_t op, int dt, const MapPlan& p, hipStream_t s);    // Divide, Modulo, MaxElemwise, MinElemwise
+int32_t binary_second_unit(int32_t op, int dt, const MapPlan& p, hipStream_t s);    // Divide, Modulo
+int32_t binary_third_unit(int32_t op, int dt, const MapPlan& p, hipStream_t s);     // MaxElemwise, MinElemwise
+int32_t binary_fourth_unit(int32_t op, int dt, const MapPlan& p, hipStream_t s);    // Multiply, Power
 int32_t compare_second_unit(int32_t op, int dt, const MapPlan& p, hipStream_t s);   // LessOrEqual, Greater, GreaterOrEqual
 
 }  // namespace dnh
