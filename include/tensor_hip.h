@@ -65,7 +65,9 @@ typedef enum DnhDType {
 /* Replaces the by-value kernel argument struct Tensor<T,N> (Cuda/Kernels/Tensor.cuh:7-16,
  * Cuda/NativeTensor.fs:96-112): one rank-agnostic, blittable descriptor. */
 typedef struct DnhTensor {
-    void*   base;                  /* device pointer to element 0 of the storage                 */
+    void*   base;                  /* device pointer to element 0 of the storage, aligned to the
+                                    * element size (no more is asked for: offsets, pitches and
+                                    * extents are free, odd ones included)                        */
     int64_t offset;                /* TensorLayout.Offset (elements)                             */
     int32_t ndims;                 /* 0..DNH_MAX_DIMS                                            */
     int32_t dtype;                 /* DnhDType                                                   */
