@@ -358,8 +358,9 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
 
     if (!(dc >= 0 && n >= 8) && n >= 16) {
         // rows
-        bool vec = VEC > 1 && sr == 1 && aligned_to(src, 16);
-        for (int d = 0; d < o.nd && vec; d++) vec = (o.sstride[d] % VEC) == 0;
+        // (vectors of 4- and 8-byte elements are fetched at element alignment, so shifted views and odd pitches keep them)
+        bool vec = VEC > 1 && sr == 1 && vector_address(src, VEC, sizeof(In));
+        for (int d = 0; d < o.nd && vec; d++) vec = vector_stride(o.sstride[d], VEC, sizeof(In));
         const int v = vec ? VEC : 1;
         // threads per row: at least four vectors per thread (measured on 16 Mi fp32: rows of 256-512 elements run 15-30 % faster
         // with 16 threads than with 64, rows of 1024-2048 fastest with 64, 4096 and longer with 256)
@@ -417,8 +418,8 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
             others *= o.shape[d];
             oo.nd++;
         }
-        bool vec = VEC > 1 && aligned_to(src, 16) && (nc % VEC) == 0 && (sr % VEC) == 0;
-        for (int d = 0; d < oo.nd && vec; d++) vec = (oo.sstride[d] % VEC) == 0;
+        bool vec = VEC > 1 && vector_address(src, VEC, sizeof(In)) && (nc % VEC) == 0 && vector_stride(sr, VEC, sizeof(In));
+        for (int d = 0; d < oo.nd && vec; d++) vec = vector_stride(oo.sstride[d], VEC, sizeof(In));
         const int v = vec ? VEC : 1;
         // Lanes along the kept dimension: the whole block when that still yields about four blocks per CU (4 KB contiguous per
         // row visit, no LDS step), else 64 lanes x 4 wavefronts sharing the reduced axis.  A block never takes fewer rows than

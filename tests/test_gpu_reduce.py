@@ -172,6 +172,26 @@ def _seq_fold(x, is_max):
     return out
 
 
+@pytest.mark.parametrize("dt", [np.float32, np.float64, np.int32, np.int64])
+def test_folds_of_shifted_views(G, rng, dt):
+    """Folds over views that start at odd elements and have odd row pitches (their rows are fetched in vectors at element
+    alignment): along both axes, row lengths with and without a vector tail; NumPy is the checker."""
+    x = (rng.standard_normal((1025, 4099)) * 100).astype(dt)
+    tx = G.ofNumpy(x)
+    for (r0, r1, c0, c1) in [(0, 1025, 3, 4099), (1, 1025, 1, 4098), (2, 1001, 5, 2054)]:
+        v, tv = x[r0:r1, c0:c1], tx[r0:r1, c0:c1]
+        for ax in (1, 0):
+            assert_exact(v.max(axis=ax), G.toNumpy(tv.maxAxis(ax)))
+            assert_exact(v.argmax(axis=ax).astype(np.int64), G.toNumpy(tv.argMaxAxis(ax)))
+            got = G.toNumpy(tv.sumAxis(ax))
+            if np.dtype(dt).kind == "f":
+                want = v.astype(np.float64).sum(axis=ax)
+                bound = (v.shape[ax] + 64) * (np.finfo(dt).eps / 2) * np.abs(v.astype(np.float64)).sum(axis=ax)
+                assert np.all(np.abs(got.astype(np.float64) - want) <= bound)
+            else:
+                assert_exact(v.sum(axis=ax, dtype=dt), got)
+
+
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 @pytest.mark.parametrize("shape", [(37, 300), (3, 70000), (600, 40), (1, 5), (2000, 16), (40, 2, 513)])
 def test_max_min_follow_the_sequential_rule_with_nans(H, G, rng, dt, shape):
