@@ -505,7 +505,7 @@ struct X3Stage {
             if constexpr (KC) {
                 // plain (temporal) 16-byte loads: the other half of each 128-byte line is wanted at the next K step and by the
                 // workgroups of the same tile row (load_pack's non-temporal loads measured 2.5-4 % slower at 4000^3 / 4096^3)
-                typedef float f32x4v __attribute__((ext_vector_type(4)));
+                typedef float f32x4v __attribute__((ext_vector_type(4), aligned(4)));   // any dword address (rows of views that start at odd elements)
                 const f32x4v v0 = *reinterpret_cast<const f32x4v*>(p0 + k0 + kofs), v1 = *reinterpret_cast<const f32x4v*>(p1 + k0 + kofs);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -1174,23 +1174,16 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
     bool x3 = false, big = false;
     bool a_kc = false, b_kc = false;
     if constexpr (sizeof(T) == 4) {
-        // each operand either k-contiguous with 16-byte aligned rows, or contiguous along its other dimension
-        a_kc = g.sak == 1 && (g.sam % 4) == 0 && aligned_to(a, 16);
-        b_kc = g.sbk == 1 && (g.sbn % 4) == 0 && aligned_to(b, 16);
-        for (int d = 0; d < g.nbatch; d++) {
-            a_kc = a_kc && (g.bsa[d] % 4) == 0;
-            b_kc = b_kc && (g.bsb[d] % 4) == 0;
-        }
+        // each operand either k-contiguous (its 16-byte fetches are declared at element alignment: any offset and pitch), or
+        // contiguous along its other dimension
+        a_kc = g.sak == 1;
+        b_kc = g.sbk == 1;
         x3 = g.K >= kX3BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_bf16x3();
     }
     bool f64p = false;   // double precision on gemm_f64_kernel: each operand contiguous along one of its dimensions
     if constexpr (sizeof(T) == 8) {
-        a_kc = g.sak == 1 && (g.sam % 2) == 0 && aligned_to(a, 16);
-        b_kc = g.sbk == 1 && (g.sbn % 2) == 0 && aligned_to(b, 16);
-        for (int d = 0; d < g.nbatch; d++) {
-            a_kc = a_kc && (g.bsa[d] % 2) == 0;
-            b_kc = b_kc && (g.bsb[d] % 2) == 0;
-        }
+        a_kc = g.sak == 1;
+        b_kc = g.sbk == 1;
         f64p = g.K >= kF64BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && !g.accumulate && use_f64_pinned();
     }
     int64_t want = 1;
@@ -1624,7 +1617,7 @@ struct I8Stage {
     __device__ __forceinline__ void load(int64_t k0, int64_t K, uint32_t (&r)[8]) const {
         if (!TAIL || k0 + kI8BK <= K) {
             if constexpr (KC) {
-                typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+                typedef uint32_t u32x4v __attribute__((ext_vector_type(4), aligned(4)));
                 const u32x4v v0 = *reinterpret_cast<const u32x4v*>(p0 + k0 + kofs), v1 = *reinterpret_cast<const u32x4v*>(p1 + k0 + kofs);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
@@ -1973,12 +1966,7 @@ template <class T>
 int32_t launch_gemm_int(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hipStream_t stream) {
     if constexpr (sizeof(T) == 4) {
         // each operand either k-contiguous with 16-byte aligned rows, or contiguous along its other dimension
-        bool a_kc = g.sak == 1 && (g.sam % 4) == 0 && aligned_to(a, 16);
-        bool b_kc = g.sbk == 1 && (g.sbn % 4) == 0 && aligned_to(b, 16);
-        for (int d = 0; d < g.nbatch; d++) {
-            a_kc = a_kc && (g.bsa[d] % 4) == 0;
-            b_kc = b_kc && (g.bsb[d] % 4) == 0;
-        }
+        bool a_kc = g.sak == 1, b_kc = g.sbk == 1;   // (k-contiguous rows are fetched at element alignment)
         if (g.K >= kI8BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && use_int_mfma()) {
             g.tiles_m = (uint32_t)cdiv(g.M, (int64_t)BM);
             g.tiles_n = (uint32_t)cdiv(g.N, (int64_t)BN);
@@ -2001,12 +1989,7 @@ int32_t launch_gemm_int(GemmArgs g, T* c, const T* a, const T* b, int64_t batch,
         }
     }
     if constexpr (sizeof(T) == 8) {
-        bool a_kc = g.sak == 1 && (g.sam % 2) == 0 && aligned_to(a, 16);
-        bool b_kc = g.sbk == 1 && (g.sbn % 2) == 0 && aligned_to(b, 16);
-        for (int d = 0; d < g.nbatch; d++) {
-            a_kc = a_kc && (g.bsa[d] % 2) == 0;
-            b_kc = b_kc && (g.bsb[d] % 2) == 0;
-        }
+        bool a_kc = g.sak == 1, b_kc = g.sbk == 1;
         if (g.K >= kI8BK && (a_kc || g.sam == 1) && (b_kc || g.sbn == 1) && use_int_mfma()) {
             g.tiles_m = (uint32_t)cdiv(g.M, (int64_t)kI64BM);
             g.tiles_n = (uint32_t)cdiv(g.N, (int64_t)kI64BN);

@@ -571,3 +571,43 @@ def test_dot_random_shapes_types_and_views(G, seed):
             with np.errstate(over="ignore"):
                 want = np.matmul(a, b)
             assert got.dtype == np.dtype(dt) and np.array_equal(got, want), what
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64, np.int32, np.int64])
+def test_dot_on_shifted_views_and_odd_pitches(G, dt):
+    """Operands that are views starting at odd elements, with odd row pitches (k-contiguous rows fetched at element alignment),
+    transposed and not, a K tail, a batch: integers bit for bit, floats within 16 u S (fp64: 2K + 64) of the fp64 product."""
+    rng = np.random.default_rng(77)
+    info = None if np.dtype(dt).kind == "f" else np.iinfo(dt)
+
+    def rand(shape):
+        if info is None:
+            return rng.standard_normal(shape).astype(dt)
+        return rng.integers(info.min, info.max, size=shape, dtype=dt, endpoint=True)
+
+    def check(a, b, got, what):
+        if info is None:
+            u = np.finfo(dt).eps / 2
+            exact = np.matmul(a.astype(np.float64), b.astype(np.float64))
+            S = np.matmul(np.abs(a).astype(np.float64), np.abs(b).astype(np.float64))
+            bound = (16 if dt == np.float32 else 2 * a.shape[-1] + 64) * u * S + np.finfo(dt).tiny
+            assert got.shape == exact.shape and np.all(np.abs(got - exact) <= bound), what
+        else:
+            with np.errstate(over="ignore"):
+                want = np.matmul(a, b)
+            assert np.array_equal(got, want), what
+
+    A = rand((517, 1003))
+    B = rand((1003, 391))
+    tA, tB = G.ofNumpy(A), G.ofNumpy(B)
+    # a[1:, 3:] (513 x 1000, pitch 1003) . b[3:, 1:] (1000 x 390, pitch 391)
+    check(A[1:, 3:], B[3:, 1:], G.toNumpy(tA[1:, 3:] @ tB[3:, 1:]), "row-major shifted")
+    # a K tail: 997 inner elements
+    check(A[2:, 5:1002], B[5:1002, 0:390], G.toNumpy(tA[2:, 5:1002] @ tB[5:1002, 0:390]), "K tail")
+    # transposed shifted views: (B[3:, 1:]).T (390 x 1000, k strided) . (A[1:, 3:]).T (1000 x 516)
+    check(B[3:, 1:].T, A[1:, 3:].T, G.toNumpy(tB[3:, 1:].T @ tA[1:, 3:].T), "transposed shifted")
+    # batched, odd pitches in every dimension
+    C3 = rand((3, 131, 259))
+    D3 = rand((3, 259, 67))
+    got = G.toNumpy(G.ofNumpy(C3)[:, 1:, 2:] @ G.ofNumpy(D3)[:, 2:, 1:])
+    check(C3[:, 1:, 2:], D3[:, 2:, 1:], got, "batched shifted")
