@@ -1442,7 +1442,8 @@ bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t strea
     T* partial = nullptr;
     WorkspaceLease lease;
     if (g.sak == 1 || g.M == 1) {
-        const bool vec = g.sak == 1 && g.sbk == 1 && (g.sam % V) == 0 && aligned_to(a, 16) && aligned_to(x, 16);
+        // (vectors of 4- and 8-byte elements are fetched at element alignment: any row pitch and start)
+        const bool vec = g.sak == 1 && g.sbk == 1 && vector_stride(g.sam, V, sizeof(T)) && vector_address(a, V, sizeof(T)) && vector_address(x, V, sizeof(T));
         const int v = vec ? V : 1;
         const int tpr = g.K >= (int64_t)256 * v * 2 ? 256 : (g.K >= (int64_t)64 * v ? 64 : 16);
         const int64_t row_blocks = (M + kBlock / tpr - 1) / (kBlock / tpr);
@@ -1467,7 +1468,7 @@ bool try_gemv(const GemmArgs& g, T* y, const T* a, const T* x, hipStream_t strea
 #undef DNH_GEMV
         if (splits > 1) hipLaunchKernelGGL(gemv_finish_kernel<T>, dim3(M), dim3(kBlock), 0, stream, y, (const T*)partial, M, splits, g.scm);
     } else if (g.sam == 1) {
-        const bool vec = (M % V) == 0 && (g.sak % V) == 0 && aligned_to(a, 16);
+        const bool vec = (M % V) == 0 && vector_stride(g.sak, V, sizeof(T)) && vector_address(a, V, sizeof(T));
         const int v = vec ? V : 1;
         const int64_t mblocks = (M / v + kBlock - 1) / kBlock;
         uint32_t splits = 1;

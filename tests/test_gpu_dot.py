@@ -606,6 +606,12 @@ def test_dot_on_shifted_views_and_odd_pitches(G, dt):
     check(A[2:, 5:1002], B[5:1002, 0:390], G.toNumpy(tA[2:, 5:1002] @ tB[5:1002, 0:390]), "K tail")
     # transposed shifted views: (B[3:, 1:]).T (390 x 1000, k strided) . (A[1:, 3:]).T (1000 x 516)
     check(B[3:, 1:].T, A[1:, 3:].T, G.toNumpy(tB[3:, 1:].T @ tA[1:, 3:].T), "transposed shifted")
+    # matrix . vector and vector . vector on shifted views (rows and the transposed, column-wise form)
+    x1 = rand((1003,))
+    tx1 = G.ofNumpy(x1)
+    check(A[1:, 3:], x1[3:], G.toNumpy(tA[1:, 3:] @ tx1[3:]), "matvec rows")
+    check(A[1:, 3:].T, x1[1:518][:516], G.toNumpy(tA[1:, 3:].T @ tx1[1:517]), "matvec columns")
+    check(x1[3:][None, :], x1[1:1001][:, None], np.asarray(G.toNumpy(tx1[3:] @ tx1[1:1001])).reshape(1, 1), "vecvec")
     # batched, odd pitches in every dimension
     C3 = rand((3, 131, 259))
     D3 = rand((3, 259, 67))
