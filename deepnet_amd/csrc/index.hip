@@ -846,7 +846,9 @@ bool try_compaction_fast(const MaskArgs& m, void* full, void* out, const Lay& ol
     if (olay.nd != 1 || olay.stride[0] != 1) return false;
     if (n > (int64_t)kMaxItems || n == 0 || nout == 0) return false;
     const int vec = 16 / esize;
-    if ((n % vec) != 0 || !aligned_to(full, 16) || !aligned_to(m.mask[0], 16)) return false;
+    // (the tensor's vectors of 4- and 8-byte elements are accessed at element alignment; the mask is read in 4-byte words by the
+    // counting pass and in words of `vec` bytes by the moving pass)
+    if ((n % vec) != 0 || !vector_address(full, vec, (size_t)esize) || !aligned_to(m.mask[0], (size_t)(vec < 4 ? 4 : vec))) return false;
     switch (esize) {
         case 1: *status = run_compaction_fast<uint8_t, SET>(m.mask[0], full, out, n, nout, stream); return true;
         case 2: *status = run_compaction_fast<uint16_t, SET>(m.mask[0], full, out, n, nout, stream); return true;

@@ -135,6 +135,22 @@ def test_masked_get_1d(H, G, rng, n):
     assert_exact(a[m], got)
 
 
+@pytest.mark.parametrize("dt", [np.int32, np.float64])
+@pytest.mark.parametrize("shift", [1, 2, 3])
+def test_masked_get_and_set_on_a_shifted_view(G, rng, dt, shift):
+    """The compaction's vector path on a tensor that starts at an odd element (the mask is a tensor of its own): NumPy is the checker."""
+    n = 40000
+    a = rng.integers(-1000, 1000, n + 8).astype(dt)
+    m = rng.random(n) < 0.4
+    ta, tm = G.ofNumpy(a), G.ofNumpy(m)
+    assert_exact(a[shift:shift + n][m], G.toNumpy(ta[shift:shift + n].M(tm)))
+    vals = rng.integers(-5, 5, int(m.sum())).astype(dt)
+    want = a.copy()
+    want[shift:shift + n][m] = vals
+    ta[shift:shift + n].setM([tm], G.ofNumpy(vals))
+    assert_exact(want, G.toNumpy(ta))
+
+
 @pytest.mark.parametrize("dt", [np.float32, np.float64, np.uint8, np.bool_, np.uint16])
 def test_masked_get_set_nd(H, G, rng, dt):
     a = (rng.random((37, 41)) < 0.5) if dt == np.bool_ else rng.integers(0, 100, (37, 41)).astype(dt)
