@@ -70,6 +70,23 @@ private:
 };
 int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease);
 
+// ---- tuning switches --------------------------------------------------------------------------------------------------
+// Process-wide integers behind dnh_set_option / dnh_get_option.  Each starts from an environment variable of the same name in
+// upper case with a DNH_ prefix (dot_bf16x3 <- DNH_DOT_BF16X3) or, without one, from the default below; a change applies to the
+// calls issued after it.  None of them changes a result's contract, only which kernel computes it.
+enum Option {
+    OPT_DOT_BF16X3 = 0,      // 1: single-precision products on the bf16 matrix instructions (three parts per float); 0: fp32 instruction
+    OPT_DOT_F64_PINNED,      // 1: double-precision products on gemm_f64_kernel where the layout allows; 0: gemm_kernel<double>
+    OPT_DOT_BIG,             // -1: the cost model picks the tile form of the bf16-parts kernel; 0 / 1: 128 x 128 / 256 x 256 tiles
+    OPT_DOT_SPLITS,          // 0: the cost model picks the number of chunks along K; n > 0: that many
+    OPT_DOT_INT_MFMA,        // 1: 32 / 64-bit integer products on the int8 matrix instruction; 0: gemm_int_kernel
+    OPT_TR4,                 // 1: 4-byte transposing copies through LDS where the layout asks for them; 0: the general n-d kernel
+    OPT_SCATTER_FP_ATOMIC,   // 0: floating-point scatter adds duplicates in source order (reproducible); 1: float atomics
+    OPT_COMPACT_ONE_PASS,    // 1: maskedGet / trueIndices / countTrue of contiguous masks in one launch; 0: count + move launches
+    OPT_COUNT
+};
+int option(Option o);
+
 // ---- dtypes -----------------------------------------------------------------------------------------------------------
 
 inline int dtype_size(int dt) {

@@ -446,12 +446,12 @@ __global__ __launch_bounds__(64 * SG) void gemm_split_finish_kernel(T* __restric
 // met such an element in its rows of A or columns of B recomputes its tile with the fp32 matrix instruction (fp32_tile_fallback:
 // IEEE products and sums, inf x finite = inf, inf x 0 = NaN, as the reference's sgemm).  NaN needs no fallback: one part of a NaN is
 // a NaN.  Products with K < 16 (no whole K step; worst case 8 u per product from the three dropped terms against 1 u of one
-// rounded fp32 product) stay on the fp32 instructions.  DNH_DOT_BF16X3=0 in the environment keeps every product there.
+// rounded fp32 product) stay on the fp32 instructions.  The option dot_bf16x3 = 0 keeps every product there.
 // Every operand that is contiguous along one of its two dimensions (row-major or transposed; 16-byte aligned rows when k is the
 // contiguous one), K splits included; accumulating products and operands strided in both dimensions take gemm_kernel.
 // Two forms: 128 x 128 tiles, 256 threads, two workgroups per CU (gemm_bf16x3_kernel: every size, K splits), and 256 x 256 tiles,
 // 512 threads, one workgroup per CU (gemm_bf16x3_big_kernel: half the staging and LDS traffic per matrix instruction; taken when
-// the product has about a CU's worth of such tiles, use_big_tiles; DNH_DOT_BIG=0 / 1 in the environment forces the choice).
+// the product has about a CU's worth of such tiles, use_big_tiles; the option dot_big = 0 / 1 forces the choice).
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 constexpr int kX3BK = 16;
@@ -529,10 +529,12 @@ struct X3Stage {
     }
     // cuts the staged elements into their parts and writes them to tile[part][row][k]
     __device__ __forceinline__ void store(float (&r)[8], __bf16 (*tile)[ROWS][kX3Row]) {
-        // +-inf stays infinite under the scaling; |x| < 2^-109 (x != 0) becomes denormal; zero stays zero
-        constexpr int kClassInfOrDenormal = (1 << 2) | (1 << 4) | (1 << 7) | (1 << 9);
+        // +-inf stays infinite under the scaling; 2^-126 <= |x| < 2^-109 becomes denormal; zero stays zero.  An element that is
+        // denormal already is tested as it is: scaled, the smallest ones (|x| <= 2^-133) would round to zero and pass for zeros.
+        constexpr int kClassInfOrDenormal = (1 << 2) | (1 << 4) | (1 << 7) | (1 << 9), kClassDenormal = (1 << 4) | (1 << 7);
 #pragma unroll
-        for (int e = 0; e < 8; e++) bad |= __builtin_amdgcn_classf(r[e] * 0x1p-17f, kClassInfOrDenormal);
+        for (int e = 0; e < 8; e++)
+            bad |= __builtin_amdgcn_classf(r[e] * 0x1p-17f, kClassInfOrDenormal) | __builtin_amdgcn_classf(r[e], kClassDenormal);
         u32x4 part[3];
         split3_bf16(r, part[0], part[1], part[2]);
 #pragma unroll
@@ -563,8 +565,8 @@ struct X3Stage {
             mw[e & 1] = m;
             lw[e & 1] = __float_as_uint(r2);
         } else {
-            constexpr int kClassInfOrDenormal = (1 << 2) | (1 << 4) | (1 << 7) | (1 << 9);
-            bad |= __builtin_amdgcn_classf(r[e] * 0x1p-17f, kClassInfOrDenormal);
+            constexpr int kClassInfOrDenormal = (1 << 2) | (1 << 4) | (1 << 7) | (1 << 9), kClassDenormal = (1 << 4) | (1 << 7);
+            bad |= __builtin_amdgcn_classf(r[e] * 0x1p-17f, kClassInfOrDenormal) | __builtin_amdgcn_classf(r[e], kClassDenormal);
             if constexpr (e % 2 == 1) {
                 part[0][e / 2] = __builtin_amdgcn_perm(hw[1], hw[0], 0x07060302u);
                 part[1][e / 2] = __builtin_amdgcn_perm(mw[1], mw[0], 0x07060302u);
@@ -931,8 +933,7 @@ __global__ __launch_bounds__(kBigThreads) void gemm_bf16x3_big_kernel(float* c, 
 }
 
 bool use_bf16x3() {
-    static const bool on = [] { const char* e = getenv("DNH_DOT_BF16X3"); return !e || e[0] != '0'; }();
-    return on;
+    return option(OPT_DOT_BF16X3) != 0;
 }
 
 // ---- double precision with a pinned instruction order ------------------------------------------------------------------------
@@ -1100,8 +1101,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemm_f64_kernel(double* c, const do
 }
 
 bool use_f64_pinned() {
-    static const bool on = [] { const char* e = getenv("DNH_DOT_F64_PINNED"); return !e || e[0] != '0'; }();   // 0: gemm_kernel<double> for every layout
-    return on;
+    return option(OPT_DOT_F64_PINNED) != 0;   // 0: gemm_kernel<double> for every layout
 }
 
 // Tile form and number of K chunks of a product on the kernels with a pinned instruction order: the cheapest of the available forms
@@ -1111,10 +1111,9 @@ bool use_f64_pinned() {
 //       lower the clock); 256 x 256 tiles, one per CU: 1.75 - 2.5;
 //   double precision (K step 8), 128 x 128 tiles: 2.05 with two workgroups on a CU, 1.10 - 1.26 with one.
 // A round of workgroups costs 8 / 10 / 13 us on top (launch, first fetch, epilogue), the summing launch 5 us plus its traffic at
-// 5 TB/s.  DNH_DOT_BIG=0 / 1 and DNH_DOT_SPLITS=n in the environment force either choice (for measurements and tests).
+// 5 TB/s.  The options dot_big = 0 / 1 and dot_splits = n force either choice (for measurements and tests).
 void choose_plan(bool f64, int64_t M, int64_t N, int64_t batch, int64_t steps, bool can_split, bool* big, int64_t* want) {
-    static const int force_big = [] { const char* e = getenv("DNH_DOT_BIG"); return e ? atoi(e) : -1; }();
-    static const int force_splits = [] { const char* e = getenv("DNH_DOT_SPLITS"); return e ? atoi(e) : 0; }();
+    const int force_big = option(OPT_DOT_BIG), force_splits = option(OPT_DOT_SPLITS);
     const int64_t cus = device_cus();
     const int64_t nbig = cdiv(M, (int64_t)XBM) * cdiv(N, (int64_t)XBN) * batch, nsmall = cdiv(M, (int64_t)BM) * cdiv(N, (int64_t)BN) * batch;
     const double out_bytes = (double)batch * (double)M * (double)N * (f64 ? 8.0 : 4.0);
@@ -1196,7 +1195,7 @@ int32_t launch_gemm(GemmArgs g, T* c, const T* a, const T* b, int64_t batch, hip
         }
     } else if (g.nbatch < DNH_MAX_DIMS && blocks <= 4 * (int64_t)device_cus()) {
         want = choose_k_splits<T>(blocks, steps, batch * g.M * g.N);
-        static const int force_splits = [] { const char* e = getenv("DNH_DOT_SPLITS"); return e ? atoi(e) : 0; }();
+        const int force_splits = option(OPT_DOT_SPLITS);
         if (force_splits > 0) want = std::min<int64_t>(force_splits, std::max<int64_t>(steps / 2, 1));
     }
     if (want > 1) {   // the choosers keep chunks of at least 2 steps: the chunk below is not empty
@@ -1959,8 +1958,7 @@ __global__ __launch_bounds__(kI8Threads) void gemm_i64_i8parts_kernel(uint64_t* 
 }
 
 bool use_int_mfma() {
-    static const bool on = [] { const char* e = getenv("DNH_DOT_INT_MFMA"); return !e || e[0] != '0'; }();   // 0: every integer product on gemm_int_kernel
-    return on;
+    return option(OPT_DOT_INT_MFMA) != 0;   // 0: every integer product on gemm_int_kernel
 }
 
 template <class T>

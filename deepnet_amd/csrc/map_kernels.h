@@ -916,7 +916,7 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
             bool big = false, tall = false, tr4 = false, tr4_gen = false;
             constexpr int TALL_TA = 128, TALL_TB = WIDE ? 128 : 256;
             if constexpr (VEC == 16 / ESZ && Op::NSRC >= 1 && Op::NSRC <= 2) {
-                static const bool tr4_on = [] { const char* e = getenv("DNH_TR4"); return !e || e[0] != '0'; }();
+                const bool tr4_on = option(OPT_TR4) != 0;
                 const bool tr4_ok = tr4_on && (Op::NSRC == 1 || q.dmode != 0);
                 const bool one4 = vec && nstaged == 1 && staged_esize == ESZ;
                 big = (tr4_ok || !WIDE) && one4 && q.nb <= 256 && (q.na % BIG_TA) == 0 && (q.nb % BIG_TB) == 0 &&

@@ -28,60 +28,47 @@ template <class X> struct RProd {
     __device__ X extract(X s) const { return s; }
 };
 // Max / Min follow the reference's sequential rule `if res > v then res else v` from minValue (Host/ScalarOps.fs:620-628).  Without
-// NaNs any order gives the same value.  With a NaN the rule depends on the order: the NaN replaces the running value, and the next
-// element replaces the NaN, so the result is the fold of what follows the last NaN (NaN if it comes last).  The tree therefore carries
-// a NaN through every step and combination (a result that met one is a NaN), and the thread that stores a NaN result recomputes it in
-// order (kSeqFix, finish_value): faithful for every input, at one extra comparison per element for NaN-free data.
-template <class X> struct RMax {
+// NaNs any order gives the same value: the larger of minValue and the true maximum.  With a NaN the rule depends on the order: the NaN
+// replaces the running value, and the next element replaces the NaN, so the result is the plain maximum of what follows the last NaN
+// (NaN if it comes last; minValue plays no part any more).  The tree therefore starts from -inf, carries a NaN through every step and
+// combination (a result that met one is a NaN) and applies minValue when it extracts; a NaN result is recomputed from the axis:
+// the threads that share a row look for its last NaN and fold what follows (reduce_rows_kernel: fix_rows), a thread that owns a
+// column walks it in order (sequential).  Partials of a two-pass fold are true maxima, so only the last chunk that holds a NaN is
+// read again.  Faithful for every input, at one extra comparison per element for NaN-free data.
+template <class X, bool MAX> struct RExtreme {
     using In = X; using State = X; using Out = X;
-    static constexpr bool kSeqFix = std::is_floating_point<X>::value;
-    __device__ X init() const { return std::numeric_limits<X>::lowest(); }
-    __device__ X step(X s, X v, int64_t) const { return (s > v || s != s) ? s : v; }
-    __device__ X combine(X a, X b) const { return (a > b || a != a) ? a : b; }
-    __device__ X extract(X s) const { return s; }
+    static constexpr bool kFloat = std::is_floating_point<X>::value;
+    static constexpr bool kSeqFix = kFloat;
+    // where the reference's fold starts
+    __device__ static X start() { return MAX ? std::numeric_limits<X>::lowest() : std::numeric_limits<X>::max(); }
+    // neutral element of pick()
+    __device__ static X identity() {
+        if constexpr (kFloat) return MAX ? -std::numeric_limits<X>::infinity() : std::numeric_limits<X>::infinity();
+        else return start();
+    }
+    __device__ static bool beats(X a, X b) { return MAX ? a > b : a < b; }
+    __device__ static X pick(X a, X b) { return beats(a, b) ? a : b; }              // the reference's step; NaN-free operands commute
+    __device__ X init() const { return identity(); }
+    __device__ X step(X s, X v, int64_t) const { return (beats(s, v) || s != s) ? s : v; }
+    __device__ X combine(X a, X b) const { return (beats(a, b) || a != a) ? a : b; }
+    __device__ X extract(X s) const { return pick(start(), s); }
     __device__ bool needs_fix(X s) const { return s != s; }
-    __device__ X sequential(const X* p, int64_t n, int64_t stride) const {
-        X s = std::numeric_limits<X>::lowest();
+    // the reference's fold over p[0], p[stride] .. p[(n - 1) stride] continued from s
+    __device__ X sequential(X s, const X* p, int64_t n, int64_t stride) const {
         int64_t i = 0;
         for (; i + 16 <= n; i += 16) {   // sixteen fetches on their way at a time, applied in order
             X v[16];
 #pragma unroll
             for (int u = 0; u < 16; u++) v[u] = p[(i + u) * stride];
 #pragma unroll
-            for (int u = 0; u < 16; u++) s = s > v[u] ? s : v[u];
+            for (int u = 0; u < 16; u++) s = pick(s, v[u]);
         }
-        for (; i < n; i++) {
-            const X v = p[i * stride];
-            s = s > v ? s : v;
-        }
+        for (; i < n; i++) s = pick(s, p[i * stride]);
         return s;
     }
 };
-template <class X> struct RMin {
-    using In = X; using State = X; using Out = X;
-    static constexpr bool kSeqFix = std::is_floating_point<X>::value;
-    __device__ X init() const { return std::numeric_limits<X>::max(); }
-    __device__ X step(X s, X v, int64_t) const { return (s < v || s != s) ? s : v; }
-    __device__ X combine(X a, X b) const { return (a < b || a != a) ? a : b; }
-    __device__ X extract(X s) const { return s; }
-    __device__ bool needs_fix(X s) const { return s != s; }
-    __device__ X sequential(const X* p, int64_t n, int64_t stride) const {
-        X s = std::numeric_limits<X>::max();
-        int64_t i = 0;
-        for (; i + 16 <= n; i += 16) {   // sixteen fetches on their way at a time, applied in order
-            X v[16];
-#pragma unroll
-            for (int u = 0; u < 16; u++) v[u] = p[(i + u) * stride];
-#pragma unroll
-            for (int u = 0; u < 16; u++) s = s < v[u] ? s : v[u];
-        }
-        for (; i < n; i++) {
-            const X v = p[i * stride];
-            s = s < v ? s : v;
-        }
-        return s;
-    }
-};
+template <class X> using RMax = RExtreme<X, true>;
+template <class X> using RMin = RExtreme<X, false>;
 struct RAll {
     using In = uint8_t; using State = uint8_t; using Out = uint8_t;
     __device__ uint8_t init() const { return 1; }

@@ -57,23 +57,110 @@ __device__ __forceinline__ typename R::State group_reduce(const R& r, typename R
 }
 
 // A fold may name results that the tree cannot produce faithfully (kSeqFix: Max / Min of floats that met a NaN, whose value under
-// the reference's sequential rule depends on where the NaN stood): the thread that stores such a result recomputes it by walking the
-// reduced axis in order (elements p[0], p[stride], ... p[(n - 1) stride]).  Rare by construction; every other result is extract(state).
+// the reference's sequential rule depends on where the NaN stood).  Such a reducer also supplies start(), identity(), pick(),
+// needs_fix() and sequential(); a result that needs_fix() is recomputed from the reduced axis (elements p[0], p[stride] ..
+// p[(n - 1) stride]).  Rare by construction; every other result is extract(state).
 template <class R, class = void> struct NeedsSeqFix : std::false_type {};
 template <class R> struct NeedsSeqFix<R, std::void_t<decltype(R::kSeqFix)>> : std::integral_constant<bool, R::kSeqFix> {};
+
+// By the one thread that owns the result (column and one-thread-per-output kernels): the whole axis in order.
 template <class R>
 __device__ __forceinline__ typename R::Out finish_value(const R& r, const typename R::State& s, const typename R::In* p, int64_t n, int64_t stride) {
     if constexpr (NeedsSeqFix<R>::value) {
-        if (r.needs_fix(s)) return r.sequential(p, n, stride);
+        if (r.needs_fix(s)) return r.sequential(R::start(), p, n, stride);
     }
     return r.extract(s);
 }
 
-// fix_src / fix_n / fix_sr (FROM_STATE only): the fold's source, the length and the stride of its reduced axis, for finish_value.
+// The same for a two-pass fold whose partials q[0], q[qstride] .. q[(splits - 1) qstride] are true folds of chunks of `chunk`
+// elements (NaN when the chunk holds one): only the last chunk with a NaN is walked, the partials behind it continue the fold.
+template <class R>
+__device__ __forceinline__ typename R::Out finish_value_chunked(const R& r, const typename R::State& s, const typename R::State* q, int64_t qstride,
+                                                                uint32_t splits, const typename R::In* p, int64_t n, int64_t stride, int64_t chunk) {
+    if constexpr (NeedsSeqFix<R>::value) {
+        if (r.needs_fix(s)) {
+            int64_t j = (int64_t)splits - 1;
+            while (j > 0 && !r.needs_fix(q[j * qstride])) j--;
+            const int64_t c0 = j * chunk, c1 = (c0 + chunk < n) ? c0 + chunk : n;
+            typename R::State v = r.sequential(R::start(), p + c0 * stride, c1 - c0, stride);
+            for (int64_t k = j + 1; k < (int64_t)splits; k++) v = R::pick(v, q[k * qstride]);
+            return v;
+        }
+    }
+    return r.extract(s);
+}
+
+// All-reduce of v over the G threads that share a row (threads `threadIdx.x % G` of a group are consecutive): shuffles inside a
+// wavefront; G = kBlock: the wavefronts' values meet in `sh` (kBlock / 64 words of 8 bytes), every thread of the block calls.
+template <int G, class V, class F>
+__device__ __forceinline__ V group_all_reduce(V v, F f, uint64_t* sh) {
+#pragma unroll
+    for (int m = (G < 64 ? G : 64) / 2; m >= 1; m >>= 1) v = f(v, shfl_xor_any(v, m));
+    if constexpr (G > 64) {
+        static_assert(sizeof(V) <= 8, "group_all_reduce: value wider than a slot");
+        __syncthreads();   // an earlier use of sh is over
+        if ((threadIdx.x & 63) == 0) __builtin_memcpy(&sh[threadIdx.x / 64], &v, sizeof(V));
+        __syncthreads();
+        __builtin_memcpy(&v, &sh[0], sizeof(V));
+#pragma unroll
+        for (int w = 1; w < G / 64; w++) {
+            V o;
+            __builtin_memcpy(&o, &sh[w], sizeof(V));
+            v = f(v, o);
+        }
+    }
+    return v;
+}
+
+// The reference's sequential Max / Min over elements i0 .. i1 - 1 of an axis, for a range known to hold a NaN, by the G threads that
+// share the row: the position of the last NaN, then the plain fold of what follows it (NaN when nothing does).
+template <class R, int G>
+__device__ __forceinline__ typename R::In fold_after_last_nan(const typename R::In* p, int64_t i0, int64_t i1, int64_t stride, uint32_t lane,
+                                                              uint64_t* sh) {
+    using X = typename R::In;
+    int64_t q = i0 - 1;
+#pragma unroll 4
+    for (int64_t i = i0 + lane; i < i1; i += G) {
+        const X v = p[i * stride];
+        if (v != v) q = i;
+    }
+    q = group_all_reduce<G>(q, [](int64_t a, int64_t b) { return a > b ? a : b; }, sh);
+    X m = R::identity();
+#pragma unroll 4
+    for (int64_t i = q + 1 + lane; i < i1; i += G) m = R::pick(m, p[i * stride]);
+    m = group_all_reduce<G>(m, [](X a, X b) { return R::pick(a, b); }, sh);
+    return q == i1 - 1 ? p[q * stride] : m;
+}
+
+// A NaN result of a row, recomputed by the G threads that share it (all of them call; the result is the same in each).
+// FROM_STATE: part[0 .. splits - 1] are the chunks' partials (true folds, NaN where the chunk holds one) and `chunk` their length.
+template <class R, int G, bool FROM_STATE>
+__device__ __forceinline__ typename R::In fix_rows(const typename R::In* src, int64_t n, int64_t stride, const typename R::In* part,
+                                                   int64_t splits, int64_t chunk, uint32_t lane, uint64_t* sh) {
+    using X = typename R::In;
+    if constexpr (!FROM_STATE) {
+        return fold_after_last_nan<R, G>(src, 0, n, stride, lane, sh);
+    } else {
+        int64_t j = -1;
+        for (int64_t i = lane; i < splits; i += G)
+            if (part[i] != part[i]) j = i;
+        j = group_all_reduce<G>(j, [](int64_t a, int64_t b) { return a > b ? a : b; }, sh);
+        const int64_t c0 = j * chunk, c1 = (c0 + chunk < n) ? c0 + chunk : n;
+        const X m = fold_after_last_nan<R, G>(src, c0, c1, stride, lane, sh);
+        if (j + 1 >= splits) return m;
+        X t = R::identity();
+        for (int64_t i = j + 1 + lane; i < splits; i += G) t = R::pick(t, part[i]);
+        t = group_all_reduce<G>(t, [](X a, X b) { return R::pick(a, b); }, sh);
+        return R::pick(m, t);   // m is a NaN when its chunk ends with one: the fold goes on from the chunks behind it
+    }
+}
+
+// fix_src / fix_n / fix_sr / fix_chunk (FROM_STATE only): the fold's source, the length and the stride of its reduced axis and the
+// elements of it behind each partial, for fix_rows.
 template <class R, int VEC, int TPR, bool FROM_STATE>
 __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(R r, const void* src_, typename R::Out* out, typename R::State* partial,
                                                              OuterArgs o, uint32_t rows, int64_t n, int64_t sr, int64_t chunk, uint32_t splits,
-                                                             const typename R::In* fix_src, int64_t fix_n, int64_t fix_sr) {
+                                                             const typename R::In* fix_src, int64_t fix_n, int64_t fix_sr, int64_t fix_chunk) {
     using State = typename R::State;
     using In = typename std::conditional<FROM_STATE, State, typename R::In>::type;
     constexpr int RPB = kBlock / TPR;
@@ -137,11 +224,28 @@ __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(R r, const void* sr
             for (int w = 1; w < TPR / 64; w++) s = r.combine(s, sh[w]);
         }
     }
-    if (active && lane == 0) {
+    if constexpr (NeedsSeqFix<R>::value) {
         if (splits == 1) {
-            if constexpr (FROM_STATE) out[toff] = finish_value(r, s, fix_src + soff0, fix_n, fix_sr);
-            else out[toff] = finish_value(r, s, (const typename R::In*)src_ + soff0, n, sr);
-        } else partial[(int64_t)row * splits + blockIdx.y] = s;
+            __shared__ uint64_t fix_sh[kBlock / 64];
+            bool fix = active && r.needs_fix(s);   // the same in every thread of a row's group of up to 64
+            if constexpr (TPR > 64) {   // one row per block: thread 0 holds the block's result
+                __shared__ int fix_flag;
+                if (threadIdx.x == 0) fix_flag = fix;
+                __syncthreads();
+                fix = fix_flag != 0;
+            }
+            if (fix) {
+                typename R::In v;
+                if constexpr (FROM_STATE) v = fix_rows<R, TPR, true>(fix_src + soff0, fix_n, fix_sr, (const typename R::In*)src_ + soff, n, fix_chunk, lane, fix_sh);
+                else v = fix_rows<R, TPR, false>((const typename R::In*)src_ + soff0, n, sr, nullptr, 0, 0, lane, fix_sh);
+                if (lane == 0) out[toff] = v;
+                return;
+            }
+        }
+    }
+    if (active && lane == 0) {
+        if (splits == 1) out[toff] = r.extract(s);
+        else partial[(int64_t)row * splits + blockIdx.y] = s;
     }
 }
 
@@ -229,7 +333,7 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(R r, const typename
 template <class R, int WX>
 __global__ __launch_bounds__(kBlock) void reduce_cols_finish_kernel(R r, const typename R::State* partial, typename R::Out* out, OuterArgs o,
                                                                     uint32_t col_tiles, uint32_t nc, int64_t tc_stride, uint32_t splits,
-                                                                    const typename R::In* fix_src, int64_t fix_n, int64_t fix_sr) {
+                                                                    const typename R::In* fix_src, int64_t fix_n, int64_t fix_sr, int64_t fix_chunk) {
     using State = typename R::State;
     constexpr int NY = kBlock / WX;
     const uint32_t x = threadIdx.x % WX, y = threadIdx.x / WX;
@@ -256,7 +360,8 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_finish_kernel(R r, const t
         for (int w = 1; w < NY; w++) st = r.combine(st, sh[w][x]);
         int64_t toff, soff;
         outer_offsets(o, other, toff, soff);
-        out[toff + (int64_t)col * tc_stride] = finish_value(r, st, fix_src + soff + col, fix_n, fix_sr);
+        out[toff + (int64_t)col * tc_stride] = finish_value_chunked(r, st, partial + (int64_t)other * splits * nc + col, (int64_t)nc, splits,
+                                                                    fix_src + soff + col, fix_n, fix_sr, fix_chunk);
     }
 }
 
@@ -278,10 +383,10 @@ __global__ __launch_bounds__(kBlock) void reduce_generic_kernel(R r, const typen
 // Finishing pass of the two-pass tree: `nout` rows of `splits` State partials each.
 template <class R>
 int32_t launch_finish(const R& r, typename R::State* partial, typename R::Out* out, const OuterArgs& o, uint32_t nout, uint32_t splits,
-                      const typename R::In* fix_src, int64_t fix_n, int64_t fix_sr, hipStream_t stream) {
+                      const typename R::In* fix_src, int64_t fix_n, int64_t fix_sr, int64_t fix_chunk, hipStream_t stream) {
     using State = typename R::State;
 #define DNH_FIN(TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, 1, TPR, true>), dim3(cdiv(nout, kBlock / TPR)), dim3(kBlock), 0, stream, r, \
-                                        (const void*)partial, out, (State*)nullptr, o, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u, fix_src, fix_n, fix_sr)
+                                        (const void*)partial, out, (State*)nullptr, o, nout, (int64_t)splits, (int64_t)1, (int64_t)splits, 1u, fix_src, fix_n, fix_sr, fix_chunk)
     if (splits > 512) DNH_FIN(256);
     else if (splits > 32) DNH_FIN(64);
     else DNH_FIN(16);
@@ -388,7 +493,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         WorkspaceLease lease;
         if (splits > 1) DNH_TRY(partial_buffer(ps, stream, sizeof(State) * (size_t)nout * splits, (void**)&partial, lease, what));
         const dim3 grid((unsigned)row_blocks, splits);
-#define DNH_ROWS(V, TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, V, TPR, false>), grid, dim3(kBlock), 0, stream, r, (const void*)src, out, partial, o, nout, n, sr, chunk, splits, src, n, sr)
+#define DNH_ROWS(V, TPR) hipLaunchKernelGGL((reduce_rows_kernel<R, V, TPR, false>), grid, dim3(kBlock), 0, stream, r, (const void*)src, out, partial, o, nout, n, sr, chunk, splits, src, n, sr, chunk)
         if (vec) {
             if (tpr == 256) DNH_ROWS(VEC, 256); else if (tpr == 64) DNH_ROWS(VEC, 64); else DNH_ROWS(VEC, 16);
         } else {
@@ -398,7 +503,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
         DNH_LAUNCH_CHECK();
         if (splits > 1) {
             // finishing pass: rows of `splits` State partials
-            DNH_TRY(launch_finish(r, partial, out, o, nout, splits, src, n, sr, stream));
+            DNH_TRY(launch_finish(r, partial, out, o, nout, splits, src, n, sr, chunk, stream));
         }
         return DNH_OK;
     }
@@ -463,7 +568,7 @@ int32_t launch_reduce(const R& r, const DnhTensor* t, const DnhTensor* s, hipStr
                 constexpr int FW = 32;   // (16 and 64 columns per finishing workgroup measured 1-2 % slower on 8192 x 8192)
                 const uint32_t ftiles = cdiv(nc, FW);
                 hipLaunchKernelGGL((reduce_cols_finish_kernel<R, FW>), dim3(ftiles * others), dim3(kBlock), 0, stream, r, (const State*)partial, out,
-                                   oo, ftiles, nc, tc_stride, splits, src, n, sr);
+                                   oo, ftiles, nc, tc_stride, splits, src, n, sr, chunk);
                 DNH_LAUNCH_CHECK();
             }
             return DNH_OK;

@@ -8,6 +8,8 @@
 #include <mutex>
 #include <thread>
 #include <vector>
+#include <cctype>
+#include <cstdlib>
 #include <cstring>
 #include <unordered_map>
 
@@ -121,6 +123,47 @@ int32_t ensure_init() {
 }
 
 int device_cus() { return g_cus; }
+
+namespace {
+struct OptionDef {
+    const char* name;
+    int def, lo, hi;
+};
+// order of enum Option
+constexpr OptionDef kOptions[OPT_COUNT] = {
+    {"dot_bf16x3", 1, 0, 1},       {"dot_f64_pinned", 1, 0, 1},    {"dot_big", -1, -1, 1},          {"dot_splits", 0, 0, 1 << 20},
+    {"dot_int_mfma", 1, 0, 1},     {"tr4", 1, 0, 1},               {"scatter_fp_atomic", 0, 0, 1},  {"compact_one_pass", 1, 0, 1},
+};
+std::atomic<int> g_options[OPT_COUNT];
+std::once_flag g_options_once;
+void init_options() {
+    std::call_once(g_options_once, [] {
+        for (int o = 0; o < OPT_COUNT; o++) {
+            std::string env = "DNH_";
+            for (const char* c = kOptions[o].name; *c; c++) env += (char)toupper((unsigned char)*c);
+            const char* e = getenv(env.c_str());
+            int v = kOptions[o].def;
+            if (e && *e) {
+                v = atoi(e);
+                if (v < kOptions[o].lo) v = kOptions[o].lo;
+                if (v > kOptions[o].hi) v = kOptions[o].hi;
+            }
+            g_options[o].store(v, std::memory_order_relaxed);
+        }
+    });
+}
+int find_option(const char* name) {
+    if (!name) return -1;
+    for (int o = 0; o < OPT_COUNT; o++)
+        if (strcmp(name, kOptions[o].name) == 0) return o;
+    return -1;
+}
+}  // namespace
+
+int option(Option o) {
+    init_options();
+    return g_options[o].load(std::memory_order_relaxed);
+}
 int32_t error_flag_ptr(hipStream_t stream, int32_t** out) {
     std::lock_guard<std::mutex> lock(g_mu);
     int32_t*& p = g_error_flags[stream];
@@ -201,6 +244,23 @@ int32_t dnh_device_info(DnhDeviceInfo* info) {
     info->memory_clock_khz = prop.memoryClockRate;
     strncpy(info->name, prop.name, sizeof(info->name) - 1);
     strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
+    return DNH_OK;
+}
+
+int32_t dnh_set_option(const char* name, int32_t value) {
+    const int o = find_option(name);
+    if (o < 0) return fail(DNH_ERR_INVALID_ARG, "dnh_set_option: unknown option '%s'", name ? name : "(null)");
+    if (value < kOptions[o].lo || value > kOptions[o].hi)
+        return fail(DNH_ERR_INVALID_ARG, "dnh_set_option: %s takes %d..%d, not %d", name, kOptions[o].lo, kOptions[o].hi, value);
+    init_options();
+    g_options[o].store(value, std::memory_order_relaxed);
+    return DNH_OK;
+}
+
+int32_t dnh_get_option(const char* name, int32_t* value) {
+    const int o = find_option(name);
+    if (o < 0 || !value) return fail(DNH_ERR_INVALID_ARG, "dnh_get_option: unknown option '%s' or null argument", name ? name : "(null)");
+    *value = option((Option)o);
     return DNH_OK;
 }
 

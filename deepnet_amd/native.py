@@ -35,6 +35,8 @@ def load() -> C.CDLL:
         "dnh_device_info": [C.POINTER(abi.DnhDeviceInfo)],
         "dnh_last_error": [C.c_char_p, sz],
         "dnh_async_error": [vp, C.POINTER(i32)],
+        "dnh_set_option": [C.c_char_p, i32],
+        "dnh_get_option": [C.c_char_p, C.POINTER(i32)],
         "dnh_alloc": [sz, C.POINTER(vp)],
         "dnh_free": [vp],
         "dnh_alloc_async": [sz, vp, C.POINTER(vp)],
@@ -78,6 +80,33 @@ _EXC = {
     abi.DNH_ERR_SINGULAR_MATRIX: SingularMatrixException,
     abi.DNH_ERR_NO_CONVERGENCE: ArithmeticError,
 }
+
+
+def set_option(name: str, value: int) -> None:
+    """dnh_set_option: a process-wide tuning switch of the library (which kernel computes a result, never its contract)."""
+    check(load().dnh_set_option(name.encode(), int(value)))
+
+
+def get_option(name: str) -> int:
+    v = C.c_int32()
+    check(load().dnh_get_option(name.encode(), C.byref(v)))
+    return v.value
+
+
+class option:
+    """`with native.option("dot_bf16x3", 0): ...` sets a switch for the calls issued inside the block."""
+
+    def __init__(self, name: str, value: int):
+        self.name, self.value = name, value
+
+    def __enter__(self):
+        self.saved = get_option(self.name)
+        set_option(self.name, self.value)
+        return self
+
+    def __exit__(self, *exc):
+        set_option(self.name, self.saved)
+        return False
 
 
 def last_error() -> str:

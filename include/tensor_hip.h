@@ -152,6 +152,20 @@ int32_t dnh_init(int32_t device);
 int32_t dnh_device_info(DnhDeviceInfo* info);
 /* Copies the calling thread's last error message (NUL terminated, truncated to n). */
 int32_t dnh_last_error(char* buf, size_t n);
+/* Tuning switches (no counterpart in the reference, whose backends take theirs from Tensor.Cfg statics): process-wide integers that
+ * select which kernel computes a result, never its contract; a change applies to the calls issued after it.  Each starts from the
+ * environment variable DNH_<NAME IN UPPER CASE> when the process has one.
+ *   "dot_bf16x3"        1 (default): single-precision products on the bf16 matrix instruction, three parts per float; 0: fp32 instruction
+ *   "dot_f64_pinned"    1 (default): double-precision products on the kernel with a pinned instruction order where the layout allows
+ *   "dot_big"           -1 (default): the library picks the tile form of the bf16-parts kernel; 0 / 1: 128 x 128 / 256 x 256 tiles
+ *   "dot_splits"        0 (default): the library picks the number of chunks along K; n > 0: that many
+ *   "dot_int_mfma"      1 (default): 32- and 64-bit integer products on the int8 matrix instruction
+ *   "tr4"               1 (default): transposing copies of 4-byte elements through LDS
+ *   "scatter_fp_atomic" 0 (default): floating-point scatter adds duplicates in source order; 1: float atomics (faster, order varies)
+ *   "compact_one_pass"  1 (default): compactions of contiguous masks in one launch; 0: a counting and a moving launch
+ * Unknown names and values outside an option's range: DNH_ERR_INVALID_ARG. */
+int32_t dnh_set_option(const char* name, int32_t value);
+int32_t dnh_get_option(const char* name, int32_t* value);
 /* Reads and clears the device-side index error flag set by gather/scatter kernels on `stream`
  * (synchronises the stream; every stream has its own flag, so concurrent streams do not see each other's errors).  *code = DNH_OK or DNH_ERR_INDEX_OUT_OF_RANGE.
  * Replaces the error word + `Cfg.Stacktrace` read-back of Cuda/CudaKernels.fs:323-342, 385-398. */
@@ -264,7 +278,7 @@ int32_t dnh_true_indices(const DnhTensor* t_i64, const DnhTensor* src_bool, void
  * into three bf16 parts (six of the nine partial products; error within 16 u S of the exact product like an fp32 sgemm, u = 2^-24,
  * S = sum_k |a_ik||b_kj|); tiles whose operands hold an infinite element or a nonzero element below 2^-109, which cannot be cut
  * exactly, are computed with the fp32 instruction, so infinities and NaNs come out as IEEE arithmetic (the reference's sgemm) gives
- * them.  DNH_DOT_BF16X3=0 in the environment keeps every product on the fp32 instruction (a tuning switch, same results contract).
+ * them.  dnh_set_option("dot_bf16x3", 0) keeps every product on the fp32 instruction (a tuning switch, same results contract).
  * Denormal operands are honoured, but the single-precision matrix instruction flushes products and partial sums below 2^-126 to
  * zero: results carry an absolute error of up to K x 2^-126 on top of the bound.  The integer types wrap like the host backend's
  * multiply + sumAxis (HostBackend.fs:544-546); bool: status 2.

@@ -27,7 +27,7 @@ def check_dot(ref, got, a, b):
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
 @pytest.mark.parametrize("m,k,n", [(5, 3, 3), (128, 16, 128), (128, 512, 128), (256, 64, 384), (130, 70, 50), (1, 1, 1), (33, 1000, 7)])
-def test_matmat(H, G, rng, dt, m, k, n):
+def test_matmat(H, G, rng, dt, m, k, n, tile_form):
     a = rng.standard_normal((m, k)).astype(dt)
     b = rng.standard_normal((k, n)).astype(dt)
     ref, got = both(H, G, lambda a, b: a @ b, a, b)
@@ -81,7 +81,7 @@ def test_vecvec_matvec(H, G, rng, dt):
     ((130, 4099), (4099, 70)),         # edge tiles in m and n, K not a multiple of the K step
     ((3, 2, 100, 1500), (3, 2, 1500, 60)),   # batch dimensions in front of the chunk dimension
 ])
-def test_split_k(H, G, rng, dt, shape_a, shape_b):
+def test_split_k(H, G, rng, dt, shape_a, shape_b, tile_form):
     """Products with few output tiles are cut along K and their partials added in chunk order: same bound as the uncut product,
     for contiguous operands, for transposed views (the strided kernel) and for a strided target."""
     a = rng.standard_normal(shape_a).astype(dt)
@@ -106,7 +106,7 @@ def test_split_k(H, G, rng, dt, shape_a, shape_b):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
-def test_batched_equals_loop_and_broadcast(H, G, rng, dt):
+def test_batched_equals_loop_and_broadcast(H, G, rng, dt, tile_form):
     # Tensor.Test/BaseTests.fs:84-96: a batched product equals the loop of 2-d products
     a = rng.standard_normal((3, 4, 128, 48)).astype(dt)
     b = rng.standard_normal((3, 4, 48, 130)).astype(dt)
@@ -133,7 +133,7 @@ def test_batched_equals_loop_and_broadcast(H, G, rng, dt):
     check_dot(np.swapaxes(ref2, -1, -2), np.swapaxes(got2, -1, -2), a, b)
 
 
-def test_config5_block_small(H, G, rng):
+def test_config5_block_small(H, G, rng, tile_form):
     """batched matmul -> tanh -> row softmax (max, subtract, exp, sum, divide), the fifth benchmark configuration."""
     a = (rng.standard_normal((4, 128, 128)) / np.sqrt(128)).astype(np.float32)
     b = (rng.standard_normal((4, 128, 128)) / np.sqrt(128)).astype(np.float32)
@@ -222,7 +222,7 @@ def test_vector_forms_layouts_and_sizes(H, G, rng, dt):
 
 @pytest.mark.parametrize("shape_a,shape_b", [((200, 64), (64, 300)), ((384, 16), (16, 256)), ((3, 130, 48), (3, 48, 257)),
                                              ((2, 2, 128, 32), (2, 2, 32, 128)), ((1500, 96), (96, 1100))])
-def test_single_precision_on_bf16_parts(H, G, rng, shape_a, shape_b):
+def test_single_precision_on_bf16_parts(H, G, rng, shape_a, shape_b, tile_form):
     """Row-major single-precision products whose K is a multiple of 16 and that are not split along K run on the bf16 matrix
     instructions with every float cut into three bf16 parts.  Same contract as the fp32 instructions, and in practice the same
     accuracy: within 16 u S of the fp64 product for these sizes (the fp32 instructions measure 4-8 u S)."""
@@ -256,7 +256,7 @@ STAGINGS = [(False, False), (True, False), (False, True), (True, True)]
 @pytest.mark.parametrize("m,k,n", [(256, 64, 256),      # whole tiles, one launch
                                    (700, 900, 650),     # cut along K into chunks
                                    (130, 4099, 70)])    # edge tiles, ragged K, chunks
-def test_single_precision_special_values_follow_ieee(H, G, rng, m, k, n):
+def test_single_precision_special_values_follow_ieee(H, G, rng, m, k, n, tile_form):
     """Infinite, NaN, denormal-range and very small elements in the default single-precision product: the reference's sgemm forms
     IEEE products and sums (Host/HostBackend.fs:513-546), so inf x finite = +-inf, inf x 0 = NaN, inf - inf = NaN, NaN stays NaN.
     The class of every output (NaN / +inf / -inf / finite) must equal the oracle's and NumPy's, finite outputs keep the K-term bound."""
@@ -298,7 +298,7 @@ def test_single_precision_special_values_follow_ieee(H, G, rng, m, k, n):
 
 
 @pytest.mark.parametrize("scale", [1e-30, 1e-33, 1e-36, 1e-38])
-def test_single_precision_small_operands_keep_their_precision(G, rng, scale):
+def test_single_precision_small_operands_keep_their_precision(G, rng, scale, tile_form):
     """Elements below 2^-109 cannot be cut into three bf16 parts exactly (the lowest part would fall below the smallest bf16
     denormal); tiles that hold such elements are computed on the fp32 instruction instead: same tight bound as O(1) data."""
     a = (rng.standard_normal((256, 512)) * scale).astype(np.float32)
@@ -310,7 +310,7 @@ def test_single_precision_small_operands_keep_their_precision(G, rng, scale):
         assert _err_over_uS(b.T, a.T, G.toNumpy(x @ y)).max() <= 16
 
 
-def test_single_precision_denormal_operands_and_sums(G, rng):
+def test_single_precision_denormal_operands_and_sums(G, rng, tile_form):
     """Denormal operands (below 2^-126) are honoured; products and partial sums that are themselves below 2^-126 may be flushed
     to zero by the matrix instruction.  Stated bound: K x 2^-126 of absolute error on top of the K-term bound."""
     d = np.full((128, 16), 1e-40, np.float32)
@@ -325,6 +325,32 @@ def test_single_precision_denormal_operands_and_sums(G, rng):
         a64, b64 = a.astype(np.float64), b.astype(np.float64)
         bound = (2 * 64 + 64) * 2.0 ** -24 * (np.abs(a64) @ np.abs(b64)) + 64 * 2.0 ** -126
         assert np.all(np.abs(got - a64 @ b64) <= bound)
+
+
+@pytest.mark.parametrize("tiny", [2.0 ** -140, 2.0 ** -149, 2.0 ** -133, 1e-42, 2.0 ** -127])
+def test_single_precision_smallest_denormal_operands(G, tiny, tile_form):
+    """A denormal operand cannot be cut into bf16 parts (all its set bits lie in the low 16): its tile goes to the fp32 instruction,
+    also when the element is so small that scaling it by 2^-17 rounds to zero.  tiny x 2^100 summed K times is a normal number that
+    fp32 arithmetic gives exactly; every staging, both tile forms, one launch and chunks along K."""
+    from deepnet_amd import native
+    t32 = np.float32(tiny)
+    assert t32 != 0
+    for (m, k, n) in ((128, 16, 128), (256, 64, 384), (130, 4099, 70)):
+        a = np.zeros((m, k), np.float32)
+        b = np.full((k, n), 2.0 ** 100, np.float32)
+        a[:, :16] = t32                       # sixteen equal terms: every partial sum is exact
+        a[5, :] = 0
+        a[5, 3] = t32                         # a single tiny element in an otherwise zero row
+        want = (a.astype(np.float64) @ b.astype(np.float64)).astype(np.float32)
+        assert np.all(want[0] == np.float32(16 * float(t32) * 2.0 ** 100)) and np.all(want[5] == np.float32(float(t32) * 2.0 ** 100))
+        for ta, tb in STAGINGS:
+            x, y = _views(G, a, b, ta, tb)
+            assert np.array_equal(G.toNumpy(x @ y), want), (m, k, n, ta, tb)
+            x, y = _views(G, np.ascontiguousarray(b.T), np.ascontiguousarray(a.T), ta, tb)   # the tiny operand on the right
+            assert np.array_equal(G.toNumpy(x @ y), want.T), (m, k, n, ta, tb, "right")
+        with native.option("dot_splits", 4):
+            x, y = _views(G, a, b, False, False)
+            assert np.array_equal(G.toNumpy(x @ y), want), (m, k, n, "chunks")
 
 
 @pytest.mark.parametrize("k", [1, 2, 3, 4, 8, 15])
@@ -350,7 +376,7 @@ def test_single_precision_short_inner_dimension(H, G, rng, k):
     ((130, 4099), (4099, 70)),               # ragged K, chunks
     ((3, 2, 100, 1500), (3, 2, 1500, 60)),   # batch dimensions in front of the chunks
 ])
-def test_single_precision_tight_bound_at_benchmark_shapes(G, rng, shape_a, shape_b):
+def test_single_precision_tight_bound_at_benchmark_shapes(G, rng, shape_a, shape_b, tile_form):
     """The bf16-parts kernel keeps six of the nine partial products.  A kernel that dropped one more (mid x mid, or a hi x lo) would
     be off by about 2^-16 |a||b| per product: 256 u, all of one sign for positive data, i.e. 50 u S and more at any K.  Measured:
     at most 3.2 u S for normal data and 11.2 u S for positive data (NumPy's sgemm on the same inputs: 3.0 and 14.5), so 16 u S is
@@ -366,7 +392,7 @@ def test_single_precision_tight_bound_at_benchmark_shapes(G, rng, shape_a, shape
 
 @pytest.mark.parametrize("ta,tb", [(True, False), (False, True), (True, True)])
 @pytest.mark.parametrize("m,k,n", [(200, 64, 300), (257, 100, 130), (1100, 40, 1500)])
-def test_single_precision_on_bf16_parts_transposed_views(H, G, rng, ta, tb, m, k, n):
+def test_single_precision_on_bf16_parts_transposed_views(H, G, rng, ta, tb, m, k, n, tile_form):
     """Operands that are transposed views of row-major matrices take the same kernel with the other staging."""
     a = rng.standard_normal((k, m) if ta else (m, k)).astype(np.float32)
     b = rng.standard_normal((n, k) if tb else (k, n)).astype(np.float32)
@@ -379,31 +405,31 @@ def test_single_precision_on_bf16_parts_transposed_views(H, G, rng, ta, tb, m, k
     assert np.all(np.abs(got - exact) <= 16 * 2.0 ** -24 * S)
 
 
-def test_fp32_instruction_kernel_behind_the_switch():
-    """DNH_DOT_BF16X3=0 sends single-precision products to the fp32 matrix instructions (the switch is read once per process, so
-    this runs in a child process): same contract, same IEEE treatment of infinities."""
-    import os
-    import subprocess
-    import sys
-    code = r'''
-import numpy as np
-from deepnet_amd import hip as G
-rng = np.random.default_rng(3)
-for (m, k, n) in ((200, 64, 300), (384, 16, 256), (130, 70, 50), (1024, 1024, 1024)):
-    a = rng.standard_normal((m, k)).astype(np.float32); b = rng.standard_normal((k, n)).astype(np.float32)
-    got = G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b)).astype(np.float64)
-    exact = a.astype(np.float64) @ b.astype(np.float64)
-    S = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
-    assert np.all(np.abs(got - exact) <= (2 * k + 64) * 2.0 ** -24 * S), (m, k, n)
-a = np.ones((128, 16), np.float32); b = np.ones((16, 128), np.float32); a[3, 5] = np.inf
-got = G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b))
-assert np.all(np.isposinf(got[3])) and np.all(np.delete(got, 3, axis=0) == 16)
-print("ok")
-'''
-    env = dict(os.environ, DNH_DOT_BF16X3="0")
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    out = subprocess.run([sys.executable, "-c", code], env=env, cwd=root, capture_output=True, text=True, timeout=300)
-    assert out.returncode == 0 and out.stdout.strip().endswith("ok"), out.stdout + out.stderr
+def test_fp32_instruction_kernel_behind_the_switch(G):
+    """dnh_set_option("dot_bf16x3", 0) sends single-precision products to the fp32 matrix instructions: same contract, same IEEE
+    treatment of infinities; products of normal numbers are then single fp32 roundings, so K = 1 is exact."""
+    from deepnet_amd import native
+    rng = np.random.default_rng(3)
+    assert native.get_option("dot_bf16x3") == 1
+    with native.option("dot_bf16x3", 0):
+        assert native.get_option("dot_bf16x3") == 0
+        for (m, k, n) in ((200, 64, 300), (384, 16, 256), (130, 70, 50), (1024, 1024, 1024)):
+            a = rng.standard_normal((m, k)).astype(np.float32)
+            b = rng.standard_normal((k, n)).astype(np.float32)
+            got = G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b)).astype(np.float64)
+            exact = a.astype(np.float64) @ b.astype(np.float64)
+            S = np.abs(a).astype(np.float64) @ np.abs(b).astype(np.float64)
+            assert np.all(np.abs(got - exact) <= (2 * k + 64) * 2.0 ** -24 * S), (m, k, n)
+        a = np.ones((128, 16), np.float32)
+        b = np.ones((16, 128), np.float32)
+        a[3, 5] = np.inf
+        got = G.toNumpy(G.ofNumpy(a) @ G.ofNumpy(b))
+        assert np.all(np.isposinf(got[3])) and np.all(np.delete(got, 3, axis=0) == 16)
+    assert native.get_option("dot_bf16x3") == 1
+    with pytest.raises(ValueError):
+        native.set_option("dot_bf16x3", 2)
+    with pytest.raises(ValueError):
+        native.set_option("no_such_switch", 1)
 
 
 @pytest.mark.parametrize("ta,tb", STAGINGS)
@@ -430,20 +456,13 @@ def test_single_precision_large_tiles(G, rng, ta, tb, m, k, n):
     assert _err_over_uS(af, bf, np.where(fin, got, 0))[fin].max() <= 16
 
 
-def test_large_tile_kernel_on_every_shape_of_this_file():
-    """DNH_DOT_BIG=1 sends every product that the bf16-parts kernel takes in one launch to its large-tile form, whatever the size
-    (the switch is read once per process, so the tests of this file run again in a child process)."""
-    import os
-    import subprocess
-    import sys
-    if os.environ.get("DNH_DOT_BIG") is not None:
-        pytest.skip("already running under the switch")
-    env = dict(os.environ, DNH_DOT_BIG="1")
-    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    out = subprocess.run([sys.executable, "-m", "pytest", "-x", "-q", "-m", "gpu", "-p", "no:cacheprovider", os.path.abspath(__file__),
-                          "-k", "single_precision or matmat or batched or split_k or config5"],
-                         env=env, cwd=root, capture_output=True, text=True, timeout=900)
-    assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-2000:]
+@pytest.fixture(params=[-1, 1], ids=["tiles_auto", "tiles_256"])
+def tile_form(request):
+    """Runs a test once with the library's own choice of tile form and once with dot_big = 1, which sends every product that the
+    bf16-parts kernel takes to its 256 x 256 form, whatever the size."""
+    from deepnet_amd import native
+    with native.option("dot_big", request.param):
+        yield request.param
 
 
 @pytest.mark.parametrize("ta,tb", STAGINGS)

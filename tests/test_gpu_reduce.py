@@ -229,3 +229,41 @@ def test_max_min_follow_the_sequential_rule_with_nans(H, G, rng, dt, shape):
     assert np.array_equal(ref, got, equal_nan=True)
     ref, got = both(H, G, lambda t: t.min(), x)
     assert np.array_equal(ref, got, equal_nan=True)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_max_min_with_nans_on_long_axes(H, G, dt):
+    """NaNs in folds whose axis is cut into chunks (a whole tensor of 2^24 elements, a few rows of 2^20, a tall matrix reduced down
+    its columns): the threads that share the row redo only the last chunk that holds a NaN.  NaN in the first chunk, in the middle,
+    as the last element of a chunk that is followed by -inf only, as the very last element; bit for bit against the oracle."""
+    import time
+    rng = np.random.default_rng(5)
+    n = 1 << 24
+    base = rng.standard_normal(n).astype(dt)
+    cases = {
+        "front": [0], "middle": [n // 2 + 17], "last": [n - 1], "several": [5, n // 3, n - 70000],
+        "chunk_end_then_neg_inf": [n // 2 - 1],
+    }
+    for name, where in cases.items():
+        x = base.copy()
+        x[where] = np.nan
+        if name == "chunk_end_then_neg_inf":
+            x[n // 2:] = -np.inf      # what follows the NaN is -inf only: Max is -inf (not minValue), Min is -inf
+        for fold in ("max", "min"):
+            ref, got = both(H, G, lambda t: getattr(t, fold)(), x)
+            assert np.array_equal(ref, got, equal_nan=True), (name, fold, ref, got)
+        rows = x.reshape(16, n // 16)
+        cols = np.ascontiguousarray(x.reshape(n // 64, 64))
+        for fold in ("maxAxis", "minAxis"):
+            ref, got = both(H, G, lambda t: getattr(t, fold)(1), rows)
+            assert np.array_equal(ref, got, equal_nan=True), (name, fold, "rows")
+            ref, got = both(H, G, lambda t: getattr(t, fold)(0), cols)
+            assert np.array_equal(ref, got, equal_nan=True), (name, fold, "columns")
+    # one NaN in 2^26 elements must not turn the fold into a walk by a single thread (seconds): generous bound
+    big = G.ofNumpy(np.concatenate([base] * 4))
+    big[12345:12346].FillConst(float("nan"))
+    big.max()
+    t0 = time.perf_counter()
+    got = big.max()
+    assert time.perf_counter() - t0 < 0.25
+    assert got == np.concatenate([base] * 4)[12346:].max()
