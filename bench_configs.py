@@ -10,6 +10,7 @@ import numpy as np
 HBM_PEAK_GBS = 8000.0
 FP32_MFMA_PEAK_TFLOPS = 157.3
 FP64_MFMA_PEAK_TFLOPS = 78.6
+BF16_MFMA_PEAK_TFLOPS = 2500.0
 
 
 class Timer:
@@ -64,14 +65,36 @@ def profiled_call_traffic(tag):
     return None
 
 
-def report(log, cfg, name, ms, nbytes=None, flops=None, fp64=False):
-    """One line of the per-configuration table: `frac` is the fraction of the roofline that bounds the call (8 TB/s of HBM for
-    algorithmic bytes, or the fp32 / fp64 matrix peak for a product's FLOPs)."""
+# The matrix pipes a dot kernel can run on: MI355X's dense peak of the instruction the kernel issues, and how many flop it issues
+# per algorithmic flop (the bf16-parts kernels form six bf16 products per multiply-add of the fp32 product).
+MFMA_PIPES = {
+    "bf16x3": {"kernel": "gemm_bf16x3_kernel / gemm_bf16x3_big_kernel", "instruction": "v_mfma_f32_32x32x16_bf16", "peak_TFLOPs": BF16_MFMA_PEAK_TFLOPS, "issue": 6},
+    "fp32": {"kernel": "gemm_kernel<float>", "instruction": "v_mfma_f32_32x32x2_f32", "peak_TFLOPs": FP32_MFMA_PEAK_TFLOPS, "issue": 1},
+    "fp64": {"kernel": "gemm_f64_kernel", "instruction": "v_mfma_f64_16x16x4_f64", "peak_TFLOPs": FP64_MFMA_PEAK_TFLOPS, "issue": 1},
+}
+
+
+def report(log, cfg, name, ms, nbytes=None, flops=None, pipe=None):
+    """One line of the per-configuration table.  `frac` is the fraction of the roofline that bounds the call: 8 TB/s of HBM for
+    algorithmic bytes, or, for a product, the flop its kernel issues over the dense peak of the matrix instruction it issues them on
+    (`pipe`).  The product's own rate (2 M N K over time) is reported beside it, with its ratio to the fp32 matrix peak for
+    single-precision products whatever instruction computed them."""
     if flops:
+        p = MFMA_PIPES[pipe]
         tf = flops / (ms * 1e-3) / 1e12
-        peak = FP64_MFMA_PEAK_TFLOPS if fp64 else FP32_MFMA_PEAK_TFLOPS
-        log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {tf:8.2f} TFLOP/s  {100 * tf / peak:5.1f}% of {'fp64' if fp64 else 'fp32'} MFMA peak")
-        return {"cfg": cfg, "op": name, "us": round(ms * 1e3, 2), "flops": int(flops), "TFLOPs": round(tf, 2), "bound": "mfma", "frac": round(tf / peak, 4)}
+        issued = flops * p["issue"]
+        tf_issued = issued / (ms * 1e-3) / 1e12
+        frac = tf_issued / p["peak_TFLOPs"]
+        row = {"cfg": cfg, "op": name, "us": round(ms * 1e3, 2), "flops": int(flops), "TFLOPs": round(tf, 2), "bound": "mfma",
+               "kernel": p["kernel"], "instruction": p["instruction"], "flops_issued": int(issued), "issued_TFLOPs": round(tf_issued, 1),
+               "peak_TFLOPs": p["peak_TFLOPs"], "frac": round(frac, 4)}
+        extra = ""
+        if pipe in ("bf16x3", "fp32"):
+            row["x_fp32_mfma_peak"] = round(tf / FP32_MFMA_PEAK_TFLOPS, 4)   # a speed figure, not a roofline fraction
+            extra = f"  (product rate = {tf / FP32_MFMA_PEAK_TFLOPS:4.2f} x fp32 MFMA peak)"
+        log(f"[cfg{cfg}] {name:38s} {ms * 1e3:9.1f} us  {tf:7.2f} TFLOP/s  issues {tf_issued:7.1f} TFLOP/s on {p['instruction']} = "
+            f"{100 * frac:5.1f}% of its {p['peak_TFLOPs']:.1f} peak{extra}")
+        return row
     gb = nbytes / (ms * 1e-3) / 1e9
     log(f"[cfg{cfg}] {name:34s} {ms * 1e3:9.1f} us  {gb:8.1f} GB/s  {100 * gb / HBM_PEAK_GBS:5.1f}% of HBM peak  ({nbytes / 1e6:.1f} MB)")
     row = {"cfg": cfg, "op": name, "us": round(ms * 1e3, 2), "bytes": int(nbytes), "GBps": round(gb, 1), "bound": "hbm", "frac": round(gb / HBM_PEAK_GBS, 4)}
@@ -121,12 +144,22 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6), fp32_folds=True, reference_dot_shapes
     def new(shape, dt):
         return Tensor.new(shape, G.Dev, dt)
 
-    def timed(cfg, name, nbytes, build, flops=None, reps=20, fp64=False):
+    def timed(cfg, name, nbytes, build, flops=None, reps=20, pipe=None):
         ns = nsets_for(nbytes)
         sets = [build(i) for i in range(ns)]
         ms = T.time(sets, reps=max(reps, ns))
-        results.append(report(log, cfg, name, ms, nbytes, flops, fp64))
+        results.append(report(log, cfg, name, ms, nbytes, flops, pipe))
         keep.clear()
+
+    def timed_dot(cfg, name, nbytes, build, flops, dt):
+        """A product of single-precision operands is timed on both of its kernels: the default (bf16 matrix instruction, three parts
+        per float) and, behind the library's switch, the fp32 matrix instruction."""
+        if dt is np.float64:
+            timed(cfg, name, nbytes, build, flops=flops, pipe="fp64")
+            return
+        timed(cfg, name + " [bf16 parts]", nbytes, build, flops=flops, pipe="bf16x3")
+        with T.native.option("dot_bf16x3", 0):
+            timed(cfg, name + " [fp32 instr]", nbytes, build, flops=flops, pipe="fp32")
 
     f32 = np.float32
     if 1 in which:
@@ -260,8 +293,8 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6), fp32_folds=True, reference_dot_shapes
 
         def mk5():
             return G.ofNumpy(ha), G.ofNumpy(hb), new([Bn, n, n], f32)
-        timed(5, "BatchedMatMatDot 64x512^3 fp32", 3 * N * 4, lambda i: (lambda a, b, c: [("dot", (D(c), D(a), D(b)))])(*mk5()),
-              flops=2.0 * Bn * n ** 3)
+        timed_dot(5, "BatchedMatMatDot 64x512^3 fp32", 3 * N * 4, lambda i: (lambda a, b, c: [("dot", (D(c), D(a), D(b)))])(*mk5()),
+                  2.0 * Bn * n ** 3, f32)
         timed(5, "Tanh [64,512,512]", 2 * N * 4, lambda i: (lambda a, b, c: [("unary", (abi.DNH_TANH, D(c), D(a)))])(*mk5()))
         timed(5, "MaxAxis 2 (rows of 512)", N * 4 + R * 4,
               lambda i: (lambda a, b, c: [("reduce_last_axis", (abi.DNH_MAX, D(new([Bn, n], f32)), D(a)))])(*mk5()))
@@ -288,8 +321,8 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6), fp32_folds=True, reference_dot_shapes
                 sa = G.ofNumpy(rng.standard_normal((sq, sq)).astype(dt))
                 sb = G.ofNumpy(rng.standard_normal((sq, sq)).astype(dt))
                 sc = new([sq, sq], dt)
-                timed(5, f"MatMatDot {sq}^3 {np.dtype(dt).name}", 3 * sq * sq * sz, lambda i: [("dot", (D(sc), D(sa), D(sb)))],
-                      flops=2.0 * sq ** 3, fp64=dt is np.float64)
+                timed_dot(5, f"MatMatDot {sq}^3 {np.dtype(dt).name}", 3 * sq * sq * sz, lambda i: [("dot", (D(sc), D(sa), D(sb)))],
+                          2.0 * sq ** 3, dt)
                 del sa, sb, sc
     if 6 in which:
         # the vector forms of dot (not one of the five configurations; bandwidth-bound)

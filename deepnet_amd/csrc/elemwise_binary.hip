@@ -4,27 +4,6 @@
 
 using namespace dnh;
 
-namespace {
-
-template <template <class> class OpT>
-int32_t run_numeric(int dt, const MapPlan& p, hipStream_t s) {
-    switch (dt) {
-        case DNH_U8: return launch_map(OpT<uint8_t>{}, p, s);
-        case DNH_I8: return launch_map(OpT<int8_t>{}, p, s);
-        case DNH_I16: return launch_map(OpT<int16_t>{}, p, s);
-        case DNH_U16: return launch_map(OpT<uint16_t>{}, p, s);
-        case DNH_I32: return launch_map(OpT<int32_t>{}, p, s);
-        case DNH_U32: return launch_map(OpT<uint32_t>{}, p, s);
-        case DNH_I64: return launch_map(OpT<int64_t>{}, p, s);
-        case DNH_U64: return launch_map(OpT<uint64_t>{}, p, s);
-        case DNH_F32: return launch_map(OpT<float>{}, p, s);
-        case DNH_F64: return launch_map(OpT<double>{}, p, s);
-    }
-    return fail(DNH_ERR_NOT_SUPPORTED, "binary arithmetic op is not defined for %s", dtype_name(dt));
-}
-
-}  // namespace
-
 extern "C" int32_t dnh_binary(int32_t op, const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void* stream) {
     DNH_TRY(ensure_init());
     const DnhTensor* ops[3] = {t, a, b};
@@ -41,8 +20,8 @@ extern "C" int32_t dnh_binary(int32_t op, const DnhTensor* t, const DnhTensor* a
         return launch_map(OpXor{}, p, s);
     }
     switch (op) {
-        case DNH_ADD: return run_numeric<OpAdd>(dt, p, s);
-        case DNH_SUBTRACT: return run_numeric<OpSub>(dt, p, s);
+        case DNH_ADD: return map_numeric<OpAdd>(dt, p, s);
+        case DNH_SUBTRACT: return map_numeric<OpSub>(dt, p, s);
         case DNH_MULTIPLY: case DNH_POWER: return binary_fourth_unit(op, dt, p, s);
         case DNH_DIVIDE: case DNH_MODULO: return binary_second_unit(op, dt, p, s);
         case DNH_MAX_ELEMWISE: case DNH_MIN_ELEMWISE: return binary_third_unit(op, dt, p, s);

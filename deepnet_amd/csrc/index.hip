@@ -431,6 +431,16 @@ __global__ __launch_bounds__(kBinThreads) void bin_apply_kernel(uint32_t* __rest
     }
 }
 
+// Workspace of the binned form for m updates into a table of n elements: the per-workgroup bucket counts, the bucket totals and
+// the sorted pairs.
+constexpr size_t kBinMaxWorkspace = (size_t)1 << 30;   // beyond this the direct kernel is taken (the stream keeps its workspace)
+inline size_t binned_workspace_bytes(int64_t m, int64_t n, size_t* counts_bytes, size_t* totals_bytes) {
+    const size_t nb = (size_t)((n + kBinElems - 1) >> kBinShift), nchunks = (size_t)((m + kBinChunk - 1) / kBinChunk);
+    *counts_bytes = (nb * nchunks * 4 + 255) / 256 * 256;
+    *totals_bytes = (nb * 4 + 255) / 256 * 256;
+    return *counts_bytes + *totals_bytes + (size_t)m * 8;
+}
+
 // Takes the call when it has the binned form's shape and the binned form is the cheaper one; *status then holds its result.
 bool try_scatter_binned(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, hipStream_t stream, int32_t* err,
                         int32_t* status) {
@@ -439,16 +449,20 @@ bool try_scatter_binned(const DnhTensor* t, const DnhTensor* const* idx, int32_t
     if (t->stride[0] != 1 || src->stride[0] != 1 || idx[0]->stride[0] != 1) return false;
     const int64_t n = t->shape[0], m = src->shape[0];
     if (m < (1 << 20) || m > 0x7FFFFFFFLL || n < 1 || n > ((int64_t)kBinMaxBuckets << kBinShift)) return false;
-    // cost model (measured on MI355X): a direct update costs about 40 ps (memory-side read-modify-write); the binned form moves the
-    // table twice and the pairs four and a half times at about 5.5 TB/s, plus three more launches
-    const double direct_us = (double)m * 40e-6, binned_us = ((double)n * 8.0 + (double)m * 36.0) / 5.5e6 + 10.0;
-    if (binned_us >= direct_us) return false;
     const uint32_t nb = (uint32_t)((n + kBinElems - 1) >> kBinShift), nchunks = cdiv(m, kBinChunk);
-    const size_t counts_bytes = ((size_t)nb * nchunks * 4 + 255) / 256 * 256, totals_bytes = ((size_t)nb * 4 + 255) / 256 * 256;
+    size_t counts_bytes, totals_bytes;
+    const size_t ws_bytes = binned_workspace_bytes(m, n, &counts_bytes, &totals_bytes);
+    // cost model (measured on MI355X): a direct update costs about 40 ps (memory-side read-modify-write); the binned form moves the
+    // table twice, the pairs four and a half times and the per-workgroup bucket counts four times (written, scanned in place, read
+    // by the moving pass) at about 5.5 TB/s, plus three more launches
+    const double direct_us = (double)m * 40e-6, binned_us = ((double)n * 8.0 + (double)m * 36.0 + (double)counts_bytes * 4.0) / 5.5e6 + 10.0;
+    if (binned_us >= direct_us || ws_bytes > kBinMaxWorkspace) return false;
     char* ws = nullptr;
     WorkspaceLease lease;
-    *status = workspace(stream, counts_bytes + totals_bytes + (size_t)m * 8, (void**)&ws, lease);
-    if (*status != DNH_OK) return true;
+    if (workspace(stream, ws_bytes, (void**)&ws, lease) != DNH_OK) {
+        last_error().clear();   // the direct kernel needs no memory: take that one
+        return false;
+    }
     uint32_t* counts = (uint32_t*)ws;
     uint32_t* totals = (uint32_t*)(ws + counts_bytes);
     uint2* pairs = (uint2*)(ws + counts_bytes + totals_bytes);
@@ -460,6 +474,284 @@ bool try_scatter_binned(const DnhTensor* t, const DnhTensor* const* idx, int32_t
     hipLaunchKernelGGL(bin_apply_kernel, dim3(nb), dim3(kBinThreads), 0, stream, (uint32_t*)elem_ptr(t), n, nb, (const uint32_t*)totals, (const uint2*)pairs);
     *status = hipGetLastError() == hipSuccess ? DNH_OK : fail(DNH_ERR_HIP, "binned scatter: launch failed");
     return true;
+}
+
+// ---- ordered scatter (floating point) ------------------------------------------------------------------------------------------
+// t[idx[s]] += src[s] for single and double, any ranks and strides.  The reference adds the sources in row-major order
+// (Host/ScalarOps.fs:593-604), so a target element that several sources name receives ((t + s_a) + s_b) + ... in source order, and
+// floating-point addition does not commute with itself: atomics give another order on every run.  Here every target element receives
+// its sources in the reference's order, hence the reference's bits, whatever the duplication:
+//   1. ordered_cells:  cell[s] = row-major position in t that source s names (-1 and the error word when out of range)
+//   2. ordered_count:  per workgroup of kOrdChunk sources, how many fall into each bucket of 2^shift consecutive cells   -> counts
+//   3. bin_colscan, ordered_starts: where each workgroup's share of each bucket starts in the bucket's list             -> counts, starts
+//   4. ordered_move:   each workgroup sorts its sources by (cell, source position) in LDS (bitonic) and appends every bucket's run to
+//                      that bucket's list: a list is ordered by workgroup, then by cell, then by source position
+//   5. ordered_apply:  one workgroup per bucket keeps the bucket's cells in LDS and walks the list in batches of 1024 entries.
+//                      Entries of one cell that are neighbours in a batch form a run, which the thread at its head adds in order;
+//                      runs of one cell that are not neighbours (they come from different workgroups of pass 4) are applied in
+//                      list order: each round the first pending run of a cell claims it (LDS atomic minimum of the position).
+// A table of more than 4096 buckets is processed in slabs of 4096 x 2^shift cells (passes 2-5 per slab).
+constexpr int kOrdThreads = 1024;
+constexpr int kOrdLiBits = 13;
+constexpr uint32_t kOrdChunk = 1u << kOrdLiBits;     // sources per workgroup of passes 2 and 4
+constexpr int kOrdPer = kOrdChunk / kOrdThreads;
+constexpr int kOrdMaxShift = 13;                     // at most 8192 cells of a bucket in LDS
+constexpr uint32_t kOrdMaxBuckets = 4096;
+constexpr uint32_t kOrdNone = 0xFFFFFFFFu;
+
+__global__ __launch_bounds__(kBlock) void ordered_cells_kernel(IndexArgs a, uint32_t m, int64_t* __restrict__ cell, int32_t* err) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i >= m) return;
+    uint32_t pos[DNH_MAX_DIMS];
+    (void)unravel(a.iter, i, pos);
+    int64_t c = 0;
+    bool ok = true;
+    for (int d = 0; d < a.other.nd; d++) {
+        int64_t j;
+        if (a.idx[d]) {
+            int64_t io = 0;
+            for (int e = 0; e < a.iter.nd; e++) io += (int64_t)pos[e] * a.idx_stride[d][e];
+            j = a.idx[d][io];
+        } else {
+            j = pos[d];
+        }
+        ok = ok && j >= 0 && j < a.other_shape[d];
+        c = c * a.other_shape[d] + j;
+    }
+    if (!ok) *err = 1;
+    cell[i] = ok ? c : -1;
+}
+
+__global__ __launch_bounds__(kOrdThreads) void ordered_count_kernel(const int64_t* __restrict__ cell, uint32_t m, int64_t lo, int64_t hi, int shift,
+                                                                    uint32_t nb, uint32_t* __restrict__ counts) {
+    extern __shared__ uint32_t ord_hist[];   // nb counters
+    for (uint32_t b = threadIdx.x; b < nb; b += kOrdThreads) ord_hist[b] = 0;
+    const uint32_t i0 = blockIdx.x * kOrdChunk;
+    int64_t c[kOrdPer];
+#pragma unroll
+    for (int e = 0; e < kOrdPer; e++) {
+        const uint32_t i = i0 + e * kOrdThreads + threadIdx.x;
+        c[e] = i < m ? cell[i] : -1;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < kOrdPer; e++)
+        if (c[e] >= lo && c[e] < hi) atomicAdd(&ord_hist[(uint32_t)((c[e] - lo) >> shift)], 1u);
+    __syncthreads();
+    for (uint32_t b = threadIdx.x; b < nb; b += kOrdThreads) counts[(size_t)blockIdx.x * nb + b] = ord_hist[b];
+}
+
+// starts[b] = totals[0] + .. + totals[b - 1], one workgroup
+__global__ __launch_bounds__(kOrdThreads) void ordered_starts_kernel(const uint32_t* __restrict__ totals, uint32_t* __restrict__ starts, uint32_t nb) {
+    constexpr int PER = kOrdMaxBuckets / kOrdThreads;
+    __shared__ uint32_t wave_sum[kOrdThreads / 64];
+    uint32_t v[PER], sum = 0, total;
+#pragma unroll
+    for (int e = 0; e < PER; e++) {
+        const uint32_t b = threadIdx.x * PER + e;
+        v[e] = b < nb ? totals[b] : 0u;
+        sum += v[e];
+    }
+    uint32_t run = bin_block_scan(sum, &total, wave_sum);
+#pragma unroll
+    for (int e = 0; e < PER; e++) {
+        const uint32_t b = threadIdx.x * PER + e;
+        if (b < nb) starts[b] = run;
+        run += v[e];
+    }
+}
+
+template <class X>
+__global__ __launch_bounds__(kOrdThreads) void ordered_move_kernel(const int64_t* __restrict__ cell, const X* __restrict__ src, Lay slay, uint32_t m,
+                                                                   int64_t lo, int64_t hi, int shift, uint32_t nb,
+                                                                   const uint32_t* __restrict__ counts, const uint32_t* __restrict__ starts,
+                                                                   uint32_t* __restrict__ pc, X* __restrict__ pv) {
+    extern __shared__ __align__(16) unsigned char ord_lds[];
+    uint64_t* keys = reinterpret_cast<uint64_t*>(ord_lds);            // (cell - lo) << 13 | position in the chunk; all ones = not in this slab
+    X* vals = reinterpret_cast<X*>(keys + kOrdChunk);                  // by position in the chunk
+    uint32_t* gstart = reinterpret_cast<uint32_t*>(vals + kOrdChunk);  // where each bucket's run starts among the sorted keys
+    const uint32_t i0 = blockIdx.x * kOrdChunk;
+#pragma unroll
+    for (int e = 0; e < kOrdPer; e++) {
+        const uint32_t li = e * kOrdThreads + threadIdx.x, i = i0 + li;
+        const int64_t c = i < m ? cell[i] : -1;
+        keys[li] = (c >= lo && c < hi) ? (((uint64_t)(c - lo) << kOrdLiBits) | li) : ~0ull;
+        vals[li] = i < m ? src[offset_of(slay, i)] : X(0);
+    }
+    __syncthreads();
+    // bitonic sort, ascending (keys are distinct except for the all-ones ones, which end up last)
+    for (uint32_t k = 2; k <= kOrdChunk; k <<= 1) {
+        for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+#pragma unroll
+            for (int e = 0; e < kOrdPer / 2; e++) {
+                const uint32_t t = e * kOrdThreads + threadIdx.x;
+                const uint32_t i = ((t & ~(j - 1u)) << 1) | (t & (j - 1u)), l = i | j;
+                const bool up = (i & k) == 0;
+                const uint64_t x = keys[i], y = keys[l];
+                if ((x > y) == up) {
+                    keys[i] = y;
+                    keys[l] = x;
+                }
+            }
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < kOrdPer; e++) {
+        const uint32_t k = e * kOrdThreads + threadIdx.x;
+        const uint64_t key = keys[k];
+        if (key != ~0ull) {
+            const uint32_t b = (uint32_t)((key >> kOrdLiBits) >> shift);
+            if (k == 0 || (uint32_t)((keys[k - 1] >> kOrdLiBits) >> shift) != b) gstart[b] = k;
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int e = 0; e < kOrdPer; e++) {
+        const uint32_t k = e * kOrdThreads + threadIdx.x;
+        const uint64_t key = keys[k];
+        if (key != ~0ull) {
+            const uint64_t cl = key >> kOrdLiBits;
+            const uint32_t b = (uint32_t)(cl >> shift);
+            const uint32_t dst = starts[b] + counts[(size_t)blockIdx.x * nb + b] + (k - gstart[b]);
+            pc[dst] = (uint32_t)(cl & ((1u << shift) - 1u));
+            pv[dst] = vals[(uint32_t)key & (kOrdChunk - 1u)];
+        }
+    }
+}
+
+// element offset of row-major position i of a layout (positions beyond 2^32 included)
+__device__ __forceinline__ int64_t offset_of64(const Lay& l, int64_t i) {
+    int64_t off = 0;
+    for (int d = l.nd - 1; d >= 0; d--) {
+        const int64_t q = (d == 0) ? 0 : i / (int64_t)l.shape[d];
+        off += (i - q * (int64_t)l.shape[d]) * l.stride[d];
+        i = q;
+    }
+    return off;
+}
+
+template <class X>
+__global__ __launch_bounds__(kOrdThreads) void ordered_apply_kernel(X* __restrict__ t, Lay tlay, int dense, int64_t lo, int64_t ncells, int shift,
+                                                                    const uint32_t* __restrict__ totals, const uint32_t* __restrict__ starts,
+                                                                    const uint32_t* __restrict__ pc, const X* __restrict__ pv) {
+    extern __shared__ __align__(16) unsigned char ord_lds[];
+    const uint32_t cells = 1u << shift;
+    X* acc = reinterpret_cast<X*>(ord_lds);                         // the bucket's cells
+    X* bv = acc + cells;                                            // the batch: values
+    uint32_t* claim = reinterpret_cast<uint32_t*>(bv + kOrdThreads); // per cell: position in the batch of the first pending run, or kOrdNone
+    uint32_t* bc = claim + cells;                                   // the batch: cells (inside the bucket)
+    const uint32_t b = blockIdx.x;
+    const uint32_t cnt = totals[b];
+    if (cnt == 0) return;   // uniform: nothing lands in this bucket
+    const int64_t c0 = lo + ((int64_t)b << shift);
+    const uint32_t len = (uint32_t)((ncells - c0) < (int64_t)cells ? (ncells - c0) : (int64_t)cells);
+    for (uint32_t x = threadIdx.x; x < len; x += kOrdThreads) {
+        acc[x] = t[dense ? c0 + x : offset_of64(tlay, c0 + x)];
+        claim[x] = kOrdNone;
+    }
+    const uint32_t p0 = starts[b];
+    for (uint32_t base = 0; base < cnt; base += kOrdThreads) {
+        const uint32_t nbat = cnt - base < (uint32_t)kOrdThreads ? cnt - base : (uint32_t)kOrdThreads;
+        uint32_t c = 0;
+        if (threadIdx.x < nbat) {
+            c = pc[p0 + base + threadIdx.x];
+            bc[threadIdx.x] = c;
+            bv[threadIdx.x] = pv[p0 + base + threadIdx.x];
+        }
+        __syncthreads();   // the batch (and, the first time, the cells) are in LDS
+        bool pending = threadIdx.x < nbat && (threadIdx.x == 0 || bc[threadIdx.x - 1] != c);   // head of a run
+        for (;;) {
+            if (pending) atomicMin(&claim[c], threadIdx.x);
+            __syncthreads();
+            if (pending && claim[c] == threadIdx.x) {
+                X a = acc[c];
+                for (uint32_t k = threadIdx.x; k < nbat && bc[k] == c; k++) a = a + bv[k];
+                acc[c] = a;
+                claim[c] = kOrdNone;
+                pending = false;
+            }
+            if (!__syncthreads_or((int)pending)) break;
+        }
+    }
+    __syncthreads();
+    for (uint32_t x = threadIdx.x; x < len; x += kOrdThreads) t[dense ? c0 + x : offset_of64(tlay, c0 + x)] = acc[x];
+}
+
+// Workspace of the ordered scatter of m sources into ncells cells with buckets of 2^shift cells.
+struct OrderedPlan {
+    int shift;
+    uint32_t nb_max, nchunks;
+    size_t cell_bytes, counts_bytes, totals_bytes, pc_bytes, pv_bytes, total;
+};
+inline OrderedPlan ordered_plan(int64_t m, int64_t ncells, int esize) {
+    OrderedPlan p;
+    int lg = 0;
+    while (((int64_t)1 << lg) < ncells) lg++;
+    p.shift = lg - 10 < 4 ? 4 : (lg - 10 > kOrdMaxShift ? kOrdMaxShift : lg - 10);   // about a thousand buckets where the table allows
+    const int64_t buckets = (ncells + ((int64_t)1 << p.shift) - 1) >> p.shift;
+    p.nb_max = (uint32_t)(buckets < (int64_t)kOrdMaxBuckets ? buckets : (int64_t)kOrdMaxBuckets);
+    p.nchunks = (uint32_t)((m + kOrdChunk - 1) / kOrdChunk);
+    auto up = [](size_t b) { return (b + 255) / 256 * 256; };
+    p.cell_bytes = up((size_t)m * 8);
+    p.counts_bytes = up((size_t)p.nb_max * p.nchunks * 4);
+    p.totals_bytes = up((size_t)p.nb_max * 4);
+    p.pc_bytes = up((size_t)m * 4);
+    p.pv_bytes = up((size_t)m * (size_t)esize);
+    p.total = p.cell_bytes + p.counts_bytes + 2 * p.totals_bytes + p.pc_bytes + p.pv_bytes;
+    return p;
+}
+
+template <class X>
+int32_t scatter_ordered(const DnhTensor* t, const DnhTensor* src, const IndexArgs& a, hipStream_t stream, int32_t* err) {
+    const int64_t m = nelems(src), ncells = nelems(t);
+    const OrderedPlan p = ordered_plan(m, ncells, (int)sizeof(X));
+    char* ws = nullptr;
+    WorkspaceLease lease;
+    const int32_t st = workspace(stream, p.total, (void**)&ws, lease);
+    if (st != DNH_OK)
+        return fail(st, "dnh_scatter: no memory for the %zu-byte workspace of the ordered floating-point scatter (dnh_set_option(\"scatter_fp_atomic\", 1) "
+                        "selects the atomic form, which needs none)", p.total);
+    int64_t* cell = (int64_t*)ws;
+    uint32_t* counts = (uint32_t*)(ws + p.cell_bytes);
+    uint32_t* totals = (uint32_t*)(ws + p.cell_bytes + p.counts_bytes);
+    uint32_t* starts = (uint32_t*)(ws + p.cell_bytes + p.counts_bytes + p.totals_bytes);
+    uint32_t* pc = (uint32_t*)(ws + p.cell_bytes + p.counts_bytes + 2 * p.totals_bytes);
+    X* pv = (X*)(ws + p.cell_bytes + p.counts_bytes + 2 * p.totals_bytes + p.pc_bytes);
+    const size_t move_lds = (size_t)kOrdChunk * (8 + sizeof(X)) + (size_t)p.nb_max * 4;
+    const size_t apply_lds = ((size_t)1 << p.shift) * (sizeof(X) + 4) + (size_t)kOrdThreads * (sizeof(X) + 4);
+    static const hipError_t attr_move = hipFuncSetAttribute(reinterpret_cast<const void*>(&ordered_move_kernel<X>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                            (int)((size_t)kOrdChunk * (8 + sizeof(X)) + (size_t)kOrdMaxBuckets * 4));
+    static const hipError_t attr_apply = hipFuncSetAttribute(reinterpret_cast<const void*>(&ordered_apply_kernel<X>), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                             (int)(((size_t)1 << kOrdMaxShift) * (sizeof(X) + 4) + (size_t)kOrdThreads * (sizeof(X) + 4)));
+    if (attr_move != hipSuccess || attr_apply != hipSuccess) return fail(DNH_ERR_HIP, "dnh_scatter: cannot size the LDS of the ordered scatter");
+    // the target's cells in row-major order lie one after the other in memory?
+    int dense = 1;
+    {
+        int64_t expect = 1;
+        for (int d = t->ndims - 1; d >= 0; d--) {
+            if (t->shape[d] != 1 && t->stride[d] != expect) dense = 0;
+            expect *= t->shape[d];
+        }
+    }
+    const Lay slay = lay_of(src), tlay = lay_of(t);
+    X* tp = (X*)elem_ptr(t);
+    hipLaunchKernelGGL(ordered_cells_kernel, dim3(cdiv(m, kBlock)), dim3(kBlock), 0, stream, a, (uint32_t)m, cell, err);
+    DNH_LAUNCH_CHECK();
+    const int64_t slab = (int64_t)kOrdMaxBuckets << p.shift;
+    for (int64_t lo = 0; lo < ncells; lo += slab) {
+        const int64_t hi = lo + slab < ncells ? lo + slab : ncells;
+        const uint32_t nb = (uint32_t)((hi - lo + ((int64_t)1 << p.shift) - 1) >> p.shift);
+        hipLaunchKernelGGL(ordered_count_kernel, dim3(p.nchunks), dim3(kOrdThreads), nb * 4, stream, (const int64_t*)cell, (uint32_t)m, lo, hi, p.shift, nb, counts);
+        hipLaunchKernelGGL(bin_colscan_kernel, dim3(cdiv(nb, 64)), dim3(kBinThreads), 0, stream, counts, totals, nb, p.nchunks);
+        hipLaunchKernelGGL(ordered_starts_kernel, dim3(1), dim3(kOrdThreads), 0, stream, (const uint32_t*)totals, starts, nb);
+        hipLaunchKernelGGL((ordered_move_kernel<X>), dim3(p.nchunks), dim3(kOrdThreads), move_lds, stream, (const int64_t*)cell, (const X*)elem_ptr(src), slay,
+                           (uint32_t)m, lo, hi, p.shift, nb, (const uint32_t*)counts, (const uint32_t*)starts, pc, pv);
+        hipLaunchKernelGGL((ordered_apply_kernel<X>), dim3(nb), dim3(kOrdThreads), apply_lds, stream, tp, tlay, dense, lo, ncells, p.shift,
+                           (const uint32_t*)totals, (const uint32_t*)starts, (const uint32_t*)pc, (const X*)pv);
+        DNH_LAUNCH_CHECK();
+    }
+    return DNH_OK;
 }
 
 __global__ __launch_bounds__(kBlock) void compact_count_kernel(MaskArgs m, uint32_t n, uint32_t* counts) {
@@ -935,6 +1227,8 @@ extern "C" int32_t dnh_scatter(const DnhTensor* t, const DnhTensor* const* idx, 
     DNH_TRY(error_flag_ptr(s, &eflag));
     int32_t bst = DNH_OK;
     if (try_scatter_binned(t, idx, n_idx, src, s, eflag, &bst)) return bst;
+    if (dtype_is_fp(t->dtype) && option(OPT_SCATTER_FP_ATOMIC) == 0 && nelems(t) > 0)   // (an empty target: every index is out of range)
+        return t->dtype == DNH_F32 ? scatter_ordered<float>(t, src, a, s, eflag) : scatter_ordered<double>(t, src, a, s, eflag);
     const dim3 grid(cdiv(n, kBlock));
 #define CASE(DT, X) case DT: hipLaunchKernelGGL(scatter_kernel<X>, grid, dim3(kBlock), 0, s, (X*)elem_ptr(t), (const X*)elem_ptr(src), a, (uint32_t)n, eflag); break;
     switch (t->dtype) {

@@ -1087,7 +1087,25 @@ int32_t launch_map(const Op& op, const MapPlan& p, hipStream_t stream) {
 }
 
 // The arithmetic and comparison entry points are spread over four and two translation units (the element-wise instantiations dominate
-// the library's build time, and the units compile side by side); these take the ops of the second unit.
+// the library's build time, and the units compile side by side).
+// map_numeric: a binary arithmetic op OpT on every numeric element type; each unit instantiates it for its own ops.
+template <template <class> class OpT>
+int32_t map_numeric(int dt, const MapPlan& p, hipStream_t s) {
+    switch (dt) {
+        case DNH_U8: return launch_map(OpT<uint8_t>{}, p, s);
+        case DNH_I8: return launch_map(OpT<int8_t>{}, p, s);
+        case DNH_I16: return launch_map(OpT<int16_t>{}, p, s);
+        case DNH_U16: return launch_map(OpT<uint16_t>{}, p, s);
+        case DNH_I32: return launch_map(OpT<int32_t>{}, p, s);
+        case DNH_U32: return launch_map(OpT<uint32_t>{}, p, s);
+        case DNH_I64: return launch_map(OpT<int64_t>{}, p, s);
+        case DNH_U64: return launch_map(OpT<uint64_t>{}, p, s);
+        case DNH_F32: return launch_map(OpT<float>{}, p, s);
+        case DNH_F64: return launch_map(OpT<double>{}, p, s);
+    }
+    return fail(DNH_ERR_NOT_SUPPORTED, "binary arithmetic op is not defined for %s", dtype_name(dt));
+}
+
 int32_t binary_second_unit(int32_t op, int dt, const MapPlan& p, hipStream_t s);    // Divide, Modulo
 int32_t binary_third_unit(int32_t op, int dt, const MapPlan& p, hipStream_t s);     // MaxElemwise, MinElemwise
 int32_t binary_fourth_unit(int32_t op, int dt, const MapPlan& p, hipStream_t s);    // Multiply, Power

@@ -26,6 +26,15 @@ type Cfg private () =
         with get () = stacktrace.Value
         and set v = stacktrace.Value <- v
 
+    /// Tuning switches of the native library (dnh_set_option: which kernel computes a result, never its contract), e.g.
+    /// Cfg.SetOption ("dot_bf16x3", 0) keeps single-precision products on the fp32 matrix instruction.
+    static member SetOption (name: string, value: int) =
+        Native.check (Native.dnh_set_option (System.Text.Encoding.ASCII.GetBytes (name + "\000"), value))
+    static member GetOption (name: string) : int =
+        let mutable v = 0
+        Native.check (Native.dnh_get_option (System.Text.Encoding.ASCII.GetBytes (name + "\000"), &v))
+        v
+
 module internal Desc =
     let dtypeOf (t: Type) =
         if   t = typeof<bool>   then DType.Bool elif t = typeof<byte>   then DType.U8  elif t = typeof<sbyte>  then DType.I8

@@ -68,6 +68,9 @@ module internal Native =
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_init (int device)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_last_error (byte[] buf, unativeint n)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_async_error (nativeint stream, int& code)
+    // option names cross as NUL-terminated ASCII bytes
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_set_option (byte[] name, int value)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_get_option (byte[] name, int& value)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_alloc (unativeint bytes, nativeint& ptr)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_free (nativeint ptr)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_alloc_async (unativeint bytes, nativeint stream, nativeint& ptr)

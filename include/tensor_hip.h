@@ -259,7 +259,13 @@ int32_t dnh_find_last_axis(const void* value, const DnhTensor* t_i64, const DnhT
  * stream's error flag (dnh_async_error) and leaves the target element unwritten; it never faults the device. */
 int32_t dnh_gather(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, void* stream);
 /* ITensorBackend.Scatter (TensorBackend.fs:120; Host/ScalarOps.fs:593-604): t[idx[s]] += src[s]; the frontend
- * zero-fills t first (Tensor.fs:2159).  idx has t->ndims entries broadcast to src's shape. */
+ * zero-fills t first (Tensor.fs:2159).  idx has t->ndims entries broadcast to src's shape.
+ * Repeated indices: integer sums wrap and are the same in any order.  Single and double: every target element receives its sources
+ * one after the other in the row-major order of src, which is the order of the reference's loop, so the result has the reference's
+ * bits and is the same on every run (the sources are sorted by target element first; workspace of about 20 bytes per source element,
+ * DNH_ERR_OUT_OF_MEMORY when it cannot be had).  dnh_set_option("scatter_fp_atomic", 1) selects float atomics instead: no workspace,
+ * faster for few repeats, but the order of a cell's additions then varies from run to run; either way a target element that m_j
+ * sources name is within m_j u sum|src_s| of the exact sum (u = unit roundoff). */
 int32_t dnh_scatter(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, void* stream);
 /* ITensorBackend.CountTrue is dnh_reduce_last_axis(DNH_COUNT_TRUE).
  * ITensorBackend.MaskedGet (TensorBackend.fs:121; Host/ScalarOps.fs:667-681): masks has src->ndims entries, each NULL

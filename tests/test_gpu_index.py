@@ -64,6 +64,110 @@ def test_scatter_fp_unique(H, G, rng, dt):
     assert_exact(ref, got)
 
 
+def _wide(rng, m, dt):
+    """Values spread over twelve decades, both signs: the order of a cell's additions shows in the last bits of its sum."""
+    return (rng.standard_normal(m) * 10.0 ** rng.uniform(-6, 6, m)).astype(dt)
+
+
+def _check_fp_scatter_bound(got, idx, src, n, dt):
+    """Stated bound of floating-point scatter (either form): a cell that m_j sources name is within m_j u sum|src_s| of the exact sum."""
+    exact = np.zeros(n, np.float64)
+    np.add.at(exact, idx, src.astype(np.float64))
+    mag = np.zeros(n, np.float64)
+    np.add.at(mag, idx, np.abs(src.astype(np.float64)))
+    cnt = np.bincount(idx, minlength=n).astype(np.float64)
+    u = np.finfo(dt).eps / 2
+    assert np.all(np.abs(got.astype(np.float64) - exact) <= cnt * u * mag)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+@pytest.mark.parametrize("m,n,kind", [
+    (50_000, 777, "dup"),                      # about 64 sources per cell
+    (70_000, 1, "dup"),                        # one cell takes everything: one run per batch
+    (200_000, 5, "dup"),
+    ((1 << 20) + 123, 300_000, "dup"),         # many workgroups feed every bucket
+    (3 << 20, 5_000_000, "skewed"),            # most sources land in a few buckets, many buckets stay empty
+    (8191, 100_000, "dup"), (8193, 9000, "dup"), (1, 10, "dup"),
+    (1 << 20, 40_000_000, "dup"),              # a table of more than 4096 buckets: two slabs
+])
+def test_scatter_fp_with_duplicates_adds_in_source_order(H, G, rng, dt, m, n, kind):
+    """Floating-point scatter with repeated indices: every cell receives its sources in row-major source order, as the reference's
+    loop adds them, so the sums agree bit for bit with the oracle and with NumPy's unbuffered np.add.at (which is specified to apply
+    the updates one after the other), and two runs give the same bits."""
+    if kind == "skewed":
+        idx = np.where(rng.random(m) < 0.9, rng.integers(0, 40_000, m), rng.integers(0, n, m)).astype(np.int64)
+    else:
+        idx = rng.integers(0, n, m).astype(np.int64)
+    src = _wide(rng, m, dt)
+    ref, got = both(H, G, lambda s, i: type(s).scatter([i], [n], s), src, idx)
+    assert_exact(ref, got)
+    exp = np.zeros(n, dtype=dt)
+    np.add.at(exp, idx, src)
+    assert_exact(exp, got)
+    again = G.toNumpy(type(G.ofNumpy(src)).scatter([G.ofNumpy(idx)], [n], G.ofNumpy(src)))
+    assert_exact(got, again)
+    _check_fp_scatter_bound(got, idx, src, n, dt)
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_scatter_fp_layouts_existing_values_and_bad_indices(H, G, rng, dt):
+    """The ordered form on everything the entry point accepts: index tensors per dimension, a strided (transposed) source, a target
+    that is a strided view holding values already, identity dimensions, out-of-range indices (reported, skipped, the rest lands)."""
+    src = _wide(rng, 300 * 200, dt).reshape(300, 200)
+    i0 = rng.integers(0, 50, (300, 200)).astype(np.int64)
+    i1 = rng.integers(0, 60, (300, 200)).astype(np.int64)
+    ref, got = both(H, G, lambda s, a, b: type(s).scatter([a, b], [50, 60], s), src, i0, i1)
+    assert_exact(ref, got)
+    exp = np.zeros((50, 60), dt)
+    np.add.at(exp, (i0, i1), src)
+    assert_exact(exp, got)
+    # transposed source and index views (row-major order of the VIEW is the order of the additions)
+    ref, got = both(H, G, lambda s, a, b: type(s).scatter([a.T, b.T], [50, 60], s.T), src, i0, i1)
+    assert_exact(ref, got)
+    exp = np.zeros((50, 60), dt)
+    np.add.at(exp, (i0.T, i1.T), src.T)
+    assert_exact(exp, got)
+    # identity on dimension 0 (None), an index tensor for dimension 1
+    j1 = rng.integers(0, 7, (300, 200)).astype(np.int64)
+    ref, got = both(H, G, lambda s, b: type(s).scatter([None, b], [300, 7], s), src, j1)
+    assert_exact(ref, got)
+    # a strided target view with values in it
+    before = _wide(rng, 3 * 1000, dt).reshape(1000, 3)
+    idx = rng.integers(0, 1000, 20000).astype(np.int64)
+    vals = _wide(rng, 20000, dt)
+    exp = before.copy()
+    np.add.at(exp[:, 1], idx, vals)
+    for mod in (H, G):
+        t = mod.ofNumpy(before)
+        view = t[:, 1]                                         # one column: stride 3
+        view.Backend.Scatter(view, [mod.ofNumpy(idx)], mod.ofNumpy(vals))
+        assert_exact(exp, mod.toNumpy(t))
+    # indices outside the table
+    bad = idx.copy()
+    bad[[5, 7000, 19999]] = [1000, -1, 2 ** 40]
+    t2 = G.zeros([1000], dt)
+    with pytest.raises(IndexError):
+        t2.Backend.Scatter(t2, [G.ofNumpy(bad)], G.ofNumpy(vals))
+    keep = np.ones(20000, bool)
+    keep[[5, 7000, 19999]] = False
+    exp2 = np.zeros(1000, dt)
+    np.add.at(exp2, idx[keep], vals[keep])
+    assert_exact(exp2, G.toNumpy(t2))
+
+
+@pytest.mark.parametrize("dt", [np.float32, np.float64])
+def test_scatter_fp_atomic_form_behind_the_switch(G, rng, dt):
+    """dnh_set_option("scatter_fp_atomic", 1) selects float atomics: the order of a cell's additions then varies from run to run, the
+    stated bound still holds."""
+    from deepnet_amd import native
+    m, n = 300_000, 5000
+    idx = rng.integers(0, n, m).astype(np.int64)
+    src = _wide(rng, m, dt)
+    with native.option("scatter_fp_atomic", 1):
+        got = G.toNumpy(type(G.ofNumpy(src)).scatter([G.ofNumpy(idx)], [n], G.ofNumpy(src)))
+    _check_fp_scatter_bound(got, idx, src, n, dt)
+
+
 @pytest.mark.parametrize("dt", [np.int32, np.uint32])
 @pytest.mark.parametrize("m,n,kind", [
     ((1 << 20) + 123, 300_000, "dup"),         # many updates per element; table not a whole number of buckets
