@@ -12,8 +12,10 @@ the largest share of the step.  Consecutive ops read different 256 MiB tensors s
 serve re-reads.  `cpu_baseline` times the CPU oracle (oracle/hostref.cpp, the HostTensor restatement) on the same step.
 `configs` carries the other benchmark configurations (element-wise chain, permuted + broadcast add, double-precision
 folds, integer / bool indexing, batched dot + softmax pieces): one entry per backend call with its algorithmic bytes or
-FLOPs, the mean of >= 20 event-timed launches over rotated buffer sets and the fraction of 8 TB/s or of the fp32 / fp64
-matrix peak; `config_summary` aggregates them per configuration.  They are measured after the timed region.
+FLOPs, the mean of >= 20 event-timed launches over rotated buffer sets and the fraction of 8 TB/s or, for a product, the flop
+its kernel issues over the dense peak of the matrix instruction it issues them on (single-precision products are timed on both
+of their kernels: bf16 matrix instruction with three parts per float, and fp32 matrix instruction); `config_summary` aggregates
+them per configuration.  They are measured after the timed region.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-configs] [--all] [--no-cpu]
 """
@@ -32,21 +34,41 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0        # MI355X HBM3E, vendor figure
 FP32_MFMA_PEAK_TFLOPS = 157.3
 # HBM bytes per launch of the dominant kernel are not measured by this program: they come from two rocprofv3 --pmc runs of it
-# (FETCH_SIZE, WRITE_SIZE), whose committed summary carries a line "traffic_bytes_per_launch <op> <bytes>".
+# (FETCH_SIZE, WRITE_SIZE), whose committed summary carries a line
+#   traffic_bytes_per_launch <op> <bytes> kernel=<kernel symbol without blanks> sources=<sha256[:16] of the kernel's source files>
+# The figure is reported only while it still describes the kernel this program times: same kernel symbol, same source text.
 TRAFFIC_PROFILE = os.path.join("profiles", "bench_headline_fp32_8192x8192.txt")
+KERNEL_SOURCES = {   # op -> the files whose text makes up its kernel
+    "Add": ["deepnet_amd/csrc/map_kernels.h", "deepnet_amd/csrc/ops.h", "deepnet_amd/csrc/elemwise_binary.hip"],
+}
 
 
-def profiled_traffic(op_name):
-    """(bytes, source file) of the committed counter summary for `op_name`, or (None, None) when there is none."""
+def kernel_source_hash(op_name):
+    import hashlib
+    h = hashlib.sha256()
+    for rel in KERNEL_SOURCES.get(op_name, []):
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def profiled_traffic(op_name, kernel_symbol):
+    """(bytes, source file, note) of the committed counter summary for `op_name`; bytes is None when there is no summary or when
+    it was taken from another kernel or another version of the kernel's sources (the note then says which)."""
     try:
         with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
             for line in f:
                 parts = line.split()
-                if len(parts) == 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == op_name:
-                    return int(parts[2]), TRAFFIC_PROFILE
+                if len(parts) >= 3 and parts[0] == "traffic_bytes_per_launch" and parts[1] == op_name:
+                    tags = dict(p.split("=", 1) for p in parts[3:] if "=" in p)
+                    if tags.get("kernel") != kernel_symbol.replace(" ", ""):
+                        return None, TRAFFIC_PROFILE, f"stale: profiled kernel {tags.get('kernel')} is not {kernel_symbol}"
+                    if tags.get("sources") != kernel_source_hash(op_name):
+                        return None, TRAFFIC_PROFILE, "stale: the kernel's source files changed after the counters were read"
+                    return int(parts[2]), TRAFFIC_PROFILE, None
     except OSError:
         pass
-    return None, None
+    return None, None, "no committed counter summary"
 
 
 def log(*a):
@@ -56,8 +78,9 @@ def log(*a):
 class Op:
     """One backend call with prebuilt descriptors: fn(lib_or_oracle) issues it; `bytes` is its algorithmic traffic."""
 
-    def __init__(self, name, kernel, entry, args, nbytes, flops=0):
+    def __init__(self, name, kernel, entry, args, nbytes, flops=0, symbol=None):
         self.name, self.kernel, self.entry, self.args, self.bytes, self.flops = name, kernel, entry, args, nbytes, flops
+        self.symbol = symbol or kernel   # the kernel's symbol as rocprofv3 prints it
         self.ms = []
         self.timed_ms = []
 
@@ -95,7 +118,7 @@ def make_ops(mod, rng_seed=123, n=8192):
 
     s4 = 4
     ops = [
-        Op("Add", "map_flat", "binary", (abi.DNH_ADD, D(out_add), D(a), D(b)), 3 * N * s4),
+        Op("Add", "map_flat", "binary", (abi.DNH_ADD, D(out_add), D(a), D(b)), 3 * N * s4, symbol="map_flat_kernel<OpAdd<float>, 4, 1>"),
         Op("Tanh", "map_flat", "unary", (abi.DNH_TANH, D(out_tanh), D(x)), 2 * N * s4),
         Op("SumLastAxis(rows)", "reduce_rows", "reduce_last_axis", (abi.DNH_SUM, D(vec[0]), D(a)), N * s4 + n * s4),
         Op("MaxLastAxis(rows)", "reduce_rows", "reduce_last_axis", (abi.DNH_MAX, D(vec[1]), D(b)), N * s4 + n * s4),
@@ -241,10 +264,13 @@ def main():
     dop = ops[dom_i]
     dom_ms = float(np.mean(dop.timed_ms))
     dom_gbs = dop.bytes / (dom_ms * 1e-3) / 1e9
-    traffic, traffic_src = profiled_traffic(dop.name)
-    roofline = {"bound": "hbm", "kernel": dop.kernel, "op": dop.name, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+    traffic, traffic_src, traffic_note = profiled_traffic(dop.name, dop.symbol)
+    roofline = {"bound": "hbm", "kernel": dop.symbol, "op": dop.name, "achieved": round(dom_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                 "frac": round(dom_gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_src,
                 "avg_launch_ms": round(dom_ms, 5), "algorithmic_bytes": dop.bytes}
+    if traffic_note:
+        roofline["traffic_note"] = traffic_note
+        log(f"[bench] roofline.traffic withheld ({traffic_note})")
     ev_sum = sum(k["avg_ms"] for k in per_kernel)
     log(f"[bench] step: {ms_per_step:.3f} ms wall, {ev_sum:.3f} ms sum of event intervals, {value:.1f} GB/s = {100 * value / HBM_PEAK_GBS:.1f}% of HBM peak")
 

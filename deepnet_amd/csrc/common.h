@@ -66,9 +66,19 @@ public:
 
 private:
     friend int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease);
+    friend int32_t sync_words(hipStream_t stream, size_t bytes, void** out, uint32_t* epoch, WorkspaceLease& lease);
     std::mutex* held_ = nullptr;
 };
 int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& lease);
+// A second per-stream buffer, for the words through which the workgroups of ONE launch meet (arrival counters, tile descriptors).  It is zero when first handed out and is used for nothing else, so kernels may leave it in the state the next
+// launch expects (counters back at zero) and tag what they cannot reset with `epoch`, a number no earlier launch on the stream used
+// (30 bits; the buffer is cleared when it wraps).  Same lease discipline as workspace().
+int32_t sync_words(hipStream_t stream, size_t bytes, void** out, uint32_t* epoch, WorkspaceLease& lease);
+// Layout of that buffer: counters that every launch leaves at zero in front, epoch-tagged words behind them.
+constexpr size_t kSyncCountTop = 64;       // uint64: arrival word of the one-launch CountTrue
+constexpr size_t kSyncCountGroups = 128;   // uint64 x up to kSyncMaxCountGroups: its per-group arrival words
+constexpr size_t kSyncMaxCountGroups = 496;
+constexpr size_t kSyncTileWords = 4096;    // uint64 per tile, epoch-tagged
 
 // ---- tuning switches --------------------------------------------------------------------------------------------------
 // Process-wide integers behind dnh_set_option / dnh_get_option.  Each starts from an environment variable of the same name in
@@ -82,7 +92,9 @@ enum Option {
     OPT_DOT_INT_MFMA,        // 1: 32 / 64-bit integer products on the int8 matrix instruction; 0: gemm_int_kernel
     OPT_TR4,                 // 1: 4-byte transposing copies through LDS where the layout asks for them; 0: the general n-d kernel
     OPT_SCATTER_FP_ATOMIC,   // 0: floating-point scatter adds duplicates in source order (reproducible); 1: float atomics
-    OPT_COMPACT_ONE_PASS,    // 1: maskedGet / trueIndices / countTrue of contiguous masks in one launch; 0: count + move launches
+    OPT_COMPACT_ONE_PASS,    // 1: maskedGet / maskedSet / trueIndices of contiguous masks in one launch; 0: count + move launches
+    OPT_COUNT_ONE_LAUNCH,    // 1: countTrue of a whole contiguous mask in one launch (arrival counters); 0: the general two-pass fold
+    OPT_LOOKBACK_SPINS,      // polls a one-pass compaction's tile spends on predecessors that have not published before it counts for itself
     OPT_COUNT
 };
 int option(Option o);

@@ -163,6 +163,97 @@ int32_t run_arg(const DnhTensor* t, const DnhTensor* s, hipStream_t st, const ch
 
 }  // namespace
 
+// ---- CountTrue of a whole contiguous mask in one launch -----------------------------------------------------------------------------
+// The general fold needs a second, dependent launch to add the workgroups' partial counts.  Integer counts can be added in any order,
+// so here the workgroups meet through device-scope atomics instead: a workgroup adds (count | 1 << 48) to the word of its group of 16
+// workgroups; the one that finds 15 arrivals before it carries the group's sum on to the top word in the same way, and the last
+// arrival there stores the result.  One atomic carries count and arrival together, so no ordering between locations is relied on,
+// and no more than 16 workgroups (or groups) ever meet on one address.  Each last arrival puts its word back to zero for the next launch.
+namespace {
+constexpr int kCountGroup = 16;
+constexpr unsigned long long kCountArrival = 1ull << 48, kCountMask = kCountArrival - 1;
+
+__global__ __launch_bounds__(kBlock) void count_true_kernel(const uint8_t* __restrict__ mask, int64_t n, int64_t per_block, uint32_t nblocks,
+                                                            unsigned long long* top, unsigned long long* groups, int64_t* out) {
+    const int64_t r0 = (int64_t)blockIdx.x * per_block;
+    const int64_t r1 = r0 + per_block < n ? r0 + per_block : n;
+    uint32_t c = 0;
+    // per_block is a multiple of 16 x kBlock and the mask is 4-byte aligned: whole 16-byte pieces, then the last few bytes one by one
+    constexpr int U = 4;
+    int64_t i = r0 + (int64_t)threadIdx.x * 16;
+    for (; i + (U - 1) * kBlock * 16 + 16 <= r1; i += (int64_t)U * kBlock * 16) {
+        Pack<uint32_t, 4> v[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) v[u] = load_pack<uint32_t, 4>((const uint32_t*)(mask + i + (int64_t)u * kBlock * 16));
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const uint32_t x = v[u].v[w];
+                c += ((x & 0xFFu) != 0) + ((x & 0xFF00u) != 0) + ((x & 0xFF0000u) != 0) + ((x & 0xFF000000u) != 0);
+            }
+    }
+    for (; i < r1; i += (int64_t)kBlock * 16) {
+        if (i + 16 <= r1) {
+            const Pack<uint32_t, 4> v = load_pack<uint32_t, 4>((const uint32_t*)(mask + i));
+#pragma unroll
+            for (int w = 0; w < 4; w++) {
+                const uint32_t x = v.v[w];
+                c += ((x & 0xFFu) != 0) + ((x & 0xFF00u) != 0) + ((x & 0xFF0000u) != 0) + ((x & 0xFF000000u) != 0);
+            }
+        } else {
+            for (int64_t j = i; j < r1; j++) c += mask[j] != 0;
+        }
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) c += (uint32_t)__shfl_xor((int)c, m, 64);
+    __shared__ uint32_t part[kBlock / 64];
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = c;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned long long total = 0;
+#pragma unroll
+        for (int w = 0; w < kBlock / 64; w++) total += part[w];
+        const uint32_t g = blockIdx.x / kCountGroup, ngroups = (nblocks + kCountGroup - 1) / kCountGroup;
+        const uint32_t gsize = g + 1 < ngroups ? (uint32_t)kCountGroup : nblocks - g * kCountGroup;
+        const unsigned long long was = __hip_atomic_fetch_add(groups + g, total | kCountArrival, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((was >> 48) == gsize - 1) {
+            const unsigned long long gsum = (was & kCountMask) + total;
+            __hip_atomic_store(groups + g, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const unsigned long long twas = __hip_atomic_fetch_add(top, gsum | kCountArrival, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if ((twas >> 48) == ngroups - 1) {
+                out[0] = (int64_t)((twas & kCountMask) + gsum);
+                __hip_atomic_store(top, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+    }
+}
+
+// Takes CountTrue of one contiguous run of bools into a single int64 when that is worth a launch of its own shape.
+bool try_count_true_one_launch(const DnhTensor* t, const DnhTensor* src, hipStream_t stream, int32_t* status) {
+    if (option(OPT_COUNT_ONE_LAUNCH) == 0 || nelems(t) != 1 || src->ndims < 1) return false;
+    const int64_t n = src->shape[src->ndims - 1];
+    for (int d = 0; d + 1 < src->ndims; d++)
+        if (src->shape[d] != 1) return false;
+    const uint8_t* mask = (const uint8_t*)elem_ptr(src);
+    if (src->stride[src->ndims - 1] != 1 || n < (1 << 20) || n >= ((int64_t)1 << 47) || ((uintptr_t)mask & 3) != 0) return false;
+    const int64_t piece = (int64_t)16 * kBlock;   // bytes one round of a workgroup's loads covers
+    int64_t nblocks = 2 * (int64_t)device_cus();
+    int64_t per_block = ((n + nblocks - 1) / nblocks + piece - 1) / piece * piece;
+    nblocks = (n + per_block - 1) / per_block;
+    if (nblocks > (int64_t)kCountGroup * (int64_t)kSyncMaxCountGroups) return false;
+    char* words = nullptr;
+    uint32_t epoch = 0;
+    WorkspaceLease lease;
+    *status = sync_words(stream, kSyncTileWords, (void**)&words, &epoch, lease);
+    if (*status != DNH_OK) return true;
+    hipLaunchKernelGGL(count_true_kernel, dim3((unsigned)nblocks), dim3(kBlock), 0, stream, mask, n, per_block, (uint32_t)nblocks,
+                       (unsigned long long*)(words + kSyncCountTop), (unsigned long long*)(words + kSyncCountGroups), (int64_t*)elem_ptr(t));
+    *status = hipGetLastError() == hipSuccess ? DNH_OK : fail(DNH_ERR_HIP, "CountTrue: launch failed");
+    return true;
+}
+}  // namespace
+
 // The folds of dnh_reduce_last_axis; `ps` says where the partial results of a two-pass fold are kept.
 static int32_t reduce_impl(const char* entry, int32_t op, const DnhTensor* t, const DnhTensor* src, hipStream_t st, const PartialStore& ps) {
     DNH_TRY(check_tensor(t, entry));
@@ -173,6 +264,10 @@ static int32_t reduce_impl(const char* entry, int32_t op, const DnhTensor* t, co
     }
     if (op == DNH_COUNT_TRUE) {
         if (src->dtype != DNH_BOOL || t->dtype != DNH_I64) return fail(DNH_ERR_INVALID_ARG, "CountTrue needs a bool source and an int64 target");
+        if (t->ndims + 1 == src->ndims) {   // (a source tensor with more than 2^47 elements cannot exist: the arrival field is safe)
+            int32_t cst = DNH_OK;
+            if (try_count_true_one_launch(t, src, st, &cst)) return cst;
+        }
         return launch_reduce(RCountTrue{}, t, src, st, "CountTrueLastAxis", ps);
     }
     if (t->dtype != src->dtype) return fail(DNH_ERR_INVALID_ARG, "%s: target is %s but source is %s", entry, dtype_name(t->dtype), dtype_name(src->dtype));

@@ -29,6 +29,11 @@ struct Workspace {
     std::mutex in_use;   // held through a WorkspaceLease while an entry point queues the kernels that use the buffer
     void* ptr = nullptr;
     size_t bytes = 0;
+    // words through which the workgroups of one launch meet (arrival counters, tile descriptors): zero when allocated,
+    // never used for anything else, so a kernel may rely on what the previous launch left there
+    void* sync_ptr = nullptr;
+    size_t sync_bytes = 0;
+    uint32_t epoch = 0;   // counts the launches that used the words; 30 bits, the words are cleared when it wraps
 };
 std::map<hipStream_t, Workspace> g_ws;
 
@@ -132,7 +137,9 @@ struct OptionDef {
 // order of enum Option
 constexpr OptionDef kOptions[OPT_COUNT] = {
     {"dot_bf16x3", 1, 0, 1},       {"dot_f64_pinned", 1, 0, 1},    {"dot_big", -1, -1, 1},          {"dot_splits", 0, 0, 1 << 20},
-    {"dot_int_mfma", 1, 0, 1},     {"tr4", 1, 0, 1},               {"scatter_fp_atomic", 0, 0, 1},  {"compact_one_pass", 1, 0, 1},
+    {"dot_int_mfma", 1, 0, 1},     {"tr4", 1, 0, 1},               {"scatter_fp_atomic", 0, 0, 1},  {"compact_one_pass", 0, 0, 1},
+    {"count_one_launch", 1, 0, 1},
+    {"lookback_spins", 1 << 18, 0, 1 << 30},
 };
 std::atomic<int> g_options[OPT_COUNT];
 std::once_flag g_options_once;
@@ -202,6 +209,40 @@ int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& 
     return DNH_OK;
 }
 
+int32_t sync_words(hipStream_t stream, size_t bytes, void** out, uint32_t* epoch, WorkspaceLease& lease) {
+    Workspace* w;
+    {
+        std::lock_guard<std::mutex> lock(g_mu);
+        w = &g_ws[stream];
+    }
+    if (lease.held_ != &w->in_use) {
+        lease.release();
+        w->in_use.lock();
+        lease.held_ = &w->in_use;
+    }
+    bool clear = false;
+    if (w->sync_bytes < bytes) {
+        if (w->sync_ptr) {
+            DNH_HIP(hipStreamSynchronize(stream));
+            DNH_HIP(hipFree(w->sync_ptr));
+            w->sync_ptr = nullptr;
+            w->sync_bytes = 0;
+        }
+        const size_t want = bytes < (size_t)(64 << 10) ? (size_t)(64 << 10) : bytes * 2;
+        DNH_TRY(device_malloc(&w->sync_ptr, want, "synchronisation words"));
+        w->sync_bytes = want;
+        clear = true;
+    }
+    if (++w->epoch >= (1u << 30)) {
+        w->epoch = 1;
+        clear = true;
+    }
+    if (clear) DNH_HIP(hipMemsetAsync(w->sync_ptr, 0, w->sync_bytes, stream));   // ordered before the kernels the caller is about to queue
+    *out = w->sync_ptr;
+    *epoch = w->epoch;
+    return DNH_OK;
+}
+
 static void drop_workspace(hipStream_t stream) {
     std::lock_guard<std::mutex> lock(g_mu);
     auto ef = g_error_flags.find(stream);
@@ -212,6 +253,7 @@ static void drop_workspace(hipStream_t stream) {
     auto it = g_ws.find(stream);
     if (it != g_ws.end()) {
         if (it->second.ptr) (void)hipFree(it->second.ptr);
+        if (it->second.sync_ptr) (void)hipFree(it->second.sync_ptr);
         g_ws.erase(it);
     }
 }

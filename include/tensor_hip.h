@@ -162,7 +162,11 @@ int32_t dnh_last_error(char* buf, size_t n);
  *   "dot_int_mfma"      1 (default): 32- and 64-bit integer products on the int8 matrix instruction
  *   "tr4"               1 (default): transposing copies of 4-byte elements through LDS
  *   "scatter_fp_atomic" 0 (default): floating-point scatter adds duplicates in source order; 1: float atomics (faster, order varies)
- *   "compact_one_pass"  1 (default): compactions of contiguous masks in one launch; 0: a counting and a moving launch
+ *   "compact_one_pass"  0 (default): compactions of contiguous masks by a counting and a moving launch; 1: one launch whose
+ *                       workgroups pass their counts on through device memory (measured slower on MI355X: the counts cross XCDs)
+ *   "count_one_launch"  1 (default): CountTrue of a whole contiguous mask in one launch
+ *   "lookback_spins"    262144 (default): how often a tile of a one-pass compaction polls for the counts of the tiles before it
+ *                       before it counts them itself (0: at once; for tests of that path)
  * Unknown names and values outside an option's range: DNH_ERR_INVALID_ARG. */
 int32_t dnh_set_option(const char* name, int32_t value);
 int32_t dnh_get_option(const char* name, int32_t* value);

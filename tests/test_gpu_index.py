@@ -346,3 +346,79 @@ def test_config4_sequence_small(H, G, rng):
             assert r == g == int((a > 0).sum())
         else:
             assert_exact(r, g)
+
+
+@pytest.fixture(params=["two_launches", "one_pass", "tiles_do_not_wait"])
+def compaction_form(request):
+    """The contiguous compactions in their three forms: a counting and a moving launch (the default), one pass whose workgroups meet
+    through memory (compact_one_pass = 1), and that pass with workgroups that do not poll at all: one that finds a predecessor's count
+    unpublished counts the mask in front of its region itself (lookback_spins = 0: the bounded wait's way out, forced).  CountTrue
+    runs in its one-launch form in the first and in the general two-pass fold in the others."""
+    from deepnet_amd import native
+    if request.param == "two_launches":
+        yield request.param
+    elif request.param == "one_pass":
+        with native.option("compact_one_pass", 1), native.option("count_one_launch", 0):
+            yield request.param
+    else:
+        with native.option("compact_one_pass", 1), native.option("lookback_spins", 0), native.option("count_one_launch", 0):
+            yield request.param
+
+
+@pytest.mark.parametrize("dt", [np.int32, np.float64, np.uint8, np.int16])
+@pytest.mark.parametrize("n,density", [(16, 0.5), (4096, 0.5), (4112, 0.3), (1 << 20, 0.5), (3_000_016, 0.02), (3_000_016, 1.0),
+                                       (3_000_016, 0.0), ((1 << 22) + 64, 0.7)])
+def test_contiguous_compactions_in_every_form(G, rng, compaction_form, dt, n, density):
+    """maskedGet, maskedSet, trueIdx and countTrue of contiguous 1-d data against NumPy, bit for bit, from one tile to a thousand
+    tiles, all / none / few selected, twice in a row on the same stream (the second launch meets the words the first one left)."""
+    a = rng.integers(0, 100, n).astype(dt)
+    m = rng.random(n) < density if 0.0 < density < 1.0 else np.full(n, density == 1.0)
+    ta, tm = G.ofNumpy(a), G.ofNumpy(m)
+    k = int(m.sum())
+    for _ in range(2):
+        assert_exact(a[m], G.toNumpy(ta.M(tm)))
+        assert int(tm.countTrue()) == k
+        assert_exact(np.flatnonzero(m).astype(np.int64).reshape(-1, 1), G.toNumpy(tm.trueIdx()))
+    vals = rng.integers(100, 200, k).astype(dt)
+    want = a.copy()
+    want[m] = vals
+    ta.setM([tm], G.ofNumpy(vals))
+    assert_exact(want, G.toNumpy(ta))
+    # a 2-d mask whose elements lie in row-major order: pairs of coordinates
+    if n % 16 == 0 and n >= 4096:
+        m2 = m.reshape(-1, 16)
+        assert_exact(np.argwhere(m2).astype(np.int64), G.toNumpy(G.ofNumpy(m2).trueIdx()))
+
+
+def test_one_pass_compactions_on_two_streams(G, rng):
+    """Every stream has its own tickets and tile words: compactions queued on two streams at once do not meet each other's."""
+    import ctypes as C
+    from deepnet_amd import native
+    lib = native.load()
+    native.set_option("compact_one_pass", 1)
+    n = 1 << 21
+    a = rng.integers(0, 1000, n).astype(np.int32)
+    masks = [rng.random(n) < d for d in (0.3, 0.6)]
+    streams = [C.c_void_p(), C.c_void_p()]
+    for s in streams:
+        native.check(lib.dnh_stream_create(C.byref(s)))
+    try:
+        ta = G.ofNumpy(a)
+        tms = [G.ofNumpy(m) for m in masks]
+        outs = [G.zeros([int(m.sum())], np.int32) for m in masks]
+        native.check(lib.dnh_device_sync())
+        for rep in range(4):
+            for s, tm, out in zip(streams, tms, outs):
+                arr = (C.POINTER(type(ta.Backend._desc(ta))) * 1)()
+                dm = tm.Backend._desc(tm)
+                arr[0] = C.pointer(dm)
+                dt_, da = out.Backend._desc(out), ta.Backend._desc(ta)
+                native.check(lib.dnh_masked_get(C.byref(dt_), C.byref(da), arr, 1, s))
+        for s in streams:
+            native.check(lib.dnh_stream_sync(s))
+        for m, out in zip(masks, outs):
+            assert_exact(a[m], G.toNumpy(out))
+    finally:
+        native.set_option("compact_one_pass", 0)
+        for s in streams:
+            native.check(lib.dnh_stream_destroy(s))

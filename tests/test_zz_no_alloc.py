@@ -68,20 +68,50 @@ def test_noalloc_fold_matches_the_allocating_entry_point_twice_in_a_row(G, rng, 
         assert np.array_equal(got2, a2.max(axis=axis))
 
 
+def _free_device_bytes():
+    """hipMemGetInfo through the HIP runtime the library has already loaded into this process."""
+    hip = C.CDLL("libamdhip64.so")
+    free, total = C.c_size_t(), C.c_size_t()
+    assert hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+    return free.value
+
+
 def test_noalloc_fold_does_not_touch_the_allocator(G, rng):
+    """A two-pass fold on a stream that has no workspace yet: the allocating entry point must ask the driver for one there (its
+    partials live in the stream's workspace, which comes straight from hipMalloc and never shows in the block cache's counters),
+    the entry point that may not allocate must leave the device's free memory and the block cache exactly as they were."""
     lib = native.load()
     a = G.ofNumpy(rng.standard_normal((2048, 2048)).astype(np.float32))
     _fold(G, "dnh_reduce_last_axis_noalloc", abi.DNH_SUM, a, 0, np.float32)   # first call on the device: looks the array up
     trgt = G.zeros((2048,), np.float32)
+    want = _fold(G, "dnh_reduce_last_axis", abi.DNH_SUM, a, 0, np.float32)
     lay = a.Layout
     sd = abi.make_descriptor(a.Storage.Pointer(), a.DataType, [2048, 2048], [lay.Stride[1], lay.Stride[0]], lay.Offset)
     td = trgt.Backend._desc(trgt)
-    before, after = abi.DnhPoolStats(), abi.DnhPoolStats()
-    native.check(lib.dnh_pool_stats(C.byref(before)))
-    native.check(lib.dnh_reduce_last_axis_noalloc(abi.DNH_SUM, C.byref(td), C.byref(sd), G.Cfg.Stream))
-    native.check(lib.dnh_pool_stats(C.byref(after)))
-    assert (before.hits, before.misses, before.live_bytes) == (after.hits, after.misses, after.live_bytes)
-    assert np.array_equal(G.toNumpy(trgt), _fold(G, "dnh_reduce_last_axis", abi.DNH_SUM, a, 0, np.float32))
+    native.check(lib.dnh_device_sync())
+    fresh, control = C.c_void_p(), C.c_void_p()
+    native.check(lib.dnh_stream_create(C.byref(fresh)))
+    native.check(lib.dnh_stream_create(C.byref(control)))
+    try:
+        before, after = abi.DnhPoolStats(), abi.DnhPoolStats()
+        native.check(lib.dnh_pool_stats(C.byref(before)))
+        free0 = _free_device_bytes()
+        native.check(lib.dnh_reduce_last_axis_noalloc(abi.DNH_SUM, C.byref(td), C.byref(sd), fresh))
+        native.check(lib.dnh_stream_sync(fresh))
+        free1 = _free_device_bytes()
+        native.check(lib.dnh_pool_stats(C.byref(after)))
+        assert free1 == free0, f"the no-alloc fold changed the device's free memory by {free0 - free1} bytes"
+        assert (before.hits, before.misses, before.live_bytes, before.cached_bytes) == (after.hits, after.misses, after.live_bytes, after.cached_bytes)
+        assert np.array_equal(G.toNumpy(trgt), want)
+        # the probe does see an allocation: the same fold through the allocating entry point on a stream without a workspace
+        free2 = _free_device_bytes()
+        native.check(lib.dnh_reduce_last_axis(abi.DNH_SUM, C.byref(td), C.byref(sd), control))
+        native.check(lib.dnh_stream_sync(control))
+        assert _free_device_bytes() < free2, "control: the allocating entry point took no workspace, so this shape does not test the property"
+        assert np.array_equal(G.toNumpy(trgt), want)
+    finally:
+        native.check(lib.dnh_stream_destroy(fresh))
+        native.check(lib.dnh_stream_destroy(control))
 
 
 def test_noalloc_fold_refuses_partials_beyond_the_static_array(G, rng):
