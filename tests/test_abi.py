@@ -79,3 +79,24 @@ def test_status_codes_map_to_reference_exception_kinds():
     assert native._EXC[abi.DNH_ERR_NOT_SUPPORTED] is NotImplementedError
     assert native._EXC[abi.DNH_ERR_INDEX_OUT_OF_RANGE] is IndexError
     assert native._EXC[abi.DNH_ERR_OUT_OF_MEMORY] is MemoryError
+
+
+def test_options_are_set_and_read_without_a_device():
+    """dnh_set_option / dnh_get_option touch no GPU: defaults, round trip, refusal of unknown names and of values out of range."""
+    defaults = {"dot_bf16x3": 1, "dot_f64_pinned": 1, "dot_big": -1, "dot_splits": 0, "dot_int_mfma": 1, "tr4": 1,
+                "scatter_fp_atomic": 0, "compact_one_pass": 0, "count_one_launch": 1, "lookback_spins": 1 << 18}
+    header = open(HEADER).read()
+    for name, value in defaults.items():
+        assert f'"{name}"' in header, f"include/tensor_hip.h does not document option {name}"
+        if os.environ.get("DNH_" + name.upper()) is None:
+            assert native.get_option(name) == value
+        with native.option(name, 0):
+            assert native.get_option(name) == 0
+        assert native.get_option(name) == (value if os.environ.get("DNH_" + name.upper()) is None else native.get_option(name))
+    with pytest.raises(ValueError):
+        native.set_option("dot_big", 2)
+    with pytest.raises(ValueError):
+        native.set_option("dot_bf16x3", -1)
+    with pytest.raises(ValueError):
+        native.get_option("nonexistent")
+    assert "nonexistent" in native.last_error()
