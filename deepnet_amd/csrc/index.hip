@@ -484,8 +484,9 @@ bool try_scatter_binned(const DnhTensor* t, const DnhTensor* const* idx, int32_t
 //   1. ordered_cells:  cell[s] = row-major position in t that source s names (-1 and the error word when out of range)
 //   2. ordered_count:  per workgroup of kOrdChunk sources, how many fall into each bucket of 2^shift consecutive cells   -> counts
 //   3. bin_colscan, ordered_starts: where each workgroup's share of each bucket starts in the bucket's list             -> counts, starts
-//   4. ordered_move:   each workgroup sorts its sources by (cell, source position) in LDS (bitonic) and appends every bucket's run to
-//                      that bucket's list: a list is ordered by workgroup, then by cell, then by source position
+//   4. ordered_move:   each workgroup sorts its sources by cell in LDS (a stable radix sort: sources of one cell keep their order)
+//                      and appends every bucket's run to that bucket's list: a list is ordered by workgroup, then by cell, then by
+//                      source position
 //   5. ordered_apply:  one workgroup per bucket keeps the bucket's cells in LDS and walks the list in batches of 1024 entries.
 //                      Entries of one cell that are neighbours in a batch form a run, which the thread at its head adds in order;
 //                      runs of one cell that are not neighbours (they come from different workgroups of pass 4) are applied in
@@ -561,47 +562,89 @@ __global__ __launch_bounds__(kOrdThreads) void ordered_starts_kernel(const uint3
     }
 }
 
+// Pass 4.  The chunk's sources are sorted by cell with a least-significant-digit radix sort in LDS (digits of kOrdDigitBits bits,
+// every pass stable, so sources of one cell stay in source order).  A thread keeps its kOrdPer keys in registers; key e of thread t
+// stands at position e * 1024 + t, so a wavefront holds 64 consecutive positions ("a row") per e.  Per pass: the lanes of a row that
+// share a digit find each other with one ballot per digit bit, which gives each its rank among them and, to the first of them, their
+// number for the counter of (digit, row); an exclusive scan over the counters in (digit, row) order is every group's start; the keys
+// go to LDS at start + rank and come back by position.  Sources outside the slab carry one cell number beyond its last cell, so
+// they end up behind everything that is moved.
+constexpr int kOrdDigitBits = 5, kOrdDigits = 1 << kOrdDigitBits, kOrdRows = kOrdChunk / 64;
 template <class X>
 __global__ __launch_bounds__(kOrdThreads) void ordered_move_kernel(const int64_t* __restrict__ cell, const X* __restrict__ src, Lay slay, uint32_t m,
-                                                                   int64_t lo, int64_t hi, int shift, uint32_t nb,
+                                                                   int64_t lo, int64_t hi, int shift, uint32_t nb, int npass,
                                                                    const uint32_t* __restrict__ counts, const uint32_t* __restrict__ starts,
                                                                    uint32_t* __restrict__ pc, X* __restrict__ pv) {
     extern __shared__ __align__(16) unsigned char ord_lds[];
-    uint64_t* keys = reinterpret_cast<uint64_t*>(ord_lds);            // (cell - lo) << 13 | position in the chunk; all ones = not in this slab
-    X* vals = reinterpret_cast<X*>(keys + kOrdChunk);                  // by position in the chunk
-    uint32_t* gstart = reinterpret_cast<uint32_t*>(vals + kOrdChunk);  // where each bucket's run starts among the sorted keys
-    const uint32_t i0 = blockIdx.x * kOrdChunk;
+    uint64_t* keys = reinterpret_cast<uint64_t*>(ord_lds);            // by position: (cell - lo) << 13 | position the source had in the chunk
+    X* vals = reinterpret_cast<X*>(keys + kOrdChunk);                  // by position the source had in the chunk
+    uint32_t* cnt = reinterpret_cast<uint32_t*>(vals + kOrdChunk);     // kOrdDigits x kOrdRows counters; afterwards: where each bucket's run starts
+    uint32_t* gstart = cnt;
+    __shared__ uint32_t wave_sum[kOrdThreads / 64];
+    const uint32_t i0 = blockIdx.x * kOrdChunk, lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    const uint64_t outside = (uint64_t)(hi - lo);
+    uint64_t key[kOrdPer];
 #pragma unroll
     for (int e = 0; e < kOrdPer; e++) {
         const uint32_t li = e * kOrdThreads + threadIdx.x, i = i0 + li;
         const int64_t c = i < m ? cell[i] : -1;
-        keys[li] = (c >= lo && c < hi) ? (((uint64_t)(c - lo) << kOrdLiBits) | li) : ~0ull;
+        key[e] = (((c >= lo && c < hi) ? (uint64_t)(c - lo) : outside) << kOrdLiBits) | li;
         vals[li] = i < m ? src[offset_of(slay, i)] : X(0);
     }
-    __syncthreads();
-    // bitonic sort, ascending (keys are distinct except for the all-ones ones, which end up last)
-    for (uint32_t k = 2; k <= kOrdChunk; k <<= 1) {
-        for (uint32_t j = k >> 1; j > 0; j >>= 1) {
+    constexpr int CPT = kOrdDigits * kOrdRows / kOrdThreads;   // counters per thread in the scan
+    for (int pass = 0; pass < npass; pass++) {
+        const int sh = kOrdLiBits + pass * kOrdDigitBits;
 #pragma unroll
-            for (int e = 0; e < kOrdPer / 2; e++) {
-                const uint32_t t = e * kOrdThreads + threadIdx.x;
-                const uint32_t i = ((t & ~(j - 1u)) << 1) | (t & (j - 1u)), l = i | j;
-                const bool up = (i & k) == 0;
-                const uint64_t x = keys[i], y = keys[l];
-                if ((x > y) == up) {
-                    keys[i] = y;
-                    keys[l] = x;
-                }
+        for (int q = 0; q < CPT; q++) cnt[threadIdx.x * CPT + q] = 0;
+        __syncthreads();   // counters cleared (and the previous pass's keys read back)
+        uint32_t rank[kOrdPer], slot[kOrdPer];
+#pragma unroll
+        for (int e = 0; e < kOrdPer; e++) {
+            const uint32_t d = (uint32_t)(key[e] >> sh) & (kOrdDigits - 1);
+            unsigned long long peers = ~0ull;
+#pragma unroll
+            for (int bit = 0; bit < kOrdDigitBits; bit++) {
+                const bool set = (d >> bit) & 1u;
+                const unsigned long long with = __ballot(set);
+                peers &= set ? with : ~with;
             }
-            __syncthreads();
+            rank[e] = (uint32_t)__popcll(peers & ((1ull << lane) - 1ull));
+            slot[e] = d * kOrdRows + (uint32_t)e * (kOrdThreads / 64) + wave;
+            if (rank[e] == 0) cnt[slot[e]] = (uint32_t)__popcll(peers);
         }
+        __syncthreads();
+        {
+            uint32_t v[CPT], sum = 0, total;
+#pragma unroll
+            for (int q = 0; q < CPT; q++) {
+                v[q] = cnt[threadIdx.x * CPT + q];
+                sum += v[q];
+            }
+            uint32_t run = bin_block_scan(sum, &total, wave_sum);   // (two barriers inside)
+#pragma unroll
+            for (int q = 0; q < CPT; q++) {
+                cnt[threadIdx.x * CPT + q] = run;
+                run += v[q];
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < kOrdPer; e++) keys[cnt[slot[e]] + rank[e]] = key[e];
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < kOrdPer; e++) key[e] = keys[e * kOrdThreads + threadIdx.x];
     }
+    if (npass == 0) {
+#pragma unroll
+        for (int e = 0; e < kOrdPer; e++) keys[e * kOrdThreads + threadIdx.x] = key[e];
+    }
+    __syncthreads();   // keys[] holds the sorted keys; cnt is free for the buckets' starts
 #pragma unroll
     for (int e = 0; e < kOrdPer; e++) {
         const uint32_t k = e * kOrdThreads + threadIdx.x;
-        const uint64_t key = keys[k];
-        if (key != ~0ull) {
-            const uint32_t b = (uint32_t)((key >> kOrdLiBits) >> shift);
+        const uint64_t cl = key[e] >> kOrdLiBits;
+        if (cl < outside) {
+            const uint32_t b = (uint32_t)(cl >> shift);
             if (k == 0 || (uint32_t)((keys[k - 1] >> kOrdLiBits) >> shift) != b) gstart[b] = k;
         }
     }
@@ -609,13 +652,12 @@ __global__ __launch_bounds__(kOrdThreads) void ordered_move_kernel(const int64_t
 #pragma unroll
     for (int e = 0; e < kOrdPer; e++) {
         const uint32_t k = e * kOrdThreads + threadIdx.x;
-        const uint64_t key = keys[k];
-        if (key != ~0ull) {
-            const uint64_t cl = key >> kOrdLiBits;
+        const uint64_t cl = key[e] >> kOrdLiBits;
+        if (cl < outside) {
             const uint32_t b = (uint32_t)(cl >> shift);
             const uint32_t dst = starts[b] + counts[(size_t)blockIdx.x * nb + b] + (k - gstart[b]);
             pc[dst] = (uint32_t)(cl & ((1u << shift) - 1u));
-            pv[dst] = vals[(uint32_t)key & (kOrdChunk - 1u)];
+            pv[dst] = vals[(uint32_t)key[e] & (kOrdChunk - 1u)];
         }
     }
 }
@@ -637,10 +679,10 @@ __global__ __launch_bounds__(kOrdThreads) void ordered_apply_kernel(X* __restric
                                                                     const uint32_t* __restrict__ pc, const X* __restrict__ pv) {
     extern __shared__ __align__(16) unsigned char ord_lds[];
     const uint32_t cells = 1u << shift;
-    X* acc = reinterpret_cast<X*>(ord_lds);                         // the bucket's cells
-    X* bv = acc + cells;                                            // the batch: values
-    uint32_t* claim = reinterpret_cast<uint32_t*>(bv + kOrdThreads); // per cell: position in the batch of the first pending run, or kOrdNone
-    uint32_t* bc = claim + cells;                                   // the batch: cells (inside the bucket)
+    X* acc = reinterpret_cast<X*>(ord_lds);                                      // the bucket's cells
+    X* bv = acc + cells;                                                         // the batch: values
+    uint32_t* claim = reinterpret_cast<uint32_t*>(bv + kOrdThreads);             // per cell: position in the batch of the first pending run, or kOrdNone
+    uint32_t* bc = claim + cells;                                                // the batch: cells (inside the bucket)
     const uint32_t b = blockIdx.x;
     const uint32_t cnt = totals[b];
     if (cnt == 0) return;   // uniform: nothing lands in this bucket
@@ -665,6 +707,9 @@ __global__ __launch_bounds__(kOrdThreads) void ordered_apply_kernel(X* __restric
             if (pending) atomicMin(&claim[c], threadIdx.x);
             __syncthreads();
             if (pending && claim[c] == threadIdx.x) {
+                // the run is added in order, entry by entry (a cell that receives L sources is a chain of L dependent additions; fetching
+                // the entries of long runs ahead of the additions measured 3x faster for a single cell that takes everything, and
+                // 15-50 % slower for everything else: the fetched entries' registers cost the common, short runs more than they save)
                 X a = acc[c];
                 for (uint32_t k = threadIdx.x; k < nbat && bc[k] == c; k++) a = a + bv[k];
                 acc[c] = a;
@@ -718,10 +763,11 @@ int32_t scatter_ordered(const DnhTensor* t, const DnhTensor* src, const IndexArg
     uint32_t* starts = (uint32_t*)(ws + p.cell_bytes + p.counts_bytes + p.totals_bytes);
     uint32_t* pc = (uint32_t*)(ws + p.cell_bytes + p.counts_bytes + 2 * p.totals_bytes);
     X* pv = (X*)(ws + p.cell_bytes + p.counts_bytes + 2 * p.totals_bytes + p.pc_bytes);
-    const size_t move_lds = (size_t)kOrdChunk * (8 + sizeof(X)) + (size_t)p.nb_max * 4;
+    static_assert(kOrdDigits * kOrdRows <= (int)kOrdMaxBuckets, "the radix counters share the bucket starts' array");
+    const size_t move_lds = (size_t)kOrdChunk * (8 + sizeof(X)) + (size_t)kOrdMaxBuckets * 4;   // keys, values, then the counters / bucket starts
     const size_t apply_lds = ((size_t)1 << p.shift) * (sizeof(X) + 4) + (size_t)kOrdThreads * (sizeof(X) + 4);
     static const hipError_t attr_move = hipFuncSetAttribute(reinterpret_cast<const void*>(&ordered_move_kernel<X>), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                            (int)((size_t)kOrdChunk * (8 + sizeof(X)) + (size_t)kOrdMaxBuckets * 4));
+                                                            (int)move_lds);
     static const hipError_t attr_apply = hipFuncSetAttribute(reinterpret_cast<const void*>(&ordered_apply_kernel<X>), hipFuncAttributeMaxDynamicSharedMemorySize,
                                                              (int)(((size_t)1 << kOrdMaxShift) * (sizeof(X) + 4) + (size_t)kOrdThreads * (sizeof(X) + 4)));
     if (attr_move != hipSuccess || attr_apply != hipSuccess) return fail(DNH_ERR_HIP, "dnh_scatter: cannot size the LDS of the ordered scatter");
@@ -745,8 +791,11 @@ int32_t scatter_ordered(const DnhTensor* t, const DnhTensor* src, const IndexArg
         hipLaunchKernelGGL(ordered_count_kernel, dim3(p.nchunks), dim3(kOrdThreads), nb * 4, stream, (const int64_t*)cell, (uint32_t)m, lo, hi, p.shift, nb, counts);
         hipLaunchKernelGGL(bin_colscan_kernel, dim3(cdiv(nb, 64)), dim3(kBinThreads), 0, stream, counts, totals, nb, p.nchunks);
         hipLaunchKernelGGL(ordered_starts_kernel, dim3(1), dim3(kOrdThreads), 0, stream, (const uint32_t*)totals, starts, nb);
+        int bits = 0;   // of the largest cell number inside the slab, hi - lo, which stands for "outside"
+        while (((int64_t)1 << bits) <= hi - lo) bits++;
+        const int npass = (bits + kOrdDigitBits - 1) / kOrdDigitBits;
         hipLaunchKernelGGL((ordered_move_kernel<X>), dim3(p.nchunks), dim3(kOrdThreads), move_lds, stream, (const int64_t*)cell, (const X*)elem_ptr(src), slay,
-                           (uint32_t)m, lo, hi, p.shift, nb, (const uint32_t*)counts, (const uint32_t*)starts, pc, pv);
+                           (uint32_t)m, lo, hi, p.shift, nb, npass, (const uint32_t*)counts, (const uint32_t*)starts, pc, pv);
         hipLaunchKernelGGL((ordered_apply_kernel<X>), dim3(nb), dim3(kOrdThreads), apply_lds, stream, tp, tlay, dense, lo, ncells, p.shift,
                            (const uint32_t*)totals, (const uint32_t*)starts, (const uint32_t*)pc, (const X*)pv);
         DNH_LAUNCH_CHECK();

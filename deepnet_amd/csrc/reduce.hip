@@ -264,8 +264,8 @@ static int32_t reduce_impl(const char* entry, int32_t op, const DnhTensor* t, co
     }
     if (op == DNH_COUNT_TRUE) {
         if (src->dtype != DNH_BOOL || t->dtype != DNH_I64) return fail(DNH_ERR_INVALID_ARG, "CountTrue needs a bool source and an int64 target");
-        if (t->ndims + 1 == src->ndims) {   // (a source tensor with more than 2^47 elements cannot exist: the arrival field is safe)
-            int32_t cst = DNH_OK;
+        if (t->ndims + 1 == src->ndims && !ps.fixed) {   // (the entry point that may not allocate keeps the general fold: the arrival words
+            int32_t cst = DNH_OK;                        //  live in a buffer the library allocates on a stream's first use)
             if (try_count_true_one_launch(t, src, st, &cst)) return cst;
         }
         return launch_reduce(RCountTrue{}, t, src, st, "CountTrueLastAxis", ps);

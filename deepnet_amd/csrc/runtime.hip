@@ -209,6 +209,11 @@ int32_t workspace(hipStream_t stream, size_t bytes, void** out, WorkspaceLease& 
     return DNH_OK;
 }
 
+__global__ void zero_words_kernel(unsigned long long* p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) p[i] = 0ull;
+}
+
 int32_t sync_words(hipStream_t stream, size_t bytes, void** out, uint32_t* epoch, WorkspaceLease& lease) {
     Workspace* w;
     {
@@ -228,7 +233,7 @@ int32_t sync_words(hipStream_t stream, size_t bytes, void** out, uint32_t* epoch
             w->sync_ptr = nullptr;
             w->sync_bytes = 0;
         }
-        const size_t want = bytes < (size_t)(64 << 10) ? (size_t)(64 << 10) : bytes * 2;
+        const size_t want = (bytes < (size_t)(64 << 10) ? (size_t)(64 << 10) : bytes * 2 + 7) / 8 * 8;
         DNH_TRY(device_malloc(&w->sync_ptr, want, "synchronisation words"));
         w->sync_bytes = want;
         clear = true;
@@ -237,7 +242,11 @@ int32_t sync_words(hipStream_t stream, size_t bytes, void** out, uint32_t* epoch
         w->epoch = 1;
         clear = true;
     }
-    if (clear) DNH_HIP(hipMemsetAsync(w->sync_ptr, 0, w->sync_bytes, stream));   // ordered before the kernels the caller is about to queue
+    if (clear) {   // a fill kernel, not a memset node: the call may be under stream capture; ordered before the kernels the caller queues next
+        const size_t nwords = w->sync_bytes / 8;
+        hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)((nwords + 255) / 256)), dim3(256), 0, stream, (unsigned long long*)w->sync_ptr, nwords);
+        DNH_LAUNCH_CHECK();
+    }
     *out = w->sync_ptr;
     *epoch = w->epoch;
     return DNH_OK;

@@ -103,6 +103,18 @@ def test_noalloc_fold_does_not_touch_the_allocator(G, rng):
         assert free1 == free0, f"the no-alloc fold changed the device's free memory by {free0 - free1} bytes"
         assert (before.hits, before.misses, before.live_bytes, before.cached_bytes) == (after.hits, after.misses, after.live_bytes, after.cached_bytes)
         assert np.array_equal(G.toNumpy(trgt), want)
+        # CountTrue of a whole mask: the allocating entry point takes a one-launch form whose arrival words the library allocates on a
+        # stream's first use; the entry point that may not allocate must keep the fold that needs only the static array
+        mask = rng.random(1 << 22) < 0.5
+        tm = G.ofNumpy(mask)
+        cnt = G.zeros([], np.int64)
+        md, cd = tm.Backend._desc(tm), cnt.Backend._desc(cnt)
+        native.check(lib.dnh_device_sync())
+        free_c = _free_device_bytes()
+        native.check(lib.dnh_reduce_last_axis_noalloc(abi.DNH_COUNT_TRUE, C.byref(cd), C.byref(md), fresh))
+        native.check(lib.dnh_stream_sync(fresh))
+        assert _free_device_bytes() == free_c
+        assert int(G.toNumpy(cnt)) == int(mask.sum())
         # the probe does see an allocation: the same fold through the allocating entry point on a stream without a workspace
         free2 = _free_device_bytes()
         native.check(lib.dnh_reduce_last_axis(abi.DNH_SUM, C.byref(td), C.byref(sd), control))
