@@ -51,9 +51,9 @@ def nsets_for(nbytes):
 
 def profiled_call_traffic(tag):
     """HBM bytes one call moves according to the committed hardware-counter summary (`traffic_bytes_per_call <tag> <bytes>` lines of
-    profiles/configs_1_to_6_all_kernels.txt), or None.  Used for the calls whose traffic is far from their algorithmic bytes."""
+    profiles/configs_all_kernels.txt), or None.  Used for the calls whose traffic is far from their algorithmic bytes."""
     import os
-    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "configs_1_to_6_all_kernels.txt")
+    path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles", "configs_all_kernels.txt")
     try:
         with open(path) as f:
             for line in f:
@@ -100,11 +100,11 @@ def report(log, cfg, name, ms, nbytes=None, flops=None, pipe=None):
     row = {"cfg": cfg, "op": name, "us": round(ms * 1e3, 2), "bytes": int(nbytes), "GBps": round(gb, 1), "bound": "hbm", "frac": round(gb / HBM_PEAK_GBS, 4)}
     # gather / scatter move far more than their algorithmic bytes (a cache line per random 4-byte access): the counter-measured
     # traffic of the call and the rate it stands for are reported beside the algorithmic figures
-    tag = "Gather" if name.startswith("Gather") else "Scatter" if "Scatter" in name else None
+    tag = ("Gather" if name.startswith("Gather") else "Scatter" if "Scatter" in name else None) if cfg == 4 else None
     traffic = profiled_call_traffic(tag) if tag else None
     if traffic:
         row.update({"traffic_bytes": traffic, "traffic_GBps": round(traffic / (ms * 1e-3) / 1e9, 1),
-                    "traffic_frac": round(traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic_source": "profiles/configs_1_to_6_all_kernels.txt"})
+                    "traffic_frac": round(traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4), "traffic_source": "profiles/configs_all_kernels.txt"})
         log(f"       (counter-measured traffic of this call {traffic / 1e6:.1f} MB = {traffic / (ms * 1e-3) / 1e9:.0f} GB/s = {100 * traffic / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS:.1f}% of HBM peak)")
     return row
 
@@ -361,6 +361,28 @@ def run_all(log, which=(1, 2, 3, 4, 5, 6), fp32_folds=True, reference_dot_shapes
                 log(f"[cfg7] {name} 256 MiB {kind:8s} host memory {ms:9.2f} ms  {nbytes / ms / 1e6:8.1f} GB/s")
                 results.append({"cfg": 7, "op": f"{name} {kind}", "us": round(ms * 1e3, 1), "GBps": round(nbytes / ms / 1e6, 1)})
         check(lib.dnh_host_free(pinned))
+    if 8 in which:
+        # floating-point scatter with repeated indices (not one of the five configurations): the ordered form, which adds a cell's
+        # sources in the reference's order, beside float atomics; 4 Mi sources into 16 Mi cells, uniform random indices
+        N, M = 1 << 24, 1 << 22
+        hidx = rng.integers(0, N, M).astype(np.int64)
+        for dt, sz in ((np.float32, 4), (np.float64, 8)):
+            hsrc = rng.standard_normal(M).astype(dt)
+
+            def sca8(i):
+                src = G.ofNumpy(hsrc)
+                idx = G.ofNumpy(hidx)
+                t = new([N], dt)
+                arr = (C.POINTER(abi.DnhTensor) * 1)()
+                di = CAbiTensorBackend._desc(idx)
+                z = np.zeros(1, dt)
+                keep.append((idx, di, arr, z))
+                arr[0] = C.pointer(di)
+                return [("fill_const", (D(t), z.ctypes.data_as(C.c_void_p))), ("scatter", (D(t), arr, 1, D(src)))]
+            nm = np.dtype(dt).name
+            timed(8, f"FillConst 0 + Scatter {nm} ordered", N * sz + M * 8 + M * sz + M * sz, sca8, reps=6)
+            with T.native.option("scatter_fp_atomic", 1):
+                timed(8, f"FillConst 0 + Scatter {nm} atomics", N * sz + M * 8 + M * sz + M * sz, sca8, reps=6)
     return results
 
 
