@@ -51,6 +51,14 @@ def test_positions_beyond_32_bits(G):
     s = T.scatter([G.ofNumpy(idx)], [N], G.ofNumpy(vals))
     assert_exact(vals, G.toNumpy(T.gather([G.ofNumpy(idx)], s)))
     assert int(s.sum()) == int(vals.sum())
+    del s
+    # the same in single precision with a repeated index: the ordered form walks the 2^32 + 4096 cells in slabs of 4096 buckets
+    fidx = np.array([far, 3, N - 1, 1 << 32, far, 3], np.int64)
+    fvals = np.array([1e8, 0.5, -2.0, 7.25, 1.0, 1e-9], np.float32)
+    fs = T.scatter([G.ofNumpy(fidx)], [N], G.ofNumpy(fvals))
+    got = G.toNumpy(T.gather([G.ofNumpy(fidx[:4])], fs))
+    want = np.array([np.float32(np.float32(0) + np.float32(1e8)) + np.float32(1.0), np.float32(0.5) + np.float32(1e-9), -2.0, 7.25], np.float32)
+    assert_exact(want, got)
 
 
 def test_compaction_beyond_32_bits_is_refused_not_wrapped(G):

@@ -107,7 +107,13 @@ def test_random_gather_scatter(H, G, seed):
     for case in range(15):
         nd = int(rng.integers(1, 4))
         shape = [int(rng.choice([1, 3, 8, 17, 64, 100])) for _ in range(nd)]
-        src_np = rng.integers(-1000, 1000, size=shape).astype(np.int32)
+        # integers, and floats spread over many decades: scatter adds repeated indices in source order on both devices, so the
+        # floating-point sums agree bit for bit as well
+        dtype = [np.int32, np.float32, np.float64][int(rng.integers(0, 3))]
+        if dtype == np.int32:
+            src_np = rng.integers(-1000, 1000, size=shape).astype(np.int32)
+        else:
+            src_np = (rng.standard_normal(shape) * 10.0 ** rng.uniform(-6, 6, shape)).astype(dtype)
         ishape = [int(rng.choice([1, 5, 33, 200])) for _ in range(int(rng.integers(1, 3)))]
         use = [bool(rng.random() < 0.7) for _ in range(nd)]
         if not any(use):
