@@ -153,7 +153,7 @@ STATIC_SCRATCH_BYTES = 8 << 20
 
 # every symbol include/tensor_hip.h declares
 EXPORTED_SYMBOLS = [
-    "dnh_init", "dnh_device_info", "dnh_last_error", "dnh_async_error", "dnh_set_option", "dnh_get_option",
+    "dnh_init", "dnh_device_info", "dnh_last_error", "dnh_async_error", "dnh_set_option", "dnh_get_option", "dnh_scatter_workspace_bytes",
     "dnh_alloc", "dnh_free", "dnh_alloc_async", "dnh_free_async", "dnh_pool_trim", "dnh_pool_set_limit", "dnh_pool_stats",
     "dnh_host_alloc", "dnh_host_free", "dnh_memset",
     "dnh_memcpy_h2d", "dnh_memcpy_d2h", "dnh_memcpy_d2d",

@@ -441,6 +441,18 @@ inline size_t binned_workspace_bytes(int64_t m, int64_t n, size_t* counts_bytes,
     return *counts_bytes + *totals_bytes + (size_t)m * 8;
 }
 
+// Whether m updates of 32-bit integers into a rank-1 table of n elements take the binned form: its workspace in bytes, or 0 for the
+// direct kernel.  Cost model (measured on MI355X): a direct update costs about 40 ps (memory-side read-modify-write); the binned form
+// moves the table twice, the pairs four and a half times and the per-workgroup bucket counts four times (written, scanned in place,
+// read by the moving pass) at about 5.5 TB/s, plus three more launches.
+inline size_t binned_choice(int64_t m, int64_t n, size_t* counts_bytes, size_t* totals_bytes) {
+    if (m < (1 << 20) || m > 0x7FFFFFFFLL || n < 1 || n > ((int64_t)kBinMaxBuckets << kBinShift)) return 0;
+    const size_t ws_bytes = binned_workspace_bytes(m, n, counts_bytes, totals_bytes);
+    const double direct_us = (double)m * 40e-6, binned_us = ((double)n * 8.0 + (double)m * 36.0 + (double)*counts_bytes * 4.0) / 5.5e6 + 10.0;
+    if (binned_us >= direct_us || ws_bytes > kBinMaxWorkspace) return 0;
+    return ws_bytes;
+}
+
 // Takes the call when it has the binned form's shape and the binned form is the cheaper one; *status then holds its result.
 bool try_scatter_binned(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, hipStream_t stream, int32_t* err,
                         int32_t* status) {
@@ -448,15 +460,10 @@ bool try_scatter_binned(const DnhTensor* t, const DnhTensor* const* idx, int32_t
     if (t->ndims != 1 || src->ndims != 1 || n_idx != 1 || !idx[0] || idx[0]->ndims != 1) return false;
     if (t->stride[0] != 1 || src->stride[0] != 1 || idx[0]->stride[0] != 1) return false;
     const int64_t n = t->shape[0], m = src->shape[0];
-    if (m < (1 << 20) || m > 0x7FFFFFFFLL || n < 1 || n > ((int64_t)kBinMaxBuckets << kBinShift)) return false;
-    const uint32_t nb = (uint32_t)((n + kBinElems - 1) >> kBinShift), nchunks = cdiv(m, kBinChunk);
     size_t counts_bytes, totals_bytes;
-    const size_t ws_bytes = binned_workspace_bytes(m, n, &counts_bytes, &totals_bytes);
-    // cost model (measured on MI355X): a direct update costs about 40 ps (memory-side read-modify-write); the binned form moves the
-    // table twice, the pairs four and a half times and the per-workgroup bucket counts four times (written, scanned in place, read
-    // by the moving pass) at about 5.5 TB/s, plus three more launches
-    const double direct_us = (double)m * 40e-6, binned_us = ((double)n * 8.0 + (double)m * 36.0 + (double)counts_bytes * 4.0) / 5.5e6 + 10.0;
-    if (binned_us >= direct_us || ws_bytes > kBinMaxWorkspace) return false;
+    const size_t ws_bytes = binned_choice(m, n, &counts_bytes, &totals_bytes);
+    if (ws_bytes == 0) return false;
+    const uint32_t nb = (uint32_t)((n + kBinElems - 1) >> kBinShift), nchunks = cdiv(m, kBinChunk);
     char* ws = nullptr;
     WorkspaceLease lease;
     if (workspace(stream, ws_bytes, (void**)&ws, lease) != DNH_OK) {
@@ -1445,6 +1452,20 @@ extern "C" int32_t dnh_scatter(const DnhTensor* t, const DnhTensor* const* idx, 
     }
 #undef CASE
     DNH_LAUNCH_CHECK();
+    return DNH_OK;
+}
+
+extern "C" int32_t dnh_scatter_workspace_bytes(int32_t dtype, int64_t sources, int64_t cells, size_t* bytes) {
+    if (!bytes || sources < 0 || cells < 0 || dtype < 0 || dtype >= DNH_DTYPE_COUNT)
+        return fail(DNH_ERR_INVALID_ARG, "dnh_scatter_workspace_bytes: bad argument");
+    *bytes = 0;
+    if (sources == 0 || cells == 0) return DNH_OK;
+    if (dtype == DNH_I32 || dtype == DNH_U32) {
+        size_t c, t;
+        *bytes = binned_choice(sources, cells, &c, &t);
+    } else if (dtype_is_fp(dtype) && option(OPT_SCATTER_FP_ATOMIC) == 0) {
+        *bytes = ordered_plan(sources, cells, dtype_size(dtype)).total;
+    }
     return DNH_OK;
 }
 

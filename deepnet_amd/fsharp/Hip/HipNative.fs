@@ -71,6 +71,7 @@ module internal Native =
     // option names cross as NUL-terminated ASCII bytes
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_set_option (byte[] name, int value)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_get_option (byte[] name, int& value)
+    [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_scatter_workspace_bytes (int dtype, int64 sources, int64 cells, unativeint& bytes)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_alloc (unativeint bytes, nativeint& ptr)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_free (nativeint ptr)
     [<DllImport(Lib, CallingConvention=CallingConvention.Cdecl)>] extern int dnh_alloc_async (unativeint bytes, nativeint stream, nativeint& ptr)

@@ -37,6 +37,7 @@ def load() -> C.CDLL:
         "dnh_async_error": [vp, C.POINTER(i32)],
         "dnh_set_option": [C.c_char_p, i32],
         "dnh_get_option": [C.c_char_p, C.POINTER(i32)],
+        "dnh_scatter_workspace_bytes": [i32, C.c_int64, C.c_int64, C.POINTER(sz)],
         "dnh_alloc": [sz, C.POINTER(vp)],
         "dnh_free": [vp],
         "dnh_alloc_async": [sz, vp, C.POINTER(vp)],

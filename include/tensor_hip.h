@@ -271,6 +271,11 @@ int32_t dnh_gather(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_id
  * faster for few repeats, but the order of a cell's additions then varies from run to run; either way a target element that m_j
  * sources name is within m_j u sum|src_s| of the exact sum (u = unit roundoff). */
 int32_t dnh_scatter(const DnhTensor* t, const DnhTensor* const* idx, int32_t n_idx, const DnhTensor* src, void* stream);
+/* How much of the stream's workspace a dnh_scatter of `sources` elements into a target of `cells` elements asks for (no counterpart in
+ * the reference; for hosts that plan device memory): 0 for the forms that need none (atomics), the sorted pairs and counters of the
+ * binned form for 32-bit integers on rank-1 contiguous tensors when that form is chosen, about 20 bytes per source for the ordered
+ * floating-point form.  Touches no device. */
+int32_t dnh_scatter_workspace_bytes(int32_t dtype, int64_t sources, int64_t cells, size_t* bytes);
 /* ITensorBackend.CountTrue is dnh_reduce_last_axis(DNH_COUNT_TRUE).
  * ITensorBackend.MaskedGet (TensorBackend.fs:121; Host/ScalarOps.fs:667-681): masks has src->ndims entries, each NULL
  * or a rank-1 bool tensor of length src->shape[d]; selected elements are written to t in row-major order. */

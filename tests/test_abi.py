@@ -100,3 +100,45 @@ def test_options_are_set_and_read_without_a_device():
     with pytest.raises(ValueError):
         native.get_option("nonexistent")
     assert "nonexistent" in native.last_error()
+
+
+def test_scatter_workspace_sizes():
+    """The workspace a scatter asks for, against the formulas restated here: the binned form for 32-bit integers (per-workgroup
+    bucket counts, bucket totals, 8 bytes per pair; taken only when its cost model beats 40 ps per direct update and the workspace
+    stays within 1 GiB), the ordered form for floats (cells, counts, totals and starts, sorted cells and values)."""
+    lib = native.load()
+
+    def ask(dtype, m, n):
+        b = C.c_size_t()
+        native.check(lib.dnh_scatter_workspace_bytes(dtype, m, n, C.byref(b)))
+        return b.value
+
+    up = lambda x: (x + 255) // 256 * 256
+    # 32-bit integers
+    def binned(m, n):
+        nb, nchunks = -(-n // 16384), -(-m // 8192)
+        counts = up(nb * nchunks * 4)
+        ws = counts + up(nb * 4) + 8 * m
+        cheaper = (n * 8.0 + m * 36.0 + counts * 4.0) / 5.5e6 + 10.0 < m * 40e-6
+        return ws if (m >= 1 << 20 and m <= 2 ** 31 - 1 and 1 <= n <= 4096 * 16384 and cheaper and ws <= 1 << 30) else 0
+    for m, n in ((1 << 22, 1 << 24), (1 << 20, 300_000), ((1 << 20) - 1, 1 << 24), (1 << 21, 1 << 26), (1 << 28, 1 << 26), (1 << 22, (1 << 26) + 1)):
+        assert ask(abi.DNH_I32, m, n) == binned(m, n), (m, n)
+        assert ask(abi.DNH_U32, m, n) == binned(m, n)
+    assert ask(abi.DNH_I32, 1 << 22, 1 << 24) == 2 * 1024 * 1024 + 4096 + 8 * (1 << 22)
+    assert ask(abi.DNH_I32, 1 << 28, 1 << 26) == 0        # 512 MB of counts + 2 GB of pairs: beyond the cap, the direct kernel is taken
+    assert ask(abi.DNH_I64, 1 << 22, 1 << 24) == 0 and ask(abi.DNH_U8, 1 << 22, 1 << 24) == 0
+    # floats
+    def ordered(m, n, esize):
+        lg = max(n - 1, 0).bit_length()
+        shift = min(max(lg - 10, 4), 13)
+        nb = min(-(-n // (1 << shift)), 4096)
+        nchunks = -(-m // 8192)
+        return up(8 * m) + up(nb * nchunks * 4) + 2 * up(nb * 4) + up(4 * m) + up(esize * m)
+    for m, n in ((1 << 22, 1 << 24), (50_000, 777), (1, 1), (70_000, 1), (1 << 20, 40_000_000), (8191, 100_000)):
+        assert ask(abi.DNH_F32, m, n) == ordered(m, n, 4), (m, n)
+        assert ask(abi.DNH_F64, m, n) == ordered(m, n, 8), (m, n)
+    with native.option("scatter_fp_atomic", 1):
+        assert ask(abi.DNH_F32, 1 << 22, 1 << 24) == 0
+    assert ask(abi.DNH_F32, 0, 100) == 0 and ask(abi.DNH_F32, 100, 0) == 0
+    b = C.c_size_t()
+    assert lib.dnh_scatter_workspace_bytes(99, 1, 1, C.byref(b)) == abi.DNH_ERR_INVALID_ARG

@@ -40,7 +40,7 @@ def c_kind(param):
     table = {
         "const DnhTensor*": "desc", "const DnhTensor* const*": "descarray",
         "void*": "ptr", "const void*": "ptr", "void**": "ptrref",
-        "int32_t": "i32", "int32_t*": "i32ref", "size_t": "size",
+        "int32_t": "i32", "int32_t*": "i32ref", "size_t": "size", "int64_t": "i64", "size_t*": "sizeref",
         "char*": "bytes", "const char*": "bytes", "float*": "f32ref",
         "DnhDeviceInfo*": "structref", "DnhPoolStats*": "structref",
     }
@@ -62,7 +62,7 @@ def fs_kind(param):
     p = param.strip()
     ty = p.rsplit(" ", 1)[0].strip()
     table = {"DnhTensor&": "desc", "nativeint[]": "descarray", "nativeint": "ptr", "nativeint&": "ptrref", "int": "i32", "int&": "i32ref",
-             "unativeint": "size", "byte[]": "bytes"}
+             "unativeint": "size", "byte[]": "bytes", "int64": "i64", "unativeint&": "sizeref"}
     assert ty in table, f"unclassified F# parameter '{param}'"
     return table[ty]
 
