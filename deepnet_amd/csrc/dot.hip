@@ -866,30 +866,60 @@ __global__ __launch_bounds__(kBigThreads) void gemm_bf16x3_big_kernel(float* c, 
         }
     };
 
+    // Elements are fetched two K steps ahead of the step that multiplies them: those of step s + 2 are requested in the middle of step s
+    // (A) and near its end (B), cut into parts and written to the other LDS buffer during step s + 1, and multiplied in step s + 2, so
+    // that a fetch has two thirds of a step (about 3000 cycles) to arrive before its first use.  The barrier at the end of a step
+    // therefore has fetches in flight across it: it orders the LDS accesses only (lds_barrier), never the global ones.
+    auto lds_barrier = [] {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+    };
     const int64_t nsteps = (K + kX3BK - 1) / kX3BK;
-    sa.template load<TAIL>(0, K, ra);
-    sb.template load<TAIL>(0, K, rb);
+    if (nsteps == 1) {
+        sa.template load<TAIL>(0, K, ra);
+        sb.template load<TAIL>(0, K, rb);
+    } else {
+        sa.template load<false>(0, K, ra);
+        sb.template load<false>(0, K, rb);
+    }
     sa.store(ra, As[0]);
     sb.store(rb, Bs[0]);
-    __syncthreads();
+    if (nsteps == 2) {
+        sa.template load<TAIL>(kX3BK, K, ra);
+        sb.template load<TAIL>(kX3BK, K, rb);
+    } else if (nsteps > 2) {
+        sa.template load<false>(kX3BK, K, ra);
+        sb.template load<false>(kX3BK, K, rb);
+    }
+    lds_barrier();
     int cur = 0;
-    // One K step: fetch the next step's elements, multiply the current step's tiles, cut the fetched elements into parts and write them
-    // to the other buffer.  The instruction order is pinned by scheduling barriers (left alone, the compiler puts the fetches after most
-    // of the matrix instructions and the cutting after all of them: each wavefront then waits for memory with the matrix pipe idle):
-    // fetches first; the LDS reads of B and of the first 32 rows of A; then the 48 matrix instructions, the remaining LDS reads behind
-    // the first nine, and behind the later ones the 32 pieces of the cutting (X3Stage::piece) with their LDS writes.
-    auto k_step = [&](auto tail_tag, int64_t k_next) {
-        constexpr bool TL = decltype(tail_tag)::value;
-        sa.template load<TL>(k_next, K, ra);
-        sb.template load<TL>(k_next, K, rb);
+    // One K step: multiply the current step's tiles, cut the elements fetched during the previous step into parts and write them to the
+    // other buffer, request the elements of the step after the next (FETCH: 0 none, 1 whole K step, 2 the partial last one).  The
+    // instruction order is pinned by scheduling barriers (left alone, the compiler puts the fetches after most of the matrix instructions
+    // and the cutting after all of them: each wavefront then waits for memory with the matrix pipe idle): the LDS reads of B and of the
+    // first 32 rows of A; then the 48 matrix instructions, the remaining LDS reads behind the first nine, the 16 pieces of cutting A
+    // (X3Stage::piece) behind instructions 8-23, the request for A's next elements behind the 24th, B's pieces behind 24-39 and its
+    // request behind the 40th.
+    auto k_step = [&](auto fetch_tag, int64_t k_fetch) {
+        constexpr int FETCH = decltype(fetch_tag)::value;
         __builtin_amdgcn_sched_barrier(0);
         bf16x8 av[4][3], bv[2][3];
-#pragma unroll
-        for (int j = 0; j < 2; j++)
-#pragma unroll
-            for (int s = 0; s < 3; s++) bv[j][s] = *reinterpret_cast<const bf16x8*>(&Bs[cur][s][wn + j * 32 + lm][lk * 8]);
-#pragma unroll
-        for (int s = 0; s < 3; s++) av[0][s] = *reinterpret_cast<const bf16x8*>(&As[cur][s][wm + lm][lk * 8]);
+        // In the order of first use (the first matrix instruction multiplies the mid parts, the second hi by lo, the third lo by hi),
+        // the order pinned pair by pair: the eight wavefronts leave the barrier together and queue 72 reads of 1 KB at the LDS, so a
+        // first instruction that needs two of its wavefront's reads starts some 400 cycles before one that needs eight.
+        av[0][1] = *reinterpret_cast<const bf16x8*>(&As[cur][1][wm + lm][lk * 8]);
+        bv[0][1] = *reinterpret_cast<const bf16x8*>(&Bs[cur][1][wn + lm][lk * 8]);
+        __builtin_amdgcn_sched_barrier(0);
+        av[0][0] = *reinterpret_cast<const bf16x8*>(&As[cur][0][wm + lm][lk * 8]);
+        bv[0][2] = *reinterpret_cast<const bf16x8*>(&Bs[cur][2][wn + lm][lk * 8]);
+        __builtin_amdgcn_sched_barrier(0);
+        av[0][2] = *reinterpret_cast<const bf16x8*>(&As[cur][2][wm + lm][lk * 8]);
+        bv[0][0] = *reinterpret_cast<const bf16x8*>(&Bs[cur][0][wn + lm][lk * 8]);
+        __builtin_amdgcn_sched_barrier(0);
+        bv[1][1] = *reinterpret_cast<const bf16x8*>(&Bs[cur][1][wn + 32 + lm][lk * 8]);
+        bv[1][2] = *reinterpret_cast<const bf16x8*>(&Bs[cur][2][wn + 32 + lm][lk * 8]);
+        bv[1][0] = *reinterpret_cast<const bf16x8*>(&Bs[cur][0][wn + 32 + lm][lk * 8]);
         __builtin_amdgcn_sched_barrier(0);
         static_for<48>([&](auto tt) {
             constexpr int t = decltype(tt)::value, i = t / 12, j = (t % 12) / 6, p = t % 6;
@@ -897,16 +927,19 @@ __global__ __launch_bounds__(kBigThreads) void gemm_bf16x3_big_kernel(float* c, 
             constexpr int pb = p == 0 ? 1 : p == 1 ? 2 : p == 2 ? 0 : p == 3 ? 1 : p == 4 ? 0 : 0;
             acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(av[i][pa], bv[j][pb], acc[i][j], 0, 0, 0);
             if constexpr (t < 9) av[1 + t / 3][t % 3] = *reinterpret_cast<const bf16x8*>(&As[cur][t % 3][wm + (1 + t / 3) * 32 + lm][lk * 8]);
-            if constexpr (t >= 16 && t < 32) sa.template piece<t - 16>(ra, As[cur ^ 1]);   // pieces 0-15 cut A, 16-31 cut B
-            if constexpr (t >= 32) sb.template piece<t - 32>(rb, Bs[cur ^ 1]);
+            if constexpr (t >= 8 && t < 24) sa.template piece<t - 8>(ra, As[cur ^ 1]);
+            if constexpr (t >= 24 && t < 40) sb.template piece<t - 24>(rb, Bs[cur ^ 1]);
+            if constexpr (t == 24 && FETCH != 0) sa.template load<FETCH == 2>(k_fetch, K, ra);
+            if constexpr (t == 40 && FETCH != 0) sb.template load<FETCH == 2>(k_fetch, K, rb);
             __builtin_amdgcn_sched_barrier(0);
         });
-        __syncthreads();
+        lds_barrier();
         cur ^= 1;
     };
-    // K steps 1 .. nsteps - 2 are whole
-    for (int64_t s = 0; s + 2 < nsteps; s++) k_step(std::false_type(), (s + 1) * kX3BK);
-    if (nsteps >= 2) k_step(std::integral_constant<bool, TAIL>(), (nsteps - 1) * kX3BK);
+    // step s (0 <= s <= nsteps - 2) cuts the elements of step s + 1 and requests those of step s + 2; the last request may be a partial step
+    for (int64_t s = 0; s + 3 < nsteps; s++) k_step(std::integral_constant<int, 1>(), (s + 2) * kX3BK);
+    if (nsteps >= 3) k_step(std::integral_constant<int, TAIL ? 2 : 1>(), (nsteps - 1) * kX3BK);
+    if (nsteps >= 2) k_step(std::integral_constant<int, 0>(), 0);
     compute(cur);
 
     // an element that cannot be cut into bf16 parts was staged by some thread: the four 128 x 128 quarters of the tile are redone on the

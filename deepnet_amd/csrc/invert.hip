@@ -14,6 +14,7 @@
 // A pivot that is exactly zero marks the matrix singular (LAPACK's info > 0), reported as DNH_ERR_SINGULAR_MATRIX.
 // Floating point only; the work is 2 n^3 flops per matrix, nearly all of it in step 3.
 #include "common.h"
+#include <utility>
 #include "wave_argmax.h"
 
 namespace dnh {
@@ -331,8 +332,10 @@ __global__ __launch_bounds__(256) void invert_extract_g_kernel(const T* __restri
 // The exchanges are first replayed on row numbers (thread 0, at most 2 * NB rows take part: the block's rows and their
 // partners), which gives for every affected row the row its final content comes from; the columns then see one round of
 // independent loads and one round of stores instead of wc dependent round trips.
+// OWN: the block's own columns are exchanged as well (their T stays zero); the panel kernels that eliminate column by column have
+// exchanged them already.
 constexpr int kSwapThreads = 64;
-template <class T>
+template <class T, bool OWN>
 __global__ __launch_bounds__(kSwapThreads) void invert_swap_kernel(T* __restrict__ w, T* __restrict__ tbuf, const int32_t* __restrict__ ipiv,
                                                                    int n, int ld, int kb, int wc, int c_begin, int c_end, int64_t bs_w,
                                                                    int64_t bs_t) {
@@ -349,7 +352,8 @@ __global__ __launch_bounds__(kSwapThreads) void invert_swap_kernel(T* __restrict
     if (c >= c_end) return;
     T* P = w + (int64_t)blockIdx.y * bs_w;
     T* Tb = tbuf + (int64_t)blockIdx.y * bs_t;
-    if (c >= kb && c < kb + wc) {
+    const bool own = c >= kb && c < kb + wc;
+    if (own && !OWN) {
         for (int j = 0; j < wc; j++) Tb[(int64_t)j * ld + c] = T(0);
         return;
     }
@@ -362,7 +366,313 @@ __global__ __launch_bounds__(kSwapThreads) void invert_swap_kernel(T* __restrict
     for (int i = 0; i < 2 * NB; i++)
         if (i < m) {
             if (src[i] != pos[i]) P[(int64_t)pos[i] * ld + c] = val[i];
-            if (i < wc) Tb[(int64_t)i * ld + c] = val[i];
+            if (i < wc) Tb[(int64_t)i * ld + c] = own ? T(0) : val[i];
+        }
+}
+
+// ---- pivots by tournament ---------------------------------------------------------------------------------------------------------
+// Eliminating a panel column by column makes every step wait for a pivot search over all remaining rows, which one workgroup can do
+// at LDS speed but many cannot do at all without a trip through memory per step.  A block Gauss-Jordan step needs less: once the
+// block's NB pivot rows are known and exchanged into place, with P their NB x NB block and C the rest of the panel,
+//     G = [ -C P^-1 ; P^-1 ]    (the rows of P^-1 at the block's rows)
+// is the panel of the product of the NB elimination steps, and every row of it is independent of the others.  The pivot rows are
+// chosen by tournament (communication-avoiding LU): a wavefront holds 64 rows of the panel, one per lane in registers, runs Gaussian
+// elimination with partial pivoting on them without leaving its registers (the largest entry by lane moves, the pivot row read
+// lane by lane into scalars) and names the rows it pivoted on; pairs of wavefronts' choices, 64 rows again with their original
+// values, go through the same elimination, and so on: a workgroup of kTournRows threads reduces its rows to NB, rounds of such
+// workgroups reduce the panel's rows to at most kTournLast, on which one workgroup runs the last games: the pivots of its last
+// wavefront, in their order, are the block's.  Every game picks as partial pivoting picks (largest magnitude; the lowest lane on
+// ties); over several games the growth bound is weaker in theory and as good in practice.  The elimination inside a game only
+// ranks rows, so it multiplies by a reciprocal; P^-1 and G are computed from the original values with true divisions.
+constexpr int kTournRows = 256, kTournLast = 512;
+
+template <class F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>()), ...); }
+template <int N, class F>
+__device__ __forceinline__ void static_for(F&& f) { static_for_impl(f, std::make_integer_sequence<int, N>()); }
+
+template <class T>
+__device__ __forceinline__ T read_lane(T v, int lane) {
+    if constexpr (sizeof(T) == 4) {
+        return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+    } else {
+        const long long b = __double_as_longlong(v);
+        const int lo = __builtin_amdgcn_readlane((int)(unsigned)(b & 0xFFFFFFFFLL), lane);
+        const int hi = __builtin_amdgcn_readlane((int)(b >> 32), lane);
+        return __longlong_as_double(((long long)hi << 32) | (unsigned)lo);
+    }
+}
+
+// The largest value of a wavefront, in every lane.  Values are >= 0 and no NaN, so single precision compares its bit patterns as
+// integers (one instruction per step with the lane move folded in).
+__device__ __forceinline__ float wave_max(float x) {
+    unsigned u = __float_as_uint(x);
+    u = max(u, (unsigned)dpp_move<0x111, 0xF>((int)u));   // row_shr:1
+    u = max(u, (unsigned)dpp_move<0x112, 0xF>((int)u));   // row_shr:2
+    u = max(u, (unsigned)dpp_move<0x114, 0xF>((int)u));   // row_shr:4
+    u = max(u, (unsigned)dpp_move<0x118, 0xF>((int)u));   // row_shr:8
+    u = max(u, (unsigned)dpp_move<0x142, 0xA>((int)u));   // row_bcast:15 into rows 1 and 3
+    u = max(u, (unsigned)dpp_move<0x143, 0xC>((int)u));   // row_bcast:31 into rows 2 and 3
+    return __uint_as_float((unsigned)__builtin_amdgcn_readlane((int)u, 63));
+}
+__device__ __forceinline__ double wave_max(double x) {
+    x = __builtin_fmax(x, dpp_move<0x111, 0xF>(x));
+    x = __builtin_fmax(x, dpp_move<0x112, 0xF>(x));
+    x = __builtin_fmax(x, dpp_move<0x114, 0xF>(x));
+    x = __builtin_fmax(x, dpp_move<0x118, 0xF>(x));
+    x = __builtin_fmax(x, dpp_move<0x142, 0xA>(x));
+    x = __builtin_fmax(x, dpp_move<0x143, 0xC>(x));
+    return read_lane(x, 63);
+}
+__device__ __forceinline__ float fma_of(float a, float b, float c) { return __builtin_fmaf(a, b, c); }
+__device__ __forceinline__ double fma_of(double a, double b, double c) { return __builtin_fma(a, b, c); }
+// 1 / x to within a few units of the last place: the games only rank rows with it.
+__device__ __forceinline__ float quick_rcp(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ double quick_rcp(double x) {
+    const double r = __builtin_amdgcn_rcp(x);
+    return r * (2.0 - x * r);
+}
+
+// A thread's row of the panel (live threads), zeros beyond the panel's width.
+template <class T>
+__device__ __forceinline__ void tourn_load_row(T (&v)[NB], const T* P, bool live, int id, int ld, int kb, int wc) {
+    typedef T vec4 __attribute__((ext_vector_type(4)));   // rows start 16-byte aligned (ld and kb are multiples of 4)
+    if (wc == NB) {
+        const vec4* src = reinterpret_cast<const vec4*>(P + (int64_t)(live ? id : 0) * ld + kb);
+#pragma unroll
+        for (int q = 0; q < NB / 4; q++) {
+            const vec4 x = src[q];
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[q * 4 + e] = live ? x[e] : T(0);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < NB; j++) v[j] = (live && j < wc) ? P[(int64_t)id * ld + kb + j] : T(0);
+    }
+}
+
+// One game: Gaussian elimination with partial pivoting over the 64 rows a wavefront holds (v: the row, destroyed; live: the lane
+// holds a row).  Returns the step at which this lane's row was pivoted on, or -1.  A column without a non-zero entry among the rows
+// left has no pivot: its step is nobody's.
+template <class T>
+__device__ __forceinline__ int tourn_game(T (&v)[NB], bool live, int wc) {
+    int mine = -1;
+    static_for<NB>([&](auto kk) {
+        constexpr int k = decltype(kk)::value;
+        if (k >= wc) return;
+        T a = abs_of(v[k]);
+        a = (live && a > T(0)) ? a : T(0);           // NaN and rows already used never win
+        const T top = wave_max(a);
+        if (!(top > T(0))) return;                   // same in every lane
+        const int owner = __builtin_ctzll(__ballot(a == top));
+        T pr[NB];
+#pragma unroll
+        for (int j = k; j < NB; j++) pr[j] = read_lane(v[j], owner);
+        if ((int)(threadIdx.x & 63) == owner) {
+            live = false;
+            mine = k;
+        }
+        const T m = live ? -v[k] * quick_rcp(pr[k]) : T(0);
+#pragma unroll
+        for (int j = k + 1; j < NB; j++) v[j] = fma_of(m, pr[j], v[j]);
+    });
+    return mine;
+}
+
+// The games of one workgroup of WAVES wavefronts (a power of two): every wavefront plays its 64 rows (orig: the row, id: its number, -1
+// for none), the winners' original rows go to LDS, half as many wavefronts take two wavefronts' winners each, until one wavefront is
+// left.  Afterwards rows[k] / ids[k] of group 0 hold the pivot row of step k (ids: -1 where a step found none).
+template <class T, int WAVES>
+struct TournShared {
+    __align__(16) T rows[WAVES][NB][NB];
+    int ids[WAVES][NB];
+};
+template <class T, int WAVES>
+__device__ __forceinline__ void tourn_play(T (&orig)[NB], int id, int wc, TournShared<T, WAVES>& sh) {
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+#pragma unroll 1
+    for (int active = WAVES;; active >>= 1) {   // one copy of the game's code: three would not fit the instruction cache
+        if (wave < active) {
+            T v[NB];
+#pragma unroll
+            for (int j = 0; j < NB; j++) v[j] = orig[j];
+            if (lane < NB) sh.ids[wave][lane] = -1;
+            const int mine = tourn_game(v, id >= 0, wc);
+            if (mine >= 0) {
+                sh.ids[wave][mine] = id;
+#pragma unroll
+                for (int q = 0; q < NB / 4; q++)
+                    *reinterpret_cast<vec4*>(&sh.rows[wave][mine][q * 4]) = vec4{orig[q * 4], orig[q * 4 + 1], orig[q * 4 + 2], orig[q * 4 + 3]};
+            }
+        }
+        if (active == 1) break;
+        __syncthreads();
+        if (wave < active / 2) {
+            const int from = 2 * wave + (lane >> 5), slot = lane & 31;
+            id = sh.ids[from][slot];
+#pragma unroll
+            for (int q = 0; q < NB / 4; q++) {
+                const vec4 x = *reinterpret_cast<const vec4*>(&sh.rows[from][slot][q * 4]);
+#pragma unroll
+                for (int e = 0; e < 4; e++) orig[q * 4 + e] = x[e];
+            }
+        }
+        __syncthreads();   // the winners of the next games overwrite what has just been read
+    }
+}
+
+// One round: workgroup x elects among rows [x * kTournRows, (x + 1) * kTournRows) of the round's list (rows_in, or the rows from kb
+// on when it is null) and writes NB row numbers (-1: none) to rows_out.
+template <class T>
+__global__ __launch_bounds__(kTournRows) void invert_tourn_round_kernel(const T* __restrict__ w, const int32_t* __restrict__ rows_in, int count,
+                                                                       int32_t* __restrict__ rows_out, int ld, int kb, int wc, int64_t bs_w,
+                                                                       int64_t bs_rows) {
+    __shared__ TournShared<T, kTournRows / 64> sh;
+    const T* P = w + (int64_t)blockIdx.y * bs_w;
+    const int t = blockIdx.x * kTournRows + threadIdx.x;
+    int id = -1;
+    if (t < count) id = rows_in ? rows_in[(int64_t)blockIdx.y * bs_rows + t] : kb + t;
+    T orig[NB];
+    tourn_load_row(orig, P, id >= 0, id, ld, kb, wc);
+    tourn_play(orig, id, wc, sh);
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    if (threadIdx.x < NB) rows_out[(int64_t)blockIdx.y * bs_rows + blockIdx.x * NB + threadIdx.x] = threadIdx.x < wc ? sh.ids[0][threadIdx.x] : -1;
+}
+
+// The last round: elects the block's pivot rows among at most kTournLast rows, records them as the exchanges of steps kb .. kb + wc - 1
+// (ipiv[kb + k] = the position row k's content has reached when its turn comes) and inverts their wc x wc block (Gauss-Jordan in
+// the order of election, whose pivots are the elimination's own) into pinv (NB x NB per matrix, row-major).  The bookkeeping and the
+// inversion are the first wavefront's alone, in registers: lane j keeps exchange j, lane (h, j) keeps rows 16 h .. 16 h + 15 of
+// column j, so neither needs a barrier.
+template <class T>
+__global__ __launch_bounds__(kTournLast) void invert_tourn_last_kernel(const T* __restrict__ w, const int32_t* __restrict__ rows_in, int count,
+                                                                      int32_t* __restrict__ ipiv, T* __restrict__ pinv, int32_t* singular, int n,
+                                                                      int ld, int kb, int wc, int64_t bs_w, int64_t bs_rows) {
+    static_assert(NB == 32, "the single-wavefront inversion holds a 32 x 32 block");
+    extern __shared__ __align__(16) unsigned char tourn_lds[];
+    typedef TournShared<T, kTournLast / 64> Shared;
+    Shared& sh = *reinterpret_cast<Shared*>(tourn_lds);
+    const T* P = w + (int64_t)blockIdx.x * bs_w;
+    const int tid = threadIdx.x;
+    {
+        int id = -1;
+        if (tid < count) id = rows_in ? rows_in[(int64_t)blockIdx.x * bs_rows + tid] : kb + tid;
+        T orig[NB];
+        tourn_load_row(orig, P, id >= 0, id, ld, kb, wc);
+        tourn_play(orig, id, wc, sh);
+    }
+    if (tid >= 64) return;
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    const int lane = tid;
+    int* ids = sh.ids[0];
+    if (__ballot(lane < wc && ids[lane] < 0)) {
+        // a column without a pivot: the matrix is singular; rows nobody elected keep the bookkeeping consistent (their panel entries
+        // stand in for the missing pivot rows)
+        if (lane == 0) {
+            *singular = 1;
+            for (int k = 0; k < wc; k++) {
+                if (ids[k] >= 0) continue;
+                for (int g = kb; g < n; g++) {
+                    bool taken = false;
+                    for (int j = 0; j < wc; j++) taken |= ids[j] == g;
+                    if (!taken) { ids[k] = g; break; }
+                }
+                for (int j = 0; j < wc; j++) sh.rows[0][k][j] = P[(int64_t)ids[k] * ld + kb + j];
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+    const int sel = lane < wc ? ids[lane] : -1;
+    int partner = 0;   // lane k: where the content of elected row k sits after the exchanges of steps 0 .. k - 1
+    for (int k = 0; k < wc; k++) {
+        int pos = __builtin_amdgcn_readlane(sel, k);
+        // exchange j moves the row when it sits at kb + j or at partner[j]; the exchanges are looked at in order, few ever match
+        unsigned long long later = ~0ull;
+        while (true) {
+            const unsigned long long hit = __ballot(lane < k && (partner == pos || kb + lane == pos)) & later;
+            if (!hit) break;
+            const int jj = __builtin_ctzll(hit);
+            const int pj = __builtin_amdgcn_readlane(partner, jj);
+            pos = (pos == kb + jj) ? pj : kb + jj;
+            later = ~0ull << (jj + 1);   // jj <= 30
+        }
+        if (lane == k) partner = pos;
+    }
+    if (lane < wc) ipiv[(int64_t)blockIdx.x * n + kb + lane] = partner;
+
+    const int j = lane & 31, h = lane >> 5;
+    T a[16];
+#pragma unroll
+    for (int ii = 0; ii < 16; ii++) {
+        const int i = h * 16 + ii;
+        a[ii] = (i < wc && j < wc) ? sh.rows[0][i][j] : (i == j ? T(1) : T(0));
+    }
+    static_for<NB>([&](auto kk) {
+        constexpr int k = decltype(kk)::value, kr = k % 16, kh = k / 16;
+        if (k >= wc) return;
+        const T pv = read_lane(a[kr], kh * 32 + k);
+        if (!(abs_of(pv) > T(0)) && lane == 0) *singular = 1;
+        const T rk = __shfl(a[kr], kh * 32 + j, 64);           // the pivot row's entry in this lane's column
+        const T sj = (j == k ? T(1) : rk) / pv;                // the pivot row, scaled: 1 / pivot where the pivot was
+        T f[16];
+#pragma unroll
+        for (int ii = 0; ii < 16; ii++) f[ii] = __shfl(a[ii], h * 32 + k, 64);   // every row's entry in the pivot column
+#pragma unroll
+        for (int ii = 0; ii < 16; ii++) {
+            const bool pivot_row = (ii == kr) && (h == kh);
+            a[ii] = pivot_row ? sj : ((j == k) ? T(0) : a[ii]) - f[ii] * sj;
+        }
+    });
+#pragma unroll
+    for (int ii = 0; ii < 16; ii++) {
+        const int i = h * 16 + ii;
+        pinv[(int64_t)blockIdx.x * NB * NB + i * NB + j] = (i < wc && j < wc) ? a[ii] : T(0);
+    }
+}
+
+// After the exchanges: the panel becomes G (row r of the block's rows: row r - kb of P^-1; any other row: minus its panel entries
+// times P^-1), and gbuf receives G - I_block for the update of the other columns.  Four threads per row, eight columns each.
+constexpr int kTournGThreads = 256;
+template <class T>
+__global__ __launch_bounds__(kTournGThreads) void invert_tourn_g_kernel(T* __restrict__ w, T* __restrict__ gbuf, const T* __restrict__ pinv, int n,
+                                                                        int ld, int kb, int wc, int64_t bs_w, int64_t bs_g) {
+    typedef T vec4 __attribute__((ext_vector_type(4)));
+    __shared__ __align__(16) T pi[NB][NB];
+    for (int e = threadIdx.x; e < NB * NB; e += kTournGThreads) pi[e / NB][e % NB] = pinv[(int64_t)blockIdx.y * NB * NB + e];
+    __syncthreads();
+    const int r = blockIdx.x * (kTournGThreads / 4) + threadIdx.x / 4, c0 = (threadIdx.x & 3) * 8;
+    if (r >= n) return;
+    T* row = w + (int64_t)blockIdx.y * bs_w + (int64_t)r * ld + kb;
+    T out[8];
+    if (r >= kb && r < kb + wc) {
+#pragma unroll
+        for (int j = 0; j < 8; j++) out[j] = pi[r - kb][c0 + j];
+    } else {
+        T c[NB];
+        tourn_load_row(c, w + (int64_t)blockIdx.y * bs_w, true, r, ld, kb, wc);
+#pragma unroll
+        for (int j = 0; j < 8; j++) out[j] = T(0);
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const vec4 p0 = *reinterpret_cast<const vec4*>(&pi[i][c0]), p1 = *reinterpret_cast<const vec4*>(&pi[i][c0 + 4]);
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                out[e] += c[i] * p0[e];
+                out[4 + e] += c[i] * p1[e];
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) out[j] = -out[j];
+    }
+    // every thread of a row has read the row's panel entries before any of them is replaced: the four sit in one wavefront
+    __builtin_amdgcn_wave_barrier();
+    T* g = gbuf + (int64_t)blockIdx.y * bs_g + (int64_t)r * NB;
+#pragma unroll
+    for (int j = 0; j < 8; j++)
+        if (c0 + j < wc) {
+            row[c0 + j] = out[j];
+            g[c0 + j] = out[j] - ((r == kb + c0 + j) ? T(1) : T(0));
         }
 }
 
@@ -423,8 +733,14 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
     const size_t sz_w = align_up((size_t)batch * bs_w * sizeof(T)), sz_g = align_up((size_t)batch * bs_g * sizeof(T));
     const size_t sz_t = align_up((size_t)batch * bs_t * sizeof(T)), sz_i = align_up((size_t)batch * n * sizeof(int32_t));
     const size_t sz_r = t_is_c ? 0 : align_up((size_t)batch * n * n * sizeof(T));
+    // pivots by tournament: two lists of candidate rows (NB per workgroup of the first round) and the inverted pivot block
+    const int tourn_opt = option(OPT_INVERT_TOURNAMENT);
+    const bool tourn = tourn_opt == 1 || (tourn_opt < 0 && n >= 1024);
+    const int64_t bs_rows = (int64_t)cdiv(n, kTournRows) * NB;
+    const size_t sz_rows = tourn ? align_up((size_t)batch * bs_rows * sizeof(int32_t)) : 0;
+    const size_t sz_pinv = tourn ? align_up((size_t)batch * NB * NB * sizeof(T)) : 0;
     void* block = nullptr;
-    DNH_TRY(dnh_alloc_async(sz_w + 2 * sz_g + sz_t + 2 * sz_i + sz_r + 256, stream, &block));
+    DNH_TRY(dnh_alloc_async(sz_w + 2 * sz_g + sz_t + 2 * sz_i + sz_r + 256 + 2 * sz_rows + sz_pinv, stream, &block));
     char* base = (char*)block;
     T* W = (T*)base;
     T* G = (T*)(base + sz_w);
@@ -434,6 +750,9 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
     T* R = t_is_c ? (T*)elem_ptr(t) : (T*)(base + sz_w + sz_g + sz_t + 2 * sz_i);
     int32_t* flag = (int32_t*)(base + sz_w + sz_g + sz_t + 2 * sz_i + sz_r);
     T* Gs = (T*)(base + sz_w + sz_g + sz_t + 2 * sz_i + sz_r + 256);   // sub-panel multipliers (n x sb per matrix, sb <= NB)
+    int32_t* rows_a = (int32_t*)(base + sz_w + 2 * sz_g + sz_t + 2 * sz_i + sz_r + 256);
+    int32_t* rows_b = (int32_t*)((char*)rows_a + sz_rows);
+    T* pinv = (T*)((char*)rows_a + 2 * sz_rows);
 
     int32_t st = DNH_OK;
     auto body = [&]() -> int32_t {
@@ -478,8 +797,32 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
 #undef DNH_SUBPANEL
             return DNH_OK;
         };
+        const size_t tourn_lds = sizeof(TournShared<T, kTournLast / 64>);
+        if (tourn && tourn_lds > 32 * 1024)
+            DNH_HIP(hipFuncSetAttribute((const void*)invert_tourn_last_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tourn_lds));
         for (int kb = 0; kb < n; kb += NB) {
             const int wc = (n - kb < NB) ? n - kb : NB;
+            if (tourn) {
+                int count = n - kb;
+                const int32_t* rows_in = nullptr;
+                int32_t* rows_out = rows_a;
+                while (count > kTournLast) {
+                    const int chunks = (int)cdiv(count, kTournRows);
+                    hipLaunchKernelGGL((invert_tourn_round_kernel<T>), dim3((unsigned)chunks, (unsigned)batch), dim3(kTournRows), 0, stream, W,
+                                       rows_in, count, rows_out, ld, kb, wc, bs_w, bs_rows);
+                    count = chunks * NB;
+                    rows_in = rows_out;
+                    rows_out = rows_out == rows_a ? rows_b : rows_a;
+                }
+                hipLaunchKernelGGL((invert_tourn_last_kernel<T>), dim3((unsigned)batch), dim3(kTournLast), tourn_lds, stream, W, rows_in, count, ipiv,
+                                   pinv, flag, n, ld, kb, wc, bs_w, bs_rows);
+                hipLaunchKernelGGL((invert_swap_kernel<T, true>), dim3((unsigned)cdiv(n, kSwapThreads), (unsigned)batch), dim3(kSwapThreads), 0,
+                                   stream, W, Tb, ipiv, n, ld, kb, wc, 0, n, bs_w, bs_t);
+                hipLaunchKernelGGL((invert_tourn_g_kernel<T>), dim3((unsigned)cdiv(n, kTournGThreads / 4), (unsigned)batch), dim3(kTournGThreads), 0,
+                                   stream, W, G, pinv, n, ld, kb, wc, bs_w, bs_g);
+                if (n > wc) DNH_TRY(gemm_accumulate(t->dtype, W, G, Tb, n, n, wc, NB, ld, ld, batch, bs_g, bs_t, bs_w, stream));
+                continue;
+            }
             if (sb == NB) {
                 DNH_TRY(launch_subpanel(NB, G, kb, wc, NB, kb, wc));
             } else if (sb > 0) {
@@ -497,7 +840,7 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
                                    bs_w, bs_g);
             }
             if (n > wc) {
-                hipLaunchKernelGGL((invert_swap_kernel<T>), dim3((unsigned)cdiv(n, kSwapThreads), (unsigned)batch), dim3(kSwapThreads), 0, stream,
+                hipLaunchKernelGGL((invert_swap_kernel<T, false>), dim3((unsigned)cdiv(n, kSwapThreads), (unsigned)batch), dim3(kSwapThreads), 0, stream,
                                    W, Tb, ipiv, n, ld, kb, wc, 0, n, bs_w, bs_t);
                 DNH_TRY(gemm_accumulate(t->dtype, W, G, Tb, n, n, wc, NB, ld, ld, batch, bs_g, bs_t, bs_w, stream));
             }

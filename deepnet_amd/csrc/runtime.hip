@@ -140,6 +140,7 @@ constexpr OptionDef kOptions[OPT_COUNT] = {
     {"dot_int_mfma", 1, 0, 1},     {"tr4", 1, 0, 1},               {"scatter_fp_atomic", 0, 0, 1},  {"compact_one_pass", 0, 0, 1},
     {"count_one_launch", 1, 0, 1},
     {"lookback_spins", 1 << 18, 0, 1 << 30},
+    {"invert_tournament", -1, -1, 1},
 };
 std::atomic<int> g_options[OPT_COUNT];
 std::once_flag g_options_once;

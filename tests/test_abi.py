@@ -84,7 +84,8 @@ def test_status_codes_map_to_reference_exception_kinds():
 def test_options_are_set_and_read_without_a_device():
     """dnh_set_option / dnh_get_option touch no GPU: defaults, round trip, refusal of unknown names and of values out of range."""
     defaults = {"dot_bf16x3": 1, "dot_f64_pinned": 1, "dot_big": -1, "dot_splits": 0, "dot_int_mfma": 1, "tr4": 1,
-                "scatter_fp_atomic": 0, "compact_one_pass": 0, "count_one_launch": 1, "lookback_spins": 1 << 18}
+                "scatter_fp_atomic": 0, "compact_one_pass": 0, "count_one_launch": 1, "lookback_spins": 1 << 18,
+                "invert_tournament": -1}
     header = open(HEADER).read()
     for name, value in defaults.items():
         assert f'"{name}"' in header, f"include/tensor_hip.h does not document option {name}"

@@ -26,7 +26,9 @@ def check_dot(ref, got, a, b):
 
 
 @pytest.mark.parametrize("dt", [np.float32, np.float64])
-@pytest.mark.parametrize("m,k,n", [(5, 3, 3), (128, 16, 128), (128, 512, 128), (256, 64, 384), (130, 70, 50), (1, 1, 1), (33, 1000, 7)])
+@pytest.mark.parametrize("m,k,n", [(5, 3, 3), (128, 16, 128), (128, 512, 128), (256, 64, 384), (130, 70, 50), (1, 1, 1), (33, 1000, 7),
+                                     # one, two, three and four K steps of 16 with a partial last one (the fetches run two steps ahead)
+                                     (256, 20, 256), (64, 31, 300), (200, 33, 100), (300, 47, 260), (257, 49, 129)])
 def test_matmat(H, G, rng, dt, m, k, n, tile_form):
     a = rng.standard_normal((m, k)).astype(dt)
     b = rng.standard_normal((k, n)).astype(dt)
@@ -434,7 +436,8 @@ def test_fp32_instruction_kernel_behind_the_switch(G):
 
 @pytest.mark.parametrize("ta,tb", STAGINGS)
 @pytest.mark.parametrize("m,k,n", [(4096, 48, 4096),     # 256 tiles of 256 x 256: the large-tile kernel by the library's own choice
-                                   (4000, 40, 4090)])    # edge tiles on both sides and a partial last K step
+                                   (4000, 40, 4090),     # edge tiles on both sides and a partial last K step
+                                   (4090, 24, 4000)])    # two K steps, the second partial: fetched before the loop starts
 def test_single_precision_large_tiles(G, rng, ta, tb, m, k, n):
     """Products with at least a CU's worth of 256 x 256 tiles run the large-tile form of the bf16-parts kernel: same parts, same six
     products, so the same 16 u S; an infinite element sends its tile to the fp32 instructions, quarter by quarter."""

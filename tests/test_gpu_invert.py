@@ -11,7 +11,16 @@ from invert_cases import hilbert, hilbert_inverse, inverse_error_bound, invert, 
 pytestmark = pytest.mark.gpu
 
 
-def test_doc_example_and_fixture(H, G):
+@pytest.fixture(params=[-1, 1], ids=["own_choice", "tournament"])
+def pivot_form(request):
+    """Runs a test once with the library's own choice of how a panel's pivots are found (column by column in one workgroup below
+    1024 rows) and once with the tournament form for every size."""
+    from deepnet_amd import native
+    with native.option("invert_tournament", request.param):
+        yield request.param
+
+
+def test_doc_example_and_fixture(H, G, pivot_form):
     got = invert(G, np.array([[1.0, 2.0], [3.0, 4.0]]))
     np.testing.assert_allclose(got, [[-2.0, 1.0], [1.5, -0.5]], rtol=0, atol=2e-15)   # cond = 15, a few ulp
     kk, chk = kk_fixture()
@@ -23,7 +32,7 @@ def test_doc_example_and_fixture(H, G):
     assert np.abs(G.toNumpy(kkinv) - ref).max() <= 20 * 50 * 2 ** -23 * np.abs(ref).max()
 
 
-def test_singular_matrix_raises(G):
+def test_singular_matrix_raises(G, pivot_form):
     with pytest.raises(SingularMatrixException):
         invert(G, np.array([[1.0, 0.0, 0.0], [1.0, 2.0, 0.0], [1.0, 0.0, 0.0]]))               # BaseTests.fs:204-211
     with pytest.raises(SingularMatrixException):
@@ -32,7 +41,7 @@ def test_singular_matrix_raises(G):
     np.testing.assert_array_equal(invert(G, np.eye(5)), np.eye(5))
 
 
-def test_exact_cases(G, rng):
+def test_exact_cases(G, rng, pivot_form):
     d = rng.uniform(0.5, 8.0, 70).astype(np.float32)
     np.testing.assert_array_equal(invert(G, np.diag(d)), np.diag(np.float32(1) / d))
     for n in (23, 64, 100):
@@ -47,8 +56,9 @@ def test_exact_cases(G, rng):
 
 
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
-@pytest.mark.parametrize("shape", [(1, 1), (2, 2), (31, 31), (32, 32), (33, 33), (3, 64, 64), (2, 3, 50, 50), (130, 130), (257, 257), (2, 500, 500)])
-def test_against_oracle_and_fp64(H, G, rng, dtype, shape):
+@pytest.mark.parametrize("shape", [(1, 1), (2, 2), (31, 31), (32, 32), (33, 33), (3, 64, 64), (2, 3, 50, 50), (130, 130), (257, 257), (2, 500, 500),
+                                   (2, 600, 600), (1100, 1100)])   # more rows than the tournament's last round takes: two rounds
+def test_against_oracle_and_fp64(H, G, rng, dtype, shape, pivot_form):
     a = well_conditioned(rng, shape, dtype)
     got = invert(G, a)
     ref = invert(H, a)
@@ -59,7 +69,7 @@ def test_against_oracle_and_fp64(H, G, rng, dtype, shape):
     assert np.all(np.abs(got.astype(np.float64) - ref.astype(np.float64)) <= 2 * bound)
 
 
-def test_pivoting_layouts_inplace_broadcast(H, G, rng):
+def test_pivoting_layouts_inplace_broadcast(H, G, rng, pivot_form):
     a = well_conditioned(rng, (70, 70), np.float64)
     a = a * (1 - np.eye(70)) + np.roll(np.eye(70), 1, axis=1) * 3            # zero diagonal
     got = invert(G, a)
@@ -94,10 +104,33 @@ def test_argument_errors(G):
     assert invert(G, np.zeros((0, 3, 3))).shape == (0, 3, 3)
 
 
-def test_large_matrix_by_identity(G, rng):
+def test_large_matrix_by_identity(G, rng, pivot_form):
     """1000 x 1000 single (a size of the reference's benchmark): inv(A) . A = I within n eps cond."""
     n = 1000
     a = (rng.standard_normal((n, n)) / np.sqrt(n) + 2 * np.eye(n)).astype(np.float32)
     ta = G.ofNumpy(a)
     prod = G.toNumpy(Tensor.invert(ta) @ ta)
     assert np.abs(prod - np.eye(n)).max() <= 8 * n * 2 ** -23 * np.linalg.cond(a.astype(np.float64))
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_tournament_pivots(G, rng, dtype):
+    """What the tournament has to get right beyond accuracy on friendly matrices: a panel whose large entries sit in few rows (every
+    workgroup of the first round must hand on more than its first choice), an entry that
+    dwarfs its column, and a singular matrix with a column of zeros."""
+    from deepnet_amd import native
+    n = 700
+    with native.option("invert_tournament", 1):
+        a = well_conditioned(rng, (n, n), dtype).astype(np.float64)
+        a[300:340] *= 1e3                                   # forty rows carry every column's largest entries
+        a[17, 5] = 1e6
+        a = a.astype(dtype)
+        got = invert(G, a)
+        inv, bound = inverse_error_bound(a, factor=32.0)
+        assert np.all(np.abs(got - inv) <= bound), float((np.abs(got - inv) / bound).max())
+        z = a.copy()
+        z[:, 40] = 0
+        with pytest.raises(SingularMatrixException):
+            invert(G, z)
+        # the games are deterministic: the same bits every time
+        np.testing.assert_array_equal(invert(G, a), got)
