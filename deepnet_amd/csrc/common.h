@@ -95,7 +95,7 @@ enum Option {
     OPT_COMPACT_ONE_PASS,    // 1: maskedGet / maskedSet / trueIndices of contiguous masks in one launch; 0: count + move launches
     OPT_COUNT_ONE_LAUNCH,    // 1: countTrue of a whole contiguous mask in one launch (arrival counters); 0: the general two-pass fold
     OPT_LOOKBACK_SPINS,      // polls a one-pass compaction's tile spends on predecessors that have not published before it counts for itself
-    OPT_INVERT_TOURNAMENT,   // -1: matrices of 1024 rows and more pick a panel's pivots by tournament; 0: never; 1: always
+    OPT_INVERT_TOURNAMENT,   // -1: matrices of more than 32 rows pick a panel's pivots by tournament; 0: never; 1: always
     OPT_COUNT
 };
 int option(Option o);

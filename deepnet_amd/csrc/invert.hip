@@ -13,7 +13,12 @@
 //   finally the row exchanges are undone as column exchanges in reverse order (composed into one permutation, one pass).
 // A pivot that is exactly zero marks the matrix singular (LAPACK's info > 0), reported as DNH_ERR_SINGULAR_MATRIX.
 // Floating point only; the work is 2 n^3 flops per matrix, nearly all of it in step 3.
+// Matrices of more than NB rows replace step 1 by a tournament for the block's pivot rows followed by G = [-C P^-1; P^-1] from the
+// exchanged panel (further down: "pivots by tournament"): no step of it waits for a search over all rows, and the update of the
+// columns the next block's tournament does not need runs beside that tournament on a second stream.  The option invert_tournament
+// forces either form.
 #include "common.h"
+#include <mutex>
 #include <utility>
 #include "wave_argmax.h"
 
@@ -376,16 +381,14 @@ __global__ __launch_bounds__(kSwapThreads) void invert_swap_kernel(T* __restrict
 // block's NB pivot rows are known and exchanged into place, with P their NB x NB block and C the rest of the panel,
 //     G = [ -C P^-1 ; P^-1 ]    (the rows of P^-1 at the block's rows)
 // is the panel of the product of the NB elimination steps, and every row of it is independent of the others.  The pivot rows are
-// chosen by tournament (communication-avoiding LU): a wavefront holds 64 rows of the panel, one per lane in registers, runs Gaussian
-// elimination with partial pivoting on them without leaving its registers (the largest entry by lane moves, the pivot row read
-// lane by lane into scalars) and names the rows it pivoted on; pairs of wavefronts' choices, 64 rows again with their original
-// values, go through the same elimination, and so on: a workgroup of kTournRows threads reduces its rows to NB, rounds of such
-// workgroups reduce the panel's rows to at most kTournLast, on which one workgroup runs the last games: the pivots of its last
-// wavefront, in their order, are the block's.  Every game picks as partial pivoting picks (largest magnitude; the lowest lane on
-// ties); over several games the growth bound is weaker in theory and as good in practice.  The elimination inside a game only
-// ranks rows, so it multiplies by a reciprocal; P^-1 and G are computed from the original values with true divisions.
-constexpr int kTournRows = 256, kTournLast = 512;
-
+// chosen by tournament (communication-avoiding LU).  A game is one wavefront's: it holds 64 R rows of the panel, R per lane in
+// registers, runs Gaussian elimination with partial pivoting on them without leaving its registers (the largest entry by lane moves,
+// the pivot row read lane by lane into scalars) and names the NB rows it pivoted on.  Rounds of games on kTournRows rows each reduce
+// the panel's rows to at most kTournLast, on which one workgroup plays four games and a last one among their winners, always on the
+// rows' original values: the last game's pivots, in their order, are the block's.  Every game picks as partial pivoting picks
+// (largest magnitude; the lowest lane on ties); over several games the growth bound is weaker in theory and as good in practice.
+// The elimination inside a game only ranks rows, so it multiplies by a reciprocal and fuses multiply and add; P^-1 and G are computed
+// from the original values with true divisions.
 template <class F, int... I>
 __device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) { (f(std::integral_constant<int, I>()), ...); }
 template <int N, class F>
@@ -451,124 +454,128 @@ __device__ __forceinline__ void tourn_load_row(T (&v)[NB], const T* P, bool live
     }
 }
 
-// One game: Gaussian elimination with partial pivoting over the 64 rows a wavefront holds (v: the row, destroyed; live: the lane
-// holds a row).  Returns the step at which this lane's row was pivoted on, or -1.  A column without a non-zero entry among the rows
-// left has no pivot: its step is nobody's.
-template <class T>
-__device__ __forceinline__ int tourn_game(T (&v)[NB], bool live, int wc) {
-    int mine = -1;
+// One game: Gaussian elimination with partial pivoting over the 64 R rows a wavefront holds, R per lane in registers (v: the rows,
+// destroyed; id: their numbers, negative for none).  mine[r] receives the step at which the lane's row r was pivoted on, or -1.  A
+// column without a non-zero entry among the rows left has no pivot: its step is nobody's.
+template <class T, int R>
+__device__ __forceinline__ void tourn_game(T (&v)[R][NB], const int (&id)[R], int wc, int (&mine)[R]) {
+    const int lane = threadIdx.x & 63;
+    T lv[R];   // 1 while the row is in the game, 0 once it was pivoted on (or was never there): a factor, not a branch
+#pragma unroll
+    for (int r = 0; r < R; r++) {
+        lv[r] = id[r] >= 0 ? T(1) : T(0);
+        mine[r] = -1;
+    }
     static_for<NB>([&](auto kk) {
         constexpr int k = decltype(kk)::value;
         if (k >= wc) return;
-        T a = abs_of(v[k]);
-        a = (live && a > T(0)) ? a : T(0);           // NaN and rows already used never win
-        const T top = wave_max(a);
-        if (!(top > T(0))) return;                   // same in every lane
-        const int owner = __builtin_ctzll(__ballot(a == top));
+        T a[R], amax = T(0);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            a[r] = abs_of(v[r][k]) * lv[r];
+            amax = max(amax, a[r]);                            // a NaN is passed over
+        }
+        const T top = wave_max(amax);
+        if (!(top > T(0))) return;                             // same in every lane
+        const int owner = __builtin_ctzll(__ballot(amax == top));
+        int rs = 0;
+#pragma unroll
+        for (int r = R - 1; r >= 0; r--) rs = (a[r] == top) ? r : rs;
+        const int rsel = R == 1 ? 0 : __builtin_amdgcn_readlane(rs, owner);
         T pr[NB];
+        static_for<R>([&](auto rr) {
+            constexpr int r = decltype(rr)::value;
+            if (rsel != r) return;                             // same in every lane
 #pragma unroll
-        for (int j = k; j < NB; j++) pr[j] = read_lane(v[j], owner);
-        if ((int)(threadIdx.x & 63) == owner) {
-            live = false;
-            mine = k;
+            for (int j = k; j < NB; j++) pr[j] = read_lane(v[r][j], owner);
+            lv[r] = lane == owner ? T(0) : lv[r];
+            mine[r] = lane == owner ? k : mine[r];
+        });
+        const T rinv = -quick_rcp(pr[k]);
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            const T m = v[r][k] * rinv * lv[r];
+#pragma unroll
+            for (int j = k + 1; j < NB; j++) v[r][j] = fma_of(m, pr[j], v[r][j]);
         }
-        const T m = live ? -v[k] * quick_rcp(pr[k]) : T(0);
-#pragma unroll
-        for (int j = k + 1; j < NB; j++) v[j] = fma_of(m, pr[j], v[j]);
     });
-    return mine;
 }
 
-// The games of one workgroup of WAVES wavefronts (a power of two): every wavefront plays its 64 rows (orig: the row, id: its number, -1
-// for none), the winners' original rows go to LDS, half as many wavefronts take two wavefronts' winners each, until one wavefront is
-// left.  Afterwards rows[k] / ids[k] of group 0 hold the pivot row of step k (ids: -1 where a step found none).
-template <class T, int WAVES>
-struct TournShared {
-    __align__(16) T rows[WAVES][NB][NB];
-    int ids[WAVES][NB];
-};
-template <class T, int WAVES>
-__device__ __forceinline__ void tourn_play(T (&orig)[NB], int id, int wc, TournShared<T, WAVES>& sh) {
-    typedef T vec4 __attribute__((ext_vector_type(4)));
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-#pragma unroll 1
-    for (int active = WAVES;; active >>= 1) {   // one copy of the game's code: three would not fit the instruction cache
-        if (wave < active) {
-            T v[NB];
+// A wavefront's game on entries [first, first + 64 R) of a list of `count` rows (list: row numbers, negative for none; null: the rows
+// from kb on), lane l taking entries first + l, first + 64 + l, ...; the winners' row numbers go to out[0 .. NB) (-1 where a step
+// found none).  out is written by this wavefront only.
+template <class T, int R>
+__device__ __forceinline__ void tourn_play(const T* P, const int32_t* list, int first, int count, int ld, int kb, int wc, int* out) {
+    const int lane = threadIdx.x & 63;
+    int id[R];
+    T v[R][NB];
 #pragma unroll
-            for (int j = 0; j < NB; j++) v[j] = orig[j];
-            if (lane < NB) sh.ids[wave][lane] = -1;
-            const int mine = tourn_game(v, id >= 0, wc);
-            if (mine >= 0) {
-                sh.ids[wave][mine] = id;
-#pragma unroll
-                for (int q = 0; q < NB / 4; q++)
-                    *reinterpret_cast<vec4*>(&sh.rows[wave][mine][q * 4]) = vec4{orig[q * 4], orig[q * 4 + 1], orig[q * 4 + 2], orig[q * 4 + 3]};
-            }
-        }
-        if (active == 1) break;
-        __syncthreads();
-        if (wave < active / 2) {
-            const int from = 2 * wave + (lane >> 5), slot = lane & 31;
-            id = sh.ids[from][slot];
-#pragma unroll
-            for (int q = 0; q < NB / 4; q++) {
-                const vec4 x = *reinterpret_cast<const vec4*>(&sh.rows[from][slot][q * 4]);
-#pragma unroll
-                for (int e = 0; e < 4; e++) orig[q * 4 + e] = x[e];
-            }
-        }
-        __syncthreads();   // the winners of the next games overwrite what has just been read
+    for (int r = 0; r < R; r++) {
+        const int e = first + r * 64 + lane;
+        id[r] = e < count ? (list ? list[e] : kb + e) : -1;
+        tourn_load_row(v[r], P, id[r] >= 0, id[r], ld, kb, wc);
     }
+    int mine[R];
+    if (lane < NB) out[lane] = -1;
+    tourn_game<T, R>(v, id, wc, mine);
+#pragma unroll
+    for (int r = 0; r < R; r++)
+        if (mine[r] >= 0) out[mine[r]] = id[r];
 }
 
-// One round: workgroup x elects among rows [x * kTournRows, (x + 1) * kTournRows) of the round's list (rows_in, or the rows from kb
-// on when it is null) and writes NB row numbers (-1: none) to rows_out.
+// One round: workgroup x (two wavefronts) elects among entries [x * kTournRows, (x + 1) * kTournRows) of the round's list (rows_in,
+// or the rows from kb on when it is null) and writes NB row numbers (-1: none) to rows_out.  Each wavefront plays 128 rows, two per
+// lane, and the first then plays their 64 winners: two short games instead of one on four rows per lane, because that one needs 170
+// registers, and a wavefront that wants more than the 128 a retiring wavefront of the update running beside it sets free waits long
+// for its place.
+constexpr int kTournRows = 256, kTournLast = 512;
 template <class T>
-__global__ __launch_bounds__(kTournRows) void invert_tourn_round_kernel(const T* __restrict__ w, const int32_t* __restrict__ rows_in, int count,
-                                                                       int32_t* __restrict__ rows_out, int ld, int kb, int wc, int64_t bs_w,
-                                                                       int64_t bs_rows) {
-    __shared__ TournShared<T, kTournRows / 64> sh;
+__global__ __launch_bounds__(128) void invert_tourn_round_kernel(const T* __restrict__ w, const int32_t* __restrict__ rows_in, int count,
+                                                                int32_t* __restrict__ rows_out, int ld, int kb, int wc, int64_t bs_w,
+                                                                int64_t bs_rows) {
+    __shared__ int won[2][NB];
+    __shared__ int out[NB];
     const T* P = w + (int64_t)blockIdx.y * bs_w;
-    const int t = blockIdx.x * kTournRows + threadIdx.x;
-    int id = -1;
-    if (t < count) id = rows_in ? rows_in[(int64_t)blockIdx.y * bs_rows + t] : kb + t;
-    T orig[NB];
-    tourn_load_row(orig, P, id >= 0, id, ld, kb, wc);
-    tourn_play(orig, id, wc, sh);
+    const int wave = threadIdx.x >> 6;
+    tourn_play<T, 2>(P, rows_in ? rows_in + (int64_t)blockIdx.y * bs_rows : nullptr, blockIdx.x * kTournRows + wave * 128,
+                     min(count, (int)(blockIdx.x + 1) * kTournRows), ld, kb, wc, won[wave]);
+    __syncthreads();
+    if (wave != 0) return;
+    tourn_play<T, 1>(P, &won[0][0], 0, 2 * NB, ld, kb, wc, out);
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    if (threadIdx.x < NB) rows_out[(int64_t)blockIdx.y * bs_rows + blockIdx.x * NB + threadIdx.x] = threadIdx.x < wc ? sh.ids[0][threadIdx.x] : -1;
+    if (threadIdx.x < NB) rows_out[(int64_t)blockIdx.y * bs_rows + blockIdx.x * NB + threadIdx.x] = out[threadIdx.x];
 }
 
-// The last round: elects the block's pivot rows among at most kTournLast rows, records them as the exchanges of steps kb .. kb + wc - 1
-// (ipiv[kb + k] = the position row k's content has reached when its turn comes) and inverts their wc x wc block (Gauss-Jordan in
-// the order of election, whose pivots are the elimination's own) into pinv (NB x NB per matrix, row-major).  The bookkeeping and the
-// inversion are the first wavefront's alone, in registers: lane j keeps exchange j, lane (h, j) keeps rows 16 h .. 16 h + 15 of
-// column j, so neither needs a barrier.
+// The last round: elects the block's pivot rows among at most kTournLast rows (four wavefronts play 128 each, the first then plays
+// their winners), records them as the exchanges of steps kb .. kb + wc - 1 (ipiv[kb + k] = the position row k's content has reached
+// when its turn comes) and inverts their wc x wc block (Gauss-Jordan in the order of election, whose pivots are the elimination's
+// own) into pinv (NB x NB per matrix, row-major).
+constexpr int kTournLastThreads = 256;
 template <class T>
-__global__ __launch_bounds__(kTournLast) void invert_tourn_last_kernel(const T* __restrict__ w, const int32_t* __restrict__ rows_in, int count,
-                                                                      int32_t* __restrict__ ipiv, T* __restrict__ pinv, int32_t* singular, int n,
-                                                                      int ld, int kb, int wc, int64_t bs_w, int64_t bs_rows) {
-    static_assert(NB == 32, "the single-wavefront inversion holds a 32 x 32 block");
-    extern __shared__ __align__(16) unsigned char tourn_lds[];
-    typedef TournShared<T, kTournLast / 64> Shared;
-    Shared& sh = *reinterpret_cast<Shared*>(tourn_lds);
+__global__ __launch_bounds__(kTournLastThreads) void invert_tourn_last_kernel(const T* __restrict__ w, const int32_t* __restrict__ rows_in,
+                                                                              int count, int32_t* __restrict__ ipiv, T* __restrict__ pinv,
+                                                                              int32_t* singular, int n, int ld, int kb, int wc, int64_t bs_w,
+                                                                              int64_t bs_rows) {
+    static_assert(NB == 32 && kTournLastThreads == 256, "the inversion deals 32 x 32 entries to 256 threads");
+    constexpr int W0 = kTournLastThreads / 64, R = kTournLast / kTournLastThreads;
+    __shared__ int won[W0][NB];
+    __shared__ int ids[NB];
+    __shared__ T pm[2][NB][NB + 1];
     const T* P = w + (int64_t)blockIdx.x * bs_w;
-    const int tid = threadIdx.x;
-    {
-        int id = -1;
-        if (tid < count) id = rows_in ? rows_in[(int64_t)blockIdx.x * bs_rows + tid] : kb + tid;
-        T orig[NB];
-        tourn_load_row(orig, P, id >= 0, id, ld, kb, wc);
-        tourn_play(orig, id, wc, sh);
+    const int32_t* list = rows_in ? rows_in + (int64_t)blockIdx.x * bs_rows : nullptr;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    // one copy of the game's code (the two rounds in a loop): three would not fit the instruction cache
+    const bool single = count <= 64 * R;
+#pragma unroll 1
+    for (int level = single ? 1 : 0; level < 2; level++) {
+        const bool second = level == 1 && !single;
+        if (level == 0 || wave == 0)
+            tourn_play<T, R>(P, second ? &won[0][0] : list, level == 0 ? wave * 64 * R : 0, second ? W0 * NB : count, ld, kb, wc,
+                             level == 0 ? won[wave] : ids);
+        __syncthreads();
     }
-    if (tid >= 64) return;
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    const int lane = tid;
-    int* ids = sh.ids[0];
-    if (__ballot(lane < wc && ids[lane] < 0)) {
-        // a column without a pivot: the matrix is singular; rows nobody elected keep the bookkeeping consistent (their panel entries
-        // stand in for the missing pivot rows)
+    if (wave == 0 && __ballot(lane < wc && ids[lane] < 0)) {
+        // a column without a pivot: the matrix is singular; rows nobody elected keep the bookkeeping consistent
         if (lane == 0) {
             *singular = 1;
             for (int k = 0; k < wc; k++) {
@@ -578,79 +585,91 @@ __global__ __launch_bounds__(kTournLast) void invert_tourn_last_kernel(const T* 
                     for (int j = 0; j < wc; j++) taken |= ids[j] == g;
                     if (!taken) { ids[k] = g; break; }
                 }
-                for (int j = 0; j < wc; j++) sh.rows[0][k][j] = P[(int64_t)ids[k] * ld + kb + j];
             }
         }
-        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    }
+    __syncthreads();
+    // The inversion: thread t keeps entries (t / 32 + 8 e, t % 32), e = 0 .. 3, in registers and posts them after every step to the
+    // LDS copy the next step reads its pivot row and column from (two copies in turn: one barrier per step).  The first wavefront
+    // also does the bookkeeping of the exchanges, one row per step: lane j keeps exchange j.
+    const int j = tid & 31, i0 = tid >> 5;
+    T a[4];
+#pragma unroll
+    for (int e = 0; e < 4; e++) {
+        const int i = i0 + 8 * e;
+        a[e] = (i < wc && j < wc) ? P[(int64_t)ids[i] * ld + kb + j] : (i == j ? T(1) : T(0));
+        pm[0][i][j] = a[e];
     }
     const int sel = lane < wc ? ids[lane] : -1;
-    int partner = 0;   // lane k: where the content of elected row k sits after the exchanges of steps 0 .. k - 1
+    int partner = 0;   // lane k of the first wavefront: where the content of elected row k sits after the exchanges of steps 0 .. k - 1
+    __syncthreads();
     for (int k = 0; k < wc; k++) {
-        int pos = __builtin_amdgcn_readlane(sel, k);
-        // exchange j moves the row when it sits at kb + j or at partner[j]; the exchanges are looked at in order, few ever match
-        unsigned long long later = ~0ull;
-        while (true) {
-            const unsigned long long hit = __ballot(lane < k && (partner == pos || kb + lane == pos)) & later;
-            if (!hit) break;
-            const int jj = __builtin_ctzll(hit);
-            const int pj = __builtin_amdgcn_readlane(partner, jj);
-            pos = (pos == kb + jj) ? pj : kb + jj;
-            later = ~0ull << (jj + 1);   // jj <= 30
+        const T(*src)[NB + 1] = pm[k & 1];
+        T(*dst)[NB + 1] = pm[(k + 1) & 1];
+        const T pv = src[k][k];
+        if (tid == 0 && !(abs_of(pv) > T(0))) *singular = 1;
+        const T sj = (j == k ? T(1) : src[k][j]) / pv;         // the pivot row, scaled: 1 / pivot where the pivot was
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int i = i0 + 8 * e;
+            const T f = src[i][k];                             // the row's entry in the pivot column
+            a[e] = (i == k) ? sj : ((j == k) ? T(0) : a[e]) - f * sj;
+            dst[i][j] = a[e];
         }
-        if (lane == k) partner = pos;
-    }
-    if (lane < wc) ipiv[(int64_t)blockIdx.x * n + kb + lane] = partner;
-
-    const int j = lane & 31, h = lane >> 5;
-    T a[16];
-#pragma unroll
-    for (int ii = 0; ii < 16; ii++) {
-        const int i = h * 16 + ii;
-        a[ii] = (i < wc && j < wc) ? sh.rows[0][i][j] : (i == j ? T(1) : T(0));
-    }
-    static_for<NB>([&](auto kk) {
-        constexpr int k = decltype(kk)::value, kr = k % 16, kh = k / 16;
-        if (k >= wc) return;
-        const T pv = read_lane(a[kr], kh * 32 + k);
-        if (!(abs_of(pv) > T(0)) && lane == 0) *singular = 1;
-        const T rk = __shfl(a[kr], kh * 32 + j, 64);           // the pivot row's entry in this lane's column
-        const T sj = (j == k ? T(1) : rk) / pv;                // the pivot row, scaled: 1 / pivot where the pivot was
-        T f[16];
-#pragma unroll
-        for (int ii = 0; ii < 16; ii++) f[ii] = __shfl(a[ii], h * 32 + k, 64);   // every row's entry in the pivot column
-#pragma unroll
-        for (int ii = 0; ii < 16; ii++) {
-            const bool pivot_row = (ii == kr) && (h == kh);
-            a[ii] = pivot_row ? sj : ((j == k) ? T(0) : a[ii]) - f[ii] * sj;
+        if (wave == 0) {
+            int pos = __builtin_amdgcn_readlane(sel, k);
+            // exchange x moves the row when it sits at kb + x or at partner[x]; the exchanges are looked at in order, few ever match
+            unsigned long long later = ~0ull;
+            while (true) {
+                const unsigned long long hit = __ballot(lane < k && (partner == pos || kb + lane == pos)) & later;
+                if (!hit) break;
+                const int x = __builtin_ctzll(hit);
+                const int px = __builtin_amdgcn_readlane(partner, x);
+                pos = (pos == kb + x) ? px : kb + x;
+                later = ~0ull << (x + 1);   // x <= 30
+            }
+            if (lane == k) partner = pos;
         }
-    });
+        __syncthreads();
+    }
+    if (wave == 0 && lane < wc) ipiv[(int64_t)blockIdx.x * n + kb + lane] = partner;
 #pragma unroll
-    for (int ii = 0; ii < 16; ii++) {
-        const int i = h * 16 + ii;
-        pinv[(int64_t)blockIdx.x * NB * NB + i * NB + j] = (i < wc && j < wc) ? a[ii] : T(0);
+    for (int e = 0; e < 4; e++) {
+        const int i = i0 + 8 * e;
+        pinv[(int64_t)blockIdx.x * NB * NB + i * NB + j] = (i < wc && j < wc) ? a[e] : T(0);
     }
 }
 
 // After the exchanges: the panel becomes G (row r of the block's rows: row r - kb of P^-1; any other row: minus its panel entries
 // times P^-1), and gbuf receives G - I_block for the update of the other columns.  Four threads per row, eight columns each.
+// The same threads apply the update to the w1 columns from next0 on (the next block's panel, which its tournament is waiting for):
+// W[r, next0 + c] += sum_j (G - I)[r, j] T[j, next0 + c], the row's 32 factors passed round its four threads through LDS.
 constexpr int kTournGThreads = 256;
 template <class T>
-__global__ __launch_bounds__(kTournGThreads) void invert_tourn_g_kernel(T* __restrict__ w, T* __restrict__ gbuf, const T* __restrict__ pinv, int n,
-                                                                        int ld, int kb, int wc, int64_t bs_w, int64_t bs_g) {
+__global__ __launch_bounds__(kTournGThreads) void invert_tourn_g_kernel(T* __restrict__ w, T* __restrict__ gbuf, const T* __restrict__ pinv,
+                                                                        const T* __restrict__ tbuf, int n, int ld, int kb, int wc, int next0,
+                                                                        int w1, int64_t bs_w, int64_t bs_g, int64_t bs_t) {
     typedef T vec4 __attribute__((ext_vector_type(4)));
     __shared__ __align__(16) T pi[NB][NB];
-    for (int e = threadIdx.x; e < NB * NB; e += kTournGThreads) pi[e / NB][e % NB] = pinv[(int64_t)blockIdx.y * NB * NB + e];
+    __shared__ __align__(16) T tn[NB][NB];
+    __shared__ __align__(16) T gsh[kTournGThreads / 4][NB + 4];
+    for (int e = threadIdx.x; e < NB * NB; e += kTournGThreads) {
+        const int i = e / NB, c = e % NB;
+        pi[i][c] = pinv[(int64_t)blockIdx.y * NB * NB + e];
+        tn[i][c] = (i < wc && c < w1) ? tbuf[(int64_t)blockIdx.y * bs_t + (int64_t)i * ld + next0 + c] : T(0);
+    }
     __syncthreads();
+    // rows beyond n keep their lanes and store nothing
     const int r = blockIdx.x * (kTournGThreads / 4) + threadIdx.x / 4, c0 = (threadIdx.x & 3) * 8;
-    if (r >= n) return;
-    T* row = w + (int64_t)blockIdx.y * bs_w + (int64_t)r * ld + kb;
+    const bool in = r < n;
+    T* row = w + (int64_t)blockIdx.y * bs_w + (int64_t)(in ? r : 0) * ld;
     T out[8];
-    if (r >= kb && r < kb + wc) {
+    if (in && r >= kb && r < kb + wc) {
 #pragma unroll
         for (int j = 0; j < 8; j++) out[j] = pi[r - kb][c0 + j];
     } else {
         T c[NB];
-        tourn_load_row(c, w + (int64_t)blockIdx.y * bs_w, true, r, ld, kb, wc);
+        tourn_load_row(c, w + (int64_t)blockIdx.y * bs_w, in, r, ld, kb, wc);
 #pragma unroll
         for (int j = 0; j < 8; j++) out[j] = T(0);
 #pragma unroll
@@ -667,13 +686,42 @@ __global__ __launch_bounds__(kTournGThreads) void invert_tourn_g_kernel(T* __res
     }
     // every thread of a row has read the row's panel entries before any of them is replaced: the four sit in one wavefront
     __builtin_amdgcn_wave_barrier();
-    T* g = gbuf + (int64_t)blockIdx.y * bs_g + (int64_t)r * NB;
+    T gi[8];   // G - I
 #pragma unroll
-    for (int j = 0; j < 8; j++)
-        if (c0 + j < wc) {
-            row[c0 + j] = out[j];
-            g[c0 + j] = out[j] - ((r == kb + c0 + j) ? T(1) : T(0));
+    for (int j = 0; j < 8; j++) gi[j] = out[j] - ((r == kb + c0 + j) ? T(1) : T(0));
+    if (in) {
+        T* g = gbuf + (int64_t)blockIdx.y * bs_g + (int64_t)r * NB;
+#pragma unroll
+        for (int j = 0; j < 8; j++)
+            if (c0 + j < wc) {
+                row[kb + c0 + j] = out[j];
+                g[c0 + j] = gi[j];
+            }
+    }
+    if (w1 <= 0) return;
+    // the row's 32 factors, from its four threads (one wavefront: no barrier, only program order)
+    const int rl = threadIdx.x / 4;
+    *reinterpret_cast<vec4*>(&gsh[rl][c0]) = vec4{gi[0], gi[1], gi[2], gi[3]};
+    *reinterpret_cast<vec4*>(&gsh[rl][c0 + 4]) = vec4{gi[4], gi[5], gi[6], gi[7]};
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    T acc[8];
+#pragma unroll
+    for (int e = 0; e < 8; e++) acc[e] = T(0);
+#pragma unroll 4   // rolled: unrolled whole, the compiler fetches every factor and every vector of tn before the first product
+    for (int j = 0; j < NB; j++) {
+        const T f = gsh[rl][j];
+        const vec4 t0 = *reinterpret_cast<const vec4*>(&tn[j][c0]), t1 = *reinterpret_cast<const vec4*>(&tn[j][c0 + 4]);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            acc[e] += f * t0[e];
+            acc[4 + e] += f * t1[e];
         }
+    }
+    if (!in) return;
+#pragma unroll
+    for (int e = 0; e < 8; e++)
+        if (c0 + e < w1) row[next0 + c0 + e] += acc[e];
 }
 
 // Composes the column permutation that undoes the row exchanges: exchanges are applied to columns in reverse order.
@@ -710,6 +758,16 @@ __global__ void invert_clear_flag_kernel(int32_t* flag) { *flag = 0; }
 
 size_t align_up(size_t x) { return (x + 255) / 256 * 256; }
 
+// One more stream, created on first use and kept: the update of the columns a tournament does not need runs on it beside the tournament.
+int32_t side_stream(hipStream_t* out) {
+    static std::mutex mu;
+    static hipStream_t s = nullptr;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!s) DNH_HIP(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));
+    *out = s;
+    return DNH_OK;
+}
+
 template <class T>
 int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream) {
     const int nd = t->ndims;
@@ -735,7 +793,7 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
     const size_t sz_r = t_is_c ? 0 : align_up((size_t)batch * n * n * sizeof(T));
     // pivots by tournament: two lists of candidate rows (NB per workgroup of the first round) and the inverted pivot block
     const int tourn_opt = option(OPT_INVERT_TOURNAMENT);
-    const bool tourn = tourn_opt == 1 || (tourn_opt < 0 && n >= 1024);
+    const bool tourn = tourn_opt == 1 || (tourn_opt < 0 && n > NB);   // measured faster from two blocks on, single and batched
     const int64_t bs_rows = (int64_t)cdiv(n, kTournRows) * NB;
     const size_t sz_rows = tourn ? align_up((size_t)batch * bs_rows * sizeof(int32_t)) : 0;
     const size_t sz_pinv = tourn ? align_up((size_t)batch * NB * NB * sizeof(T)) : 0;
@@ -754,6 +812,19 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
     int32_t* rows_b = (int32_t*)((char*)rows_a + sz_rows);
     T* pinv = (T*)((char*)rows_a + 2 * sz_rows);
 
+    // the side stream of the tournament form (the library's own, default priority), with the two events that order it against `stream`
+    hipStream_t side = nullptr;
+    hipEvent_t ev_main = nullptr, ev_side = nullptr;
+    bool side_busy = false;
+    if (tourn && n > 2 * NB) {
+        DNH_TRY(side_stream(&side));
+        if (hipEventCreateWithFlags(&ev_main, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&ev_side, hipEventDisableTiming) != hipSuccess) {
+            if (ev_main) (void)hipEventDestroy(ev_main);
+            (void)dnh_free_async(block, stream);
+            return fail(DNH_ERR_HIP, "dnh_batched_invert: cannot create an event");
+        }
+    }
     int32_t st = DNH_OK;
     auto body = [&]() -> int32_t {
         // src (any layout, broadcast batch dimensions included) -> W, rows padded to ld
@@ -797,30 +868,62 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
 #undef DNH_SUBPANEL
             return DNH_OK;
         };
-        const size_t tourn_lds = sizeof(TournShared<T, kTournLast / 64>);
-        if (tourn && tourn_lds > 32 * 1024)
-            DNH_HIP(hipFuncSetAttribute((const void*)invert_tourn_last_kernel<T>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)tourn_lds));
         for (int kb = 0; kb < n; kb += NB) {
             const int wc = (n - kb < NB) ? n - kb : NB;
             if (tourn) {
-                int count = n - kb;
-                const int32_t* rows_in = nullptr;
-                int32_t* rows_out = rows_a;
-                while (count > kTournLast) {
-                    const int chunks = (int)cdiv(count, kTournRows);
-                    hipLaunchKernelGGL((invert_tourn_round_kernel<T>), dim3((unsigned)chunks, (unsigned)batch), dim3(kTournRows), 0, stream, W,
-                                       rows_in, count, rows_out, ld, kb, wc, bs_w, bs_rows);
-                    count = chunks * NB;
-                    rows_in = rows_out;
-                    rows_out = rows_out == rows_a ? rows_b : rows_a;
+                // the tournament of a block: queued for the first block here, for every later one right behind the previous block's
+                // own-column work (below), ahead of that block's side-stream launches, so that the device never waits for it
+                auto play = [&](int pkb, int pwc) {
+                    int count = n - pkb;
+                    const int32_t* rows_in = nullptr;
+                    int32_t* rows_out = rows_a;
+                    while (count > kTournLast) {
+                        const int chunks = (int)cdiv(count, kTournRows);
+                        hipLaunchKernelGGL((invert_tourn_round_kernel<T>), dim3((unsigned)chunks, (unsigned)batch), dim3(128), 0, stream, W,
+                                           rows_in, count, rows_out, ld, pkb, pwc, bs_w, bs_rows);
+                        count = chunks * NB;
+                        rows_in = rows_out;
+                        rows_out = rows_out == rows_a ? rows_b : rows_a;
+                    }
+                    hipLaunchKernelGGL((invert_tourn_last_kernel<T>), dim3((unsigned)batch), dim3(kTournLastThreads), 0, stream, W, rows_in, count,
+                                       ipiv, pinv, flag, n, ld, pkb, pwc, bs_w, bs_rows);
+                };
+                if (kb == 0) play(kb, wc);
+                if (side_busy) {
+                    DNH_HIP(hipStreamWaitEvent(stream, ev_side, 0));
+                    side_busy = false;
                 }
-                hipLaunchKernelGGL((invert_tourn_last_kernel<T>), dim3((unsigned)batch), dim3(kTournLast), tourn_lds, stream, W, rows_in, count, ipiv,
-                                   pinv, flag, n, ld, kb, wc, bs_w, bs_rows);
-                hipLaunchKernelGGL((invert_swap_kernel<T, true>), dim3((unsigned)cdiv(n, kSwapThreads), (unsigned)batch), dim3(kSwapThreads), 0,
-                                   stream, W, Tb, ipiv, n, ld, kb, wc, 0, n, bs_w, bs_t);
+                // The exchange and the update W += (G - I) . T of the block's own columns and of the next block's (all its tournament
+                // needs) run here; the columns to their left and right get theirs on the side stream, beside that tournament.  The
+                // exchange after it waits for them: it rewrites T, and G is rewritten behind it.
+                const int next0 = kb + wc, next1 = (n - next0 < NB) ? n : next0 + NB;
+                auto exchange = [&](int c0, int c1, hipStream_t s) {
+                    if (c1 > c0)
+                        hipLaunchKernelGGL((invert_swap_kernel<T, true>), dim3((unsigned)cdiv(c1 - c0, kSwapThreads), (unsigned)batch),
+                                           dim3(kSwapThreads), 0, s, W, Tb, ipiv, n, ld, kb, wc, c0, c1, bs_w, bs_t);
+                };
+                auto update = [&](int c0, int c1, hipStream_t s) -> int32_t {
+                    if (c1 <= c0) return DNH_OK;
+                    return gemm_accumulate(t->dtype, W + c0, G, Tb + c0, n, c1 - c0, wc, NB, ld, ld, batch, bs_g, bs_t, bs_w, s);
+                };
+                exchange(0, n, stream);
                 hipLaunchKernelGGL((invert_tourn_g_kernel<T>), dim3((unsigned)cdiv(n, kTournGThreads / 4), (unsigned)batch), dim3(kTournGThreads), 0,
-                                   stream, W, G, pinv, n, ld, kb, wc, bs_w, bs_g);
-                if (n > wc) DNH_TRY(gemm_accumulate(t->dtype, W, G, Tb, n, n, wc, NB, ld, ld, batch, bs_g, bs_t, bs_w, stream));
+                                   stream, W, G, pinv, Tb, n, ld, kb, wc, next0, next1 - next0, bs_w, bs_g, bs_t);
+                hipStream_t rest = stream;
+                if (side) {
+                    DNH_HIP(hipEventRecord(ev_main, stream));
+                    if (next0 < n) play(next0, next1 - next0);
+                    DNH_HIP(hipStreamWaitEvent(side, ev_main, 0));
+                    rest = side;
+                }
+                DNH_TRY(update(0, kb, rest));
+                DNH_TRY(update(next1, n, rest));
+                if (side) {
+                    DNH_HIP(hipEventRecord(ev_side, side));
+                    side_busy = true;
+                } else if (next0 < n) {
+                    play(next0, next1 - next0);
+                }
                 continue;
             }
             if (sb == NB) {
@@ -845,6 +948,10 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
                 DNH_TRY(gemm_accumulate(t->dtype, W, G, Tb, n, n, wc, NB, ld, ld, batch, bs_g, bs_t, bs_w, stream));
             }
         }
+        if (side_busy) {
+            DNH_HIP(hipStreamWaitEvent(stream, ev_side, 0));
+            side_busy = false;
+        }
         const int use_lds = (size_t)n * sizeof(int32_t) <= 48 * 1024;
         hipLaunchKernelGGL(invert_perm_kernel, dim3((unsigned)batch), dim3(256), use_lds ? (size_t)n * sizeof(int32_t) : 0, stream, perm, ipiv,
                            n, use_lds);
@@ -866,6 +973,11 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
         return DNH_OK;
     };
     st = body();
+    if (side_busy) {   // an error left the side stream at work on the block about to be freed
+        if (hipStreamWaitEvent(stream, ev_side, 0) != hipSuccess) (void)hipStreamSynchronize(side);
+    }
+    if (ev_main) (void)hipEventDestroy(ev_main);
+    if (ev_side) (void)hipEventDestroy(ev_side);
     (void)dnh_free_async(block, stream);
     return st;
 }

@@ -167,10 +167,11 @@ int32_t dnh_last_error(char* buf, size_t n);
  *   "count_one_launch"  1 (default): CountTrue of a whole contiguous mask in one launch
  *   "lookback_spins"    262144 (default): how often a tile of a one-pass compaction polls for the counts of the tiles before it
  *                       before it counts them itself (0: at once; for tests of that path)
- *   "invert_tournament" -1 (default): BatchedInvert of matrices with 1024 rows and more chooses the 32 pivot rows of a panel by
- *                       tournament (workgroups elect candidates among 256 rows each, one workgroup elects among the candidates);
- *                       0: every size eliminates its panels column by column with partial pivoting in one workgroup; 1: tournament
- *                       for every size
+ *   "invert_tournament" -1 (default): BatchedInvert of matrices with more than 32 rows chooses the 32 pivot rows of a panel by
+ *                       tournament (wavefronts elect candidates among 128 rows each, further games among the candidates) and
+ *                       updates the columns the next panel does not need on a stream of the library's own, beside that panel's
+ *                       tournament; 0: every size eliminates its panels column by column with partial pivoting in one
+ *                       workgroup; 1: tournament for every size
  * Unknown names and values outside an option's range: DNH_ERR_INVALID_ARG. */
 int32_t dnh_set_option(const char* name, int32_t value);
 int32_t dnh_get_option(const char* name, int32_t* value);

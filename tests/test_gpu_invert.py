@@ -11,10 +11,10 @@ from invert_cases import hilbert, hilbert_inverse, inverse_error_bound, invert, 
 pytestmark = pytest.mark.gpu
 
 
-@pytest.fixture(params=[-1, 1], ids=["own_choice", "tournament"])
+@pytest.fixture(params=[0, 1], ids=["column_by_column", "tournament"])
 def pivot_form(request):
-    """Runs a test once with the library's own choice of how a panel's pivots are found (column by column in one workgroup below
-    1024 rows) and once with the tournament form for every size."""
+    """Runs a test once with every panel eliminated column by column in one workgroup and once with the panels' pivots found by
+    tournament, whatever the size (the library's own choice: the tournament from 33 rows on)."""
     from deepnet_amd import native
     with native.option("invert_tournament", request.param):
         yield request.param
