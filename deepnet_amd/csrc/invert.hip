@@ -339,7 +339,9 @@ __global__ __launch_bounds__(256) void invert_extract_g_kernel(const T* __restri
 // independent loads and one round of stores instead of wc dependent round trips.
 // OWN: the block's own columns are exchanged as well (their T stays zero); the panel kernels that eliminate column by column have
 // exchanged them already.
-constexpr int kSwapThreads = 64;
+// Four threads share a column (64 columns per workgroup), each taking every fourth of the affected rows: a quarter of the round
+// trips per thread and four times the loads in flight, which is what a kernel this small lives on when another runs beside it.
+constexpr int kSwapCols = 64, kSwapThreads = 256;
 template <class T, bool OWN>
 __global__ __launch_bounds__(kSwapThreads) void invert_swap_kernel(T* __restrict__ w, T* __restrict__ tbuf, const int32_t* __restrict__ ipiv,
                                                                    int n, int ld, int kb, int wc, int c_begin, int c_end, int64_t bs_w,
@@ -348,31 +350,35 @@ __global__ __launch_bounds__(kSwapThreads) void invert_swap_kernel(T* __restrict
     __shared__ int src[2 * NB];   // the row whose content ends up at pos[i]
     __shared__ int cnt;
     const int32_t* piv = ipiv + (int64_t)blockIdx.y * n;
-    {
+    if (threadIdx.x < 64) {
         const int m = replay_exchanges_wave(threadIdx.x < wc ? piv[kb + threadIdx.x] : 0, kb, wc, threadIdx.x, pos, src);
         if (threadIdx.x == 0) cnt = m;
     }
     __syncthreads();
-    const int c = c_begin + blockIdx.x * kSwapThreads + threadIdx.x;
-    if (c >= c_end) return;
+    const int c = c_begin + blockIdx.x * kSwapCols + (threadIdx.x & 63), part = threadIdx.x >> 6;
+    const bool in = c < c_end;
     T* P = w + (int64_t)blockIdx.y * bs_w;
     T* Tb = tbuf + (int64_t)blockIdx.y * bs_t;
     const bool own = c >= kb && c < kb + wc;
-    if (own && !OWN) {
-        for (int j = 0; j < wc; j++) Tb[(int64_t)j * ld + c] = T(0);
-        return;
-    }
+    const bool move = in && (OWN || !own);
+    if (in && !move)
+        for (int j = part; j < wc; j += 4) Tb[(int64_t)j * ld + c] = T(0);
     const int m = cnt;
-    T val[2 * NB];
+    T val[2 * NB / 4];
 #pragma unroll
-    for (int i = 0; i < 2 * NB; i++)
-        if (i < m) val[i] = P[(int64_t)src[i] * ld + c];
+    for (int u = 0; u < 2 * NB / 4; u++) {
+        const int i = part + 4 * u;
+        if (move && i < m) val[u] = P[(int64_t)src[i] * ld + c];
+    }
+    __syncthreads();   // a column's four threads have read their rows before any of them is overwritten
 #pragma unroll
-    for (int i = 0; i < 2 * NB; i++)
-        if (i < m) {
-            if (src[i] != pos[i]) P[(int64_t)pos[i] * ld + c] = val[i];
-            if (i < wc) Tb[(int64_t)i * ld + c] = own ? T(0) : val[i];
+    for (int u = 0; u < 2 * NB / 4; u++) {
+        const int i = part + 4 * u;
+        if (move && i < m) {
+            if (src[i] != pos[i]) P[(int64_t)pos[i] * ld + c] = val[u];
+            if (i < wc) Tb[(int64_t)i * ld + c] = own ? T(0) : val[u];
         }
+    }
 }
 
 // ---- pivots by tournament ---------------------------------------------------------------------------------------------------------
@@ -899,7 +905,7 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
                 const int next0 = kb + wc, next1 = (n - next0 < NB) ? n : next0 + NB;
                 auto exchange = [&](int c0, int c1, hipStream_t s) {
                     if (c1 > c0)
-                        hipLaunchKernelGGL((invert_swap_kernel<T, true>), dim3((unsigned)cdiv(c1 - c0, kSwapThreads), (unsigned)batch),
+                        hipLaunchKernelGGL((invert_swap_kernel<T, true>), dim3((unsigned)cdiv(c1 - c0, kSwapCols), (unsigned)batch),
                                            dim3(kSwapThreads), 0, s, W, Tb, ipiv, n, ld, kb, wc, c0, c1, bs_w, bs_t);
                 };
                 auto update = [&](int c0, int c1, hipStream_t s) -> int32_t {
@@ -943,7 +949,7 @@ int32_t invert_impl(const DnhTensor* t, const DnhTensor* src, hipStream_t stream
                                    bs_w, bs_g);
             }
             if (n > wc) {
-                hipLaunchKernelGGL((invert_swap_kernel<T, false>), dim3((unsigned)cdiv(n, kSwapThreads), (unsigned)batch), dim3(kSwapThreads), 0, stream,
+                hipLaunchKernelGGL((invert_swap_kernel<T, false>), dim3((unsigned)cdiv(n, kSwapCols), (unsigned)batch), dim3(kSwapThreads), 0, stream,
                                    W, Tb, ipiv, n, ld, kb, wc, 0, n, bs_w, bs_t);
                 DNH_TRY(gemm_accumulate(t->dtype, W, G, Tb, n, n, wc, NB, ld, ld, batch, bs_g, bs_t, bs_w, stream));
             }
