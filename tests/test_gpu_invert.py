@@ -113,6 +113,17 @@ def test_large_matrix_by_identity(G, rng, pivot_form):
     assert np.abs(prod - np.eye(n)).max() <= 8 * n * 2 ** -23 * np.linalg.cond(a.astype(np.float64))
 
 
+def test_two_rounds_of_games(G, rng):
+    """4400 rows: the first panels have more rows than 16 x 256, so a round of games leaves more than 512 candidates and a second round
+    runs before the last workgroup's; the pivots must still be good ones (no diagonal dominance to lean on)."""
+    n = 4400
+    q, _ = np.linalg.qr(rng.standard_normal((n, n)))
+    a = (q * rng.uniform(1.0, 4.0, n)).astype(np.float32)          # orthogonal columns scaled: condition number 4, no structure
+    ta = G.ofNumpy(a)
+    prod = G.toNumpy(Tensor.invert(ta) @ ta)
+    assert np.abs(prod - np.eye(n)).max() <= 8 * n * 2 ** -23 * 4
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.float64])
 def test_tournament_pivots(G, rng, dtype):
     """What the tournament has to get right beyond accuracy on friendly matrices: a panel whose large entries sit in few rows (every
