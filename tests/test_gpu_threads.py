@@ -61,6 +61,49 @@ def test_concurrent_threads_on_their_own_streams(G, H):
             np.testing.assert_array_equal(ref, g)
 
 
+def test_concurrent_inversions_share_the_side_stream(G):
+    """BatchedInvert by tournament updates part of the matrix on one stream of the library's own, ordered against the caller's stream
+    by events of the call.  Four host threads on four streams invert at once: their side-stream work interleaves in one queue, and
+    every result must be what the same call gives alone, bit for bit."""
+    from deepnet_amd.tensor import Tensor
+    lib = native.load()
+    nthreads = 4
+    rng = np.random.default_rng(11)
+    inputs = [(rng.standard_normal((n, n)) / np.sqrt(n) + 2 * np.eye(n)).astype(dt)
+              for n, dt in ((700, np.float32), (450, np.float64), (1100, np.float32), (260, np.float32))]
+    want = [G.toNumpy(Tensor.invert(G.ofNumpy(a))) for a in inputs]
+    got = [None] * nthreads
+    errors = []
+
+    def worker(i):
+        try:
+            s = C.c_void_p()
+            native.check(lib.dnh_stream_create(C.byref(s)))
+            G.Cfg.Stream = s.value
+            try:
+                t = G.ofNumpy(inputs[i])
+                for _ in range(3):
+                    r = Tensor.invert(t)
+                got[i] = G.toNumpy(r)
+            finally:
+                G.synchronize()
+                G.Cfg.Stream = 0
+                native.check(lib.dnh_stream_destroy(s))
+        except Exception as e:  # noqa: BLE001
+            errors.append((i, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(i,)) for i in range(nthreads)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=100)
+    assert not errors, errors
+    for i in range(nthreads):
+        np.testing.assert_array_equal(got[i], want[i])
+        n = inputs[i].shape[0]
+        assert np.abs(got[i].astype(np.float64) @ inputs[i].astype(np.float64) - np.eye(n)).max() <= 64 * n * np.finfo(inputs[i].dtype).eps
+
+
 def test_concurrent_threads_sharing_one_stream(G, H):
     """Host threads that never set Cfg.Stream all enqueue on the default stream and so share its workspace: an entry point keeps
     the buffer to itself until every kernel that uses it is queued, so split folds, compactions and split products of different
