@@ -731,21 +731,39 @@ __global__ __launch_bounds__(kTournGThreads) void invert_tourn_g_kernel(T* __res
 }
 
 // Composes the column permutation that undoes the row exchanges: exchanges are applied to columns in reverse order.
-// perm[j] = the column of the work matrix that becomes column j of the inverse.
+// perm[j] = the column of the work matrix that becomes column j of the inverse.  The exchanges of a block of NB steps touch at most
+// 2 NB entries; what they do together is found by one wavefront in registers (replay_exchanges_wave: entry pos[i] ends up with the
+// content of entry src[i] when the block's exchanges are applied in order; in reverse order, entry src[i] with that of pos[i]).  Four
+// wavefronts replay four blocks at a time, the first then applies them to the permutation, last block first: two LDS round trips a
+// block instead of four a step.
 __global__ __launch_bounds__(256) void invert_perm_kernel(int32_t* __restrict__ perm, const int32_t* __restrict__ ipiv, int n, int use_lds) {
     extern __shared__ int32_t sp[];
+    __shared__ int pos[4][2 * NB], src[4][2 * NB], cnt[4];
     int32_t* out = perm + (int64_t)blockIdx.x * n;
     const int32_t* piv = ipiv + (int64_t)blockIdx.x * n;
     int32_t* cur = use_lds ? sp : out;
     for (int i = threadIdx.x; i < n; i += 256) cur[i] = i;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        for (int k = n - 1; k >= 0; k--) {
-            const int p = piv[k];
-            if (p != k) { const int32_t t = cur[k]; cur[k] = cur[p]; cur[p] = t; }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int blocks = (n + NB - 1) / NB;
+    for (int top = blocks - 1; top >= 0; top -= 4) {
+        const int blk = top - wave;
+        if (blk >= 0) {
+            const int kb = blk * NB, wc = min(NB, n - kb);
+            const int m = replay_exchanges_wave(lane < wc ? piv[kb + lane] : 0, kb, wc, lane, pos[wave], src[wave]);
+            if (lane == 0) cnt[wave] = m;
         }
+        __syncthreads();   // also: the identity is in place before the first block is applied
+        if (wave == 0) {
+            for (int x = 0; x < 4 && top - x >= 0; x++) {
+                const bool in = lane < cnt[x];
+                const int32_t v = in ? cur[pos[x][lane]] : 0;
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");   // every lane has read before any writes
+                if (in) cur[src[x][lane]] = v;
+                __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "workgroup");   // and the next block reads what this one wrote
+            }
+        }
+        __syncthreads();
     }
-    __syncthreads();
     if (use_lds)
         for (int i = threadIdx.x; i < n; i += 256) out[i] = sp[i];
 }

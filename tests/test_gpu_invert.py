@@ -145,3 +145,23 @@ def test_tournament_pivots(G, rng, dtype):
             invert(G, z)
         # the games are deterministic: the same bits every time
         np.testing.assert_array_equal(invert(G, a), got)
+
+
+def test_large_scaled_permutation_is_exact(G, rng):
+    """12 320 rows: the panel's tournament takes two rounds of games before the last, and the permutation that undoes the row
+    exchanges no longer fits the LDS of the kernel that composes it.  A permutation matrix with rows scaled by powers of two has an
+    inverse that every step computes exactly: its transpose with the reciprocal scales."""
+    n = 12320
+    perm = rng.permutation(n)
+    scale = np.ldexp(1.0, rng.integers(-3, 4, n)).astype(np.float32)
+    a = np.zeros((n, n), np.float32)
+    a[np.arange(n), perm] = scale                       # row i holds scale[i] in column perm[i]
+    got = invert(G, a)
+    rows, cols = np.nonzero(got)
+    assert rows.size == n
+    assert np.array_equal(rows[np.argsort(rows)], np.arange(n))
+    want = np.zeros(n, np.float32)
+    want[perm] = np.float32(1) / scale                  # inverse: row perm[i] holds 1 / scale[i] in column i
+    order = np.argsort(rows)
+    assert np.array_equal(cols[order], np.argsort(perm))
+    assert np.array_equal(got[rows[order], cols[order]], want)
