@@ -35,6 +35,13 @@ type Cfg private () =
         Native.check (Native.dnh_get_option (System.Text.Encoding.ASCII.GetBytes (name + "\000"), &v))
         v
 
+    /// Bytes of the stream's workspace a Scatter of `sources` elements of the given type into a target of `cells` elements takes
+    /// (0 where atomics do the work); makes no device call, so pools can be sized before the first call.
+    static member ScatterWorkspaceBytes (dtype: DType, sources: int64, cells: int64) : uint64 =
+        let mutable bytes = 0un
+        Native.check (Native.dnh_scatter_workspace_bytes (int dtype, sources, cells, &bytes))
+        uint64 bytes
+
 module internal Desc =
     let dtypeOf (t: Type) =
         if   t = typeof<bool>   then DType.Bool elif t = typeof<byte>   then DType.U8  elif t = typeof<sbyte>  then DType.I8
