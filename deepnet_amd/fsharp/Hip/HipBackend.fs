@@ -35,13 +35,6 @@ type Cfg private () =
         Native.check (Native.dnh_get_option (System.Text.Encoding.ASCII.GetBytes (name + "\000"), &v))
         v
 
-    /// Bytes of the stream's workspace a Scatter of `sources` elements of the given type into a target of `cells` elements takes
-    /// (0 where atomics do the work); makes no device call, so pools can be sized before the first call.
-    static member ScatterWorkspaceBytes (dtype: DType, sources: int64, cells: int64) : uint64 =
-        let mutable bytes = 0un
-        Native.check (Native.dnh_scatter_workspace_bytes (int dtype, sources, cells, &bytes))
-        uint64 bytes
-
 module internal Desc =
     let dtypeOf (t: Type) =
         if   t = typeof<bool>   then DType.Bool elif t = typeof<byte>   then DType.U8  elif t = typeof<sbyte>  then DType.I8
@@ -82,6 +75,15 @@ module internal Desc =
             let h = GCHandle.Alloc (v, GCHandleType.Pinned)
             try f (h.AddrOfPinnedObject ()) finally h.Free ()
             v.[0]
+
+/// What the library reports without touching the device.
+type Planning private () =
+    /// Bytes of the stream's workspace a Scatter of `sources` elements of type 'T into a target of `cells` elements takes
+    /// (0 where atomics do the work), so that pools can be sized before the first call.
+    static member ScatterWorkspaceBytes<'T> (sources: int64, cells: int64) : uint64 =
+        let mutable bytes = 0un
+        Native.check (Native.dnh_scatter_workspace_bytes (int (Desc.dtypeOf typeof<'T>), sources, cells, &bytes))
+        uint64 bytes
 
 /// Device memory owned by one tensor storage (CudaBackend.fs:54-93).
 /// The block comes from the library's stream-ordered cache under the stream current at creation.  While every use was
