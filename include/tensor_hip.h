@@ -310,7 +310,8 @@ int32_t dnh_dot(const DnhTensor* t, const DnhTensor* a, const DnhTensor* b, void
  * t's shape by the frontend, Tensor.fs:2811-2815), single or double; any strides; t may be src.  Gauss-Jordan with row pivoting:
  * partial pivoting for matrices of up to 32 rows, tournament pivoting (the 32 pivot rows of a block of columns elected by games of
  * partial pivoting among groups of rows) above, see the option "invert_tournament"; either way the result is an inverse computed
- * by a backward-stable elimination, within n eps cond(A) max|inv(A)| of LAPACK's in the tests, not its bits.  A pivot that is
+ * by a backward-stable elimination (in the tests within 8 n eps cond(A) max|inv(A)| of the exact inverse, as LAPACK's is), not
+ * LAPACK's bits.  A pivot that is
  * exactly zero gives DNH_ERR_SINGULAR_MATRIX (LAPACK info > 0).  Synchronises the stream to read that flag. */
 int32_t dnh_batched_invert(const DnhTensor* t, const DnhTensor* src, void* stream);
 
